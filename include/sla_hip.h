@@ -1,0 +1,133 @@
+/*
+ * C ABI of the MI355X (gfx950) Sparse-Linear Attention kernels.
+ *
+ * The reference operator is Python; it has no FFI of its own.  Each entry point
+ * below replaces one device-side step of the reference and names the reference
+ * lines it stands in for (paths inside the reference checkout).
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless stated otherwise; tensors are
+ *     dense, row-major, (B,H,L,D) with D fastest;
+ *   - the caller owns every buffer including workspaces (sizes from
+ *     sla_workspace_bytes); the library allocates nothing and keeps no state;
+ *   - `stream` is a hipStream_t passed as void*; all work is enqueued on it and
+ *     no call synchronises with the host;
+ *   - return value 0 = success, negative = error (see SLA_ERR_*); the message of
+ *     the last error on the calling thread is returned by sla_last_error();
+ *   - argument validation happens before any device work, so error paths can be
+ *     exercised on a host without a GPU.
+ */
+#ifndef SLA_HIP_H
+#define SLA_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SLA_OK 0
+#define SLA_ERR_BAD_ARG (-1)      /* null pointer, non-positive size, bad enum   */
+#define SLA_ERR_UNSUPPORTED (-2)  /* shape / block size / dtype not implemented   */
+#define SLA_ERR_LAUNCH (-3)       /* the HIP runtime refused a launch             */
+#define SLA_ERR_WORKSPACE (-4)    /* workspace smaller than sla_workspace_bytes   */
+
+/* element types */
+#define SLA_F32 0
+#define SLA_BF16 1
+#define SLA_F16 2
+
+/* feature maps of the linear branch (reference core.py:43-57) */
+#define SLA_FMAP_ELU 0
+#define SLA_FMAP_RELU 1
+#define SLA_FMAP_SOFTMAX 2
+
+/* operations that need a workspace */
+#define SLA_WS_BLOCK_MAP 0
+#define SLA_WS_SPARSE_BWD 1
+#define SLA_WS_LINEAR_FWD 2
+#define SLA_WS_LINEAR_BWD 3
+#define SLA_WS_SAGE_QUANT 4
+
+int sla_version(void);
+const char* sla_last_error(void);
+
+/* Bytes of caller-provided workspace an operation needs for the given problem.
+ * Returns a negative error code for unsupported arguments. */
+int64_t sla_workspace_bytes(int op, int dtype, int B, int H, int L, int D, int BLKQ, int BLKK, int topk);
+
+/* Per-block mean over rows: x (B*H, L, D) -> out (B*H, ceil(L/BLK), D), same dtype.
+ * Replaces mean_pool + compress_kernel, sparse_linear_attention/utils.py:21-52. */
+int sla_mean_pool(const void* x, void* out, int dtype, int BH, int L, int D, int BLK, void* stream);
+
+/* Block-mask builder: K mean smoothing, block pooling, pooled scores, per-row
+ * top-k (ties to the lowest index).  Writes the int8 0/1 map (B*H, M, N) and the
+ * ascending look-up table (B*H, M, topk) with elements of lut_elem_bytes (4 or 8).
+ * topk = min(N, int(ratio*N)) is computed by the caller.
+ * Replaces get_block_map, sparse_linear_attention/utils.py:55-67. */
+int sla_block_map_fwd(const void* q, const void* k, int dtype, int B, int H, int L, int D, int BLKQ, int BLKK,
+                      int topk, void* workspace, int64_t workspace_bytes, int8_t* sparse_map, void* lut,
+                      int lut_elem_bytes, void* stream);
+
+/* Block-sparse FlashAttention forward over the look-up table.
+ * o (B,H,L,D) in `dtype`, lse (B,H,L) fp32 = m + log2(l) in qk_scale*log2(e) units.
+ * BLKQ in {64,128}, BLKK == 64, D in {64,128}, dtype bf16 or f16.
+ * Replaces _attention.forward + _attn_fwd, sparse_linear_attention/kernel.py:21-82, 242-274. */
+int sla_sparse_attn_fwd(const void* q, const void* k, const void* v, const void* lut, int lut_elem_bytes,
+                        void* o, float* lse, int dtype, int B, int H, int L, int D, int BLKQ, int BLKK,
+                        int topk, float qk_scale, void* stream);
+
+/* Block-sparse FlashAttention backward: delta, dQ over the look-up table, dK/dV
+ * over per-key-block lists built from the int8 map.
+ * Replaces _attention.backward + _attn_bwd_preprocess/_dq/_dkdv,
+ * sparse_linear_attention/kernel.py:85-237, 277-320. */
+int sla_sparse_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o,
+                        const float* lse, const int8_t* sparse_map, const void* lut, int lut_elem_bytes,
+                        void* dq, void* dk, void* dv, int dtype, int B, int H, int L, int D, int BLKQ,
+                        int BLKK, int topk, float qk_scale, void* workspace, int64_t workspace_bytes,
+                        void* stream);
+
+/* Linear branch forward: feature maps, phi(K)^T V and sum phi(K) states, phi(Q) H / (1e-5 + phi(Q) z),
+ * projection by W (D,D) fp32 and bias (D) fp32, plus `residual` (the sparse output, may be null).
+ * out = residual + proj(o_l), in `dtype`.
+ * Replaces sparse_linear_attention/core.py:90-100 (feature maps, calc_linear, proj_l, sum). */
+int sla_linear_fwd(const void* q, const void* k, const void* v, const float* weight, const float* bias,
+                   const void* residual, void* out, int dtype, int fmap, int B, int H, int L, int D,
+                   void* workspace, int64_t workspace_bytes, void* stream);
+
+/* Linear branch backward.  d_out is the gradient of `out` above.  Writes dq, dk, dv in `dtype`
+ * (gradients of the linear branch only; the residual's gradient is d_out itself) and the
+ * fp32 gradients of weight (D,D) and bias (D).
+ * Replaces torch autograd through sparse_linear_attention/core.py:90-99. */
+int sla_linear_bwd(const void* q, const void* k, const void* v, const float* weight, const float* bias,
+                   const void* d_out, void* dq, void* dk, void* dv, float* d_weight, float* d_bias,
+                   int dtype, int fmap, int B, int H, int L, int D, void* workspace,
+                   int64_t workspace_bytes, void* stream);
+
+/* SageSLA: per-block INT8 quantisation of q (BLKQ rows) and of k - mean_L(k) (BLKK rows).
+ * q_int8, k_int8 (B,H,L,D) int8; q_scale (B,H,M) fp32; k_scale (B,H,N) fp32.
+ * Replaces k.mean + spas_sage_attn.utils.get_vanilla_qk_quant, SageSLA/core.py:102-108. */
+int sage_quant_qk(const void* q, const void* k, int dtype, int B, int H, int L, int D, int BLKQ, int BLKK,
+                  int8_t* q_int8, float* q_scale, int8_t* k_int8, float* k_scale, void* workspace,
+                  int64_t workspace_bytes, void* stream);
+
+/* SageSLA: per-channel FP8 e4m3 quantisation of v.  v_fp8 (B,H,L,D) e4m3fn bytes,
+ * v_scale (B,H,D) fp32 = max_L|v| / 448.
+ * Replaces spas_sage_attn._fused.transpose_pad_permute_cuda + scale_fuse_quant_cuda,
+ * SageSLA/core.py:123-129. */
+int sage_quant_v(const void* v, int dtype, int B, int H, int L, int D, uint8_t* v_fp8, float* v_scale,
+                 void* workspace, int64_t workspace_bytes, void* stream);
+
+/* SageSLA: quantised block-sparse attention, INT8 QK^T and FP8 PV on the matrix cores.
+ * Replaces spas_sage_attn.utils.block_map_lut_triton + _qattn.qk_int8_sv_f8_*,
+ * SageSLA/core.py:109, 136-144. */
+int sage_sparse_attn_fwd(const int8_t* q_int8, const float* q_scale, const int8_t* k_int8,
+                         const float* k_scale, const uint8_t* v_fp8, const float* v_scale, const void* lut,
+                         int lut_elem_bytes, void* o, int out_dtype, int B, int H, int L, int D, int BLKQ,
+                         int BLKK, int topk, float qk_scale, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SLA_HIP_H */

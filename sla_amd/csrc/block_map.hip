@@ -1,0 +1,338 @@
+// Block-mask builder for Sparse-Linear Attention on gfx950.
+//
+// Stands in for sparse_linear_attention/utils.py:21-67 of the reference:
+//   arg_k = k - mean_L(k); pooled_q = mean_pool(q, BLKQ); pooled_k = mean_pool(arg_k, BLKK);
+//   score = pooled_q @ pooled_k^T; lut = topk(score); map = scatter(lut).
+//
+// All of this is HBM-bound streaming or tiny, so it runs on the vector ALUs with a
+// FIXED fp32 summation order that a CPU checker can follow bit for bit:
+//   block mean : rows added one at a time in ascending order, one IEEE division;
+//   column mean: 64-row chunk sums (same order), chunk sums added in ascending order,
+//                one IEEE division by L;
+//   score      : acc = acc + (a_d * b_d), d ascending, no fused multiply-add.
+// Selection is by (score descending, index ascending); -0.0 == +0.0.
+#include "common.h"
+
+#pragma clang fp contract(off)
+
+namespace sla {
+
+constexpr int KMEAN_CHUNK = 64;
+
+struct IoF32 {
+  typedef float raw;
+  static constexpr int VEC = 4;
+  static __device__ __forceinline__ float ld(raw x) { return x; }
+  static __device__ __forceinline__ raw st(float x) { return x; }
+};
+struct IoBf16 {
+  typedef uint16_t raw;
+  static constexpr int VEC = 8;
+  static __device__ __forceinline__ float ld(raw x) { return Elem<bf16_tag>::to_float(x); }
+  static __device__ __forceinline__ raw st(float x) { return Elem<bf16_tag>::from_float(x); }
+};
+struct IoF16 {
+  typedef uint16_t raw;
+  static constexpr int VEC = 8;
+  static __device__ __forceinline__ float ld(raw x) { return Elem<f16_tag>::to_float(x); }
+  static __device__ __forceinline__ raw st(float x) { return Elem<f16_tag>::from_float(x); }
+};
+
+template <typename IO>
+struct alignas(16) Vec16 {
+  typename IO::raw e[IO::VEC];
+};
+
+// MODE 0: fp32 block sums (no division)        -> out_f32 (BH, nblk, D)
+// MODE 1: block mean in the input dtype        -> out     (BH, nblk, D)
+// MODE 2: block mean of round(x - colmean)     -> out     (BH, nblk, D)
+// One thread owns VEC adjacent columns of one block and walks its rows in order.
+template <typename IO, int MODE>
+__global__ __launch_bounds__(256) void pool_kernel(const typename IO::raw* __restrict__ x,
+                                                   const typename IO::raw* __restrict__ colmean,
+                                                   void* __restrict__ out, int L, int D, int BLK, int nblk) {
+  constexpr int VEC = IO::VEC;
+  const int tpr = D / VEC;
+  const int bpw = 256 / tpr;
+  const int bh = blockIdx.y;
+  const int sub = threadIdx.x / tpr;
+  const int blk = blockIdx.x * bpw + sub;
+  const int c = (threadIdx.x - sub * tpr) * VEC;
+  if (sub >= bpw || blk >= nblk) return;
+  const int row0 = blk * BLK;
+  const int nrows = min(BLK, L - row0);
+  float acc[VEC];
+  float cm[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
+  if (MODE == 2) {
+    Vec16<IO> m = *reinterpret_cast<const Vec16<IO>*>(colmean + (size_t)bh * D + c);
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) cm[e] = IO::ld(m.e[e]);
+  }
+  const typename IO::raw* p = x + ((size_t)bh * L + row0) * D + c;
+#pragma unroll 8
+  for (int r = 0; r < nrows; ++r) {
+    Vec16<IO> v = *reinterpret_cast<const Vec16<IO>*>(p + (size_t)r * D);
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      float f = IO::ld(v.e[e]);
+      if (MODE == 2) f = IO::ld(IO::st(f - cm[e]));
+      acc[e] = acc[e] + f;
+    }
+  }
+  const size_t o = ((size_t)bh * nblk + blk) * D + c;
+  if (MODE == 0) {
+    float* of = reinterpret_cast<float*>(out) + o;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) of[e] = acc[e];
+  } else {
+    const float cnt = (float)nrows;
+    Vec16<IO> r;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) r.e[e] = IO::st(acc[e] / cnt);
+    *reinterpret_cast<Vec16<IO>*>(reinterpret_cast<typename IO::raw*>(out) + o) = r;
+  }
+}
+
+// colmean[bh][d] = (sum over chunks, ascending) / L, rounded to the input dtype.
+template <typename IO>
+__global__ void colmean_kernel(const float* __restrict__ chunk_sums, typename IO::raw* __restrict__ colmean, int nchunk,
+                               int D, int L) {
+  const int bh = blockIdx.y;
+  const int d = blockIdx.x * blockDim.x + threadIdx.x;
+  if (d >= D) return;
+  const float* p = chunk_sums + (size_t)bh * nchunk * D + d;
+  float acc = 0.f;
+#pragma unroll 8
+  for (int i = 0; i < nchunk; ++i) acc = acc + p[(size_t)i * D];
+  colmean[(size_t)bh * D + d] = IO::st(acc / (float)L);
+}
+
+// score[bh][m][n] = round_dtype( sum_d pq[m][d]*pk[n][d] ), d ascending, mul and add rounded separately.
+// 64x64 outputs per workgroup, 4x4 per thread, operands staged through LDS 32 columns at a time.
+template <typename IO>
+__global__ __launch_bounds__(256) void score_kernel(const typename IO::raw* __restrict__ pq,
+                                                    const typename IO::raw* __restrict__ pk,
+                                                    typename IO::raw* __restrict__ score, int M, int N, int D) {
+  constexpr int TS = 64, DC = 32, LD = TS + 4;
+  __shared__ __attribute__((aligned(16))) float sa[DC][LD];
+  __shared__ __attribute__((aligned(16))) float sb[DC][LD];
+  const int bh = blockIdx.z;
+  const int m0 = blockIdx.y * TS, n0 = blockIdx.x * TS;
+  const int tid = threadIdx.x;
+  const int ty = tid >> 4, tx = tid & 15;
+  float acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+  const typename IO::raw* aq = pq + (size_t)bh * M * D;
+  const typename IO::raw* bk = pk + (size_t)bh * N * D;
+  for (int d0 = 0; d0 < D; d0 += DC) {
+    __syncthreads();
+    for (int idx = tid; idx < TS * DC; idx += 256) {
+      const int row = idx / DC, dd = idx % DC;
+      const bool dok = d0 + dd < D;
+      sa[dd][row] = (m0 + row < M && dok) ? IO::ld(aq[(size_t)(m0 + row) * D + d0 + dd]) : 0.f;
+      sb[dd][row] = (n0 + row < N && dok) ? IO::ld(bk[(size_t)(n0 + row) * D + d0 + dd]) : 0.f;
+    }
+    __syncthreads();
+    const int dn = min(DC, D - d0);
+    for (int dd = 0; dd < dn; ++dd) {
+      const f32x4_t a = *reinterpret_cast<const f32x4_t*>(&sa[dd][ty * 4]);
+      const f32x4_t b = *reinterpret_cast<const f32x4_t*>(&sb[dd][tx * 4]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float prod = a[i] * b[j];
+          acc[i][j] = acc[i][j] + prod;
+        }
+    }
+  }
+  typename IO::raw* out = score + (size_t)bh * M * N;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int m = m0 + ty * 4 + i;
+    if (m >= M) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + tx * 4 + j;
+      if (n < N) out[(size_t)m * N + n] = IO::st(acc[i][j]);
+    }
+  }
+}
+
+// Monotone map float -> uint32 (larger float = larger key); -0.0 is folded onto +0.0.
+static __device__ __forceinline__ uint32_t order_key(float f) {
+  uint32_t u = __float_as_uint(f);
+  if (u == 0x80000000u) u = 0u;
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+// One wavefront per (bh, m) row: radix-select the T-th largest key bit by bit with ballot
+// counts, then emit winners in ascending index order (ties at the threshold value go to
+// the lowest indices).  Writes the int8 map row and the look-up-table row.
+template <typename IO>
+__global__ __launch_bounds__(64) void topk_kernel(const typename IO::raw* __restrict__ score,
+                                                  int8_t* __restrict__ sparse_map, void* __restrict__ lut, int lut64, int N,
+                                                  int T) {
+  extern __shared__ uint32_t keys[];
+  const size_t row = blockIdx.x;
+  const int lane = threadIdx.x;
+  const typename IO::raw* s = score + row * N;
+  for (int i = lane; i < N; i += 64) keys[i] = order_key(IO::ld(s[i]));
+  __syncthreads();
+  uint32_t thr = 0;
+  for (int bit = 31; bit >= 0; --bit) {
+    const uint32_t cand = thr | (1u << bit);
+    int cnt = 0;
+    for (int i0 = 0; i0 < N; i0 += 64) {
+      const int i = i0 + lane;
+      const bool ge = (i < N) && (keys[i] >= cand);
+      cnt += __popcll(__ballot(ge));
+    }
+    if (cnt >= T) thr = cand;
+  }
+  int n_gt = 0;
+  for (int i0 = 0; i0 < N; i0 += 64) {
+    const int i = i0 + lane;
+    n_gt += __popcll(__ballot((i < N) && (keys[i] > thr)));
+  }
+  const int need_eq = T - n_gt;
+  int run_eq = 0, run_sel = 0;
+  const unsigned long long lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+  int8_t* mrow = sparse_map + row * N;
+  for (int i0 = 0; i0 < N; i0 += 64) {
+    const int i = i0 + lane;
+    const bool in = i < N;
+    const uint32_t kv = in ? keys[i] : 0u;
+    const bool gt = in && kv > thr;
+    const bool eq = in && kv == thr;
+    const unsigned long long beq = __ballot(eq);
+    const int eq_rank = run_eq + __popcll(beq & lt_mask);
+    const bool sel = gt || (eq && eq_rank < need_eq);
+    const unsigned long long bsel = __ballot(sel);
+    const int pos = run_sel + __popcll(bsel & lt_mask);
+    if (in) mrow[i] = sel ? 1 : 0;
+    if (sel) {
+      if (lut64)
+        reinterpret_cast<long long*>(lut)[row * T + pos] = i;
+      else
+        reinterpret_cast<int*>(lut)[row * T + pos] = i;
+    }
+    run_eq += __popcll(beq);
+    run_sel += __popcll(bsel);
+  }
+}
+
+struct MapWs {
+  size_t chunk_sums, colmean, pq, pk, score, total;
+};
+
+static MapWs map_ws(int dtype, int BH, int L, int D, int BLKQ, int BLKK) {
+  const int64_t M = cdiv(L, BLKQ), N = cdiv(L, BLKK), nchunk = cdiv(L, KMEAN_CHUNK);
+  const int64_t eb = elem_bytes(dtype);
+  MapWs w;
+  size_t off = 0;
+  w.chunk_sums = off; off += align_up((int64_t)BH * nchunk * D * 4, 256);
+  w.colmean = off;    off += align_up((int64_t)BH * D * eb, 256);
+  w.pq = off;         off += align_up((int64_t)BH * M * D * eb, 256);
+  w.pk = off;         off += align_up((int64_t)BH * N * D * eb, 256);
+  w.score = off;      off += align_up((int64_t)BH * M * N * eb, 256);
+  w.total = off;
+  return w;
+}
+
+int64_t block_map_workspace_bytes(int dtype, int BH, int L, int D, int BLKQ, int BLKK) {
+  return (int64_t)map_ws(dtype, BH, L, D, BLKQ, BLKK).total;
+}
+
+static int validate_pool(int dtype, int BH, int L, int D, int BLK) {
+  SLA_REQUIRE(dtype == SLA_F32 || dtype == SLA_BF16 || dtype == SLA_F16, SLA_ERR_BAD_ARG, "unknown dtype %d", dtype);
+  SLA_REQUIRE(BH > 0 && L > 0 && D > 0 && BLK > 0, SLA_ERR_BAD_ARG, "non-positive size (BH=%d L=%d D=%d BLK=%d)", BH, L,
+              D, BLK);
+  const int vec = dtype == SLA_F32 ? 4 : 8;
+  SLA_REQUIRE(D % vec == 0 && D / vec <= 256, SLA_ERR_UNSUPPORTED, "D=%d must be a multiple of %d and at most %d", D, vec,
+              256 * vec);
+  SLA_REQUIRE(BH <= 65535, SLA_ERR_UNSUPPORTED, "B*H=%d exceeds 65535", BH);
+  return SLA_OK;
+}
+
+template <typename IO, int MODE>
+static void launch_pool(const void* x, const void* colmean, void* out, int BH, int L, int D, int BLK, hipStream_t st) {
+  const int nblk = cdiv(L, BLK);
+  const int bpw = 256 / (D / IO::VEC);
+  dim3 grid(cdiv(nblk, bpw), BH);
+  hipLaunchKernelGGL((pool_kernel<IO, MODE>), grid, dim3(256), 0, st, (const typename IO::raw*)x,
+                     (const typename IO::raw*)colmean, out, L, D, BLK, nblk);
+}
+
+template <typename IO>
+static int block_map_impl(const void* q, const void* k, int dtype, int BH, int L, int D, int BLKQ, int BLKK, int topk,
+                          char* ws, int8_t* sparse_map, void* lut, int lut64, hipStream_t st) {
+  const MapWs w = map_ws(dtype, BH, L, D, BLKQ, BLKK);
+  const int M = cdiv(L, BLKQ), N = cdiv(L, BLKK), nchunk = cdiv(L, KMEAN_CHUNK);
+  float* chunk_sums = (float*)(ws + w.chunk_sums);
+  typename IO::raw* colmean = (typename IO::raw*)(ws + w.colmean);
+  typename IO::raw* pq = (typename IO::raw*)(ws + w.pq);
+  typename IO::raw* pk = (typename IO::raw*)(ws + w.pk);
+  typename IO::raw* score = (typename IO::raw*)(ws + w.score);
+  launch_pool<IO, 0>(k, nullptr, chunk_sums, BH, L, D, KMEAN_CHUNK, st);
+  hipLaunchKernelGGL((colmean_kernel<IO>), dim3(cdiv(D, 128), BH), dim3(128), 0, st, chunk_sums, colmean, nchunk, D, L);
+  launch_pool<IO, 1>(q, nullptr, pq, BH, L, D, BLKQ, st);
+  launch_pool<IO, 2>(k, colmean, pk, BH, L, D, BLKK, st);
+  hipLaunchKernelGGL((score_kernel<IO>), dim3(cdiv(N, 64), cdiv(M, 64), BH), dim3(256), 0, st, pq, pk, score, M, N, D);
+  // topk == 0 selects nothing: the kernel then only clears the map row.
+  hipLaunchKernelGGL((topk_kernel<IO>), dim3((unsigned)((size_t)BH * M)), dim3(64), (size_t)N * 4, st, score, sparse_map,
+                     lut, lut64, N, topk);
+  return check_launch("block map");
+}
+
+}  // namespace sla
+
+using namespace sla;
+
+extern "C" int sla_mean_pool(const void* x, void* out, int dtype, int BH, int L, int D, int BLK, void* stream) {
+  int rc = validate_pool(dtype, BH, L, D, BLK);
+  if (rc) return rc;
+  SLA_REQUIRE(x && out, SLA_ERR_BAD_ARG, "null pointer");
+  SLA_REQUIRE(((uintptr_t)x | (uintptr_t)out) % 16 == 0, SLA_ERR_BAD_ARG, "pointers must be 16-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == SLA_F32) launch_pool<IoF32, 1>(x, nullptr, out, BH, L, D, BLK, st);
+  else if (dtype == SLA_BF16) launch_pool<IoBf16, 1>(x, nullptr, out, BH, L, D, BLK, st);
+  else launch_pool<IoF16, 1>(x, nullptr, out, BH, L, D, BLK, st);
+  return check_launch("mean_pool");
+}
+
+extern "C" int sla_block_map_fwd(const void* q, const void* k, int dtype, int B, int H, int L, int D, int BLKQ, int BLKK,
+                                 int topk, void* workspace, int64_t workspace_bytes, int8_t* sparse_map, void* lut,
+                                 int lut_elem_bytes, void* stream) {
+  SLA_REQUIRE(B > 0 && H > 0, SLA_ERR_BAD_ARG, "non-positive batch/head count (B=%d H=%d)", B, H);
+  const int64_t BH64 = (int64_t)B * H;
+  SLA_REQUIRE(BH64 <= 65535, SLA_ERR_UNSUPPORTED, "B*H=%lld exceeds 65535", (long long)BH64);
+  const int BH = (int)BH64;
+  int rc = validate_pool(dtype, BH, L, D, BLKQ);
+  if (rc) return rc;
+  rc = validate_pool(dtype, BH, L, D, BLKK);
+  if (rc) return rc;
+  const int M = cdiv(L, BLKQ), N = cdiv(L, BLKK);
+  SLA_REQUIRE(topk >= 0 && topk <= N, SLA_ERR_BAD_ARG, "topk=%d outside [0, %d]", topk, N);
+  SLA_REQUIRE(N <= 32768, SLA_ERR_UNSUPPORTED, "more than 32768 key blocks (%d)", N);
+  SLA_REQUIRE((int64_t)BH * M < (1ll << 31), SLA_ERR_UNSUPPORTED, "too many query-block rows");
+  SLA_REQUIRE(lut_elem_bytes == 4 || lut_elem_bytes == 8, SLA_ERR_BAD_ARG, "lut_elem_bytes must be 4 or 8, got %d",
+              lut_elem_bytes);
+  SLA_REQUIRE(q && k && workspace && sparse_map && (lut || topk == 0), SLA_ERR_BAD_ARG, "null pointer");
+  SLA_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)workspace | (uintptr_t)lut) % 16 == 0, SLA_ERR_BAD_ARG,
+              "pointers must be 16-byte aligned");
+  const int64_t need = block_map_workspace_bytes(dtype, BH, L, D, BLKQ, BLKK);
+  SLA_REQUIRE(workspace_bytes >= need, SLA_ERR_WORKSPACE, "workspace of %lld bytes, need %lld", (long long)workspace_bytes,
+              (long long)need);
+  hipStream_t st = (hipStream_t)stream;
+  char* ws = (char*)workspace;
+  const int lut64 = lut_elem_bytes == 8;
+  if (dtype == SLA_F32) return block_map_impl<IoF32>(q, k, dtype, BH, L, D, BLKQ, BLKK, topk, ws, sparse_map, lut, lut64, st);
+  if (dtype == SLA_BF16) return block_map_impl<IoBf16>(q, k, dtype, BH, L, D, BLKQ, BLKK, topk, ws, sparse_map, lut, lut64, st);
+  return block_map_impl<IoF16>(q, k, dtype, BH, L, D, BLKQ, BLKK, topk, ws, sparse_map, lut, lut64, st);
+}

@@ -1,0 +1,60 @@
+// Library-wide pieces of the C ABI: version, error text, workspace sizes.
+#include "common.h"
+
+namespace sla {
+
+static thread_local char g_err[512] = "";
+
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+}
+
+int check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    set_error("%s: launch failed: %s", what, hipGetErrorString(e));
+    return SLA_ERR_LAUNCH;
+  }
+  return SLA_OK;
+}
+
+int64_t block_map_workspace_bytes(int dtype, int BH, int L, int D, int BLKQ, int BLKK);
+int64_t sparse_bwd_workspace_bytes(int BH, int L, int D, int BLKQ, int BLKK, int topk);
+int64_t linear_fwd_workspace_bytes(int BH, int L, int D);
+int64_t linear_bwd_workspace_bytes(int BH, int L, int D);
+int64_t sage_quant_workspace_bytes(int BH, int L, int D);
+
+}  // namespace sla
+
+using namespace sla;
+
+extern "C" int sla_version(void) { return 1; }
+
+extern "C" const char* sla_last_error(void) { return g_err; }
+
+extern "C" int64_t sla_workspace_bytes(int op, int dtype, int B, int H, int L, int D, int BLKQ, int BLKK, int topk) {
+  SLA_REQUIRE(B > 0 && H > 0 && L > 0 && D > 0, SLA_ERR_BAD_ARG, "non-positive size (B=%d H=%d L=%d D=%d)", B, H, L, D);
+  SLA_REQUIRE((int64_t)B * H <= 65535, SLA_ERR_UNSUPPORTED, "B*H exceeds 65535");
+  const int BH = B * H;
+  switch (op) {
+    case SLA_WS_BLOCK_MAP:
+      SLA_REQUIRE(BLKQ > 0 && BLKK > 0, SLA_ERR_BAD_ARG, "non-positive block size");
+      SLA_REQUIRE(dtype == SLA_F32 || dtype == SLA_BF16 || dtype == SLA_F16, SLA_ERR_BAD_ARG, "unknown dtype %d", dtype);
+      return block_map_workspace_bytes(dtype, BH, L, D, BLKQ, BLKK);
+    case SLA_WS_SPARSE_BWD:
+      SLA_REQUIRE(BLKQ > 0 && BLKK > 0 && topk >= 0, SLA_ERR_BAD_ARG, "bad block size / topk");
+      return sparse_bwd_workspace_bytes(BH, L, D, BLKQ, BLKK, topk);
+    case SLA_WS_LINEAR_FWD:
+      return linear_fwd_workspace_bytes(BH, L, D);
+    case SLA_WS_LINEAR_BWD:
+      return linear_bwd_workspace_bytes(BH, L, D);
+    case SLA_WS_SAGE_QUANT:
+      return sage_quant_workspace_bytes(BH, L, D);
+    default:
+      set_error("unknown workspace op %d", op);
+      return SLA_ERR_BAD_ARG;
+  }
+}

@@ -1,0 +1,93 @@
+"""HIP block-sparse attention forward vs the CPU oracle (bf16 tolerance 2e-2, cos >= 0.999)."""
+import pytest
+import torch
+
+from conftest import cos_sim, max_abs
+from oracle import sla_oracle as O
+from sla_amd import _attention
+from sla_amd.inputs import CONFIGS, make_inputs
+
+pytestmark = pytest.mark.gpu
+
+TOL_ABS = 2e-2      # stated by the task for bf16 outputs
+TOL_COS = 0.999
+LN2 = 0.6931471805599453
+
+
+def _run(q, k, v, lut, sparse_map, T, BLKQ, dev, lut_dtype=torch.int64):
+    o = _attention.apply(q.to(dev), k.to(dev), v.to(dev), sparse_map.to(dev), lut.to(lut_dtype).to(dev), T, BLKQ, 64)
+    torch.cuda.synchronize()
+    return o.cpu()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("L,D,BLKQ,ratio", [(512, 128, 64, 0.25), (1000, 128, 64, 0.3), (777, 128, 128, 0.4),
+                                            (640, 64, 64, 0.5), (333, 64, 128, 0.34), (64, 128, 64, 1.0),
+                                            (50, 128, 64, 1.0)])
+def test_against_dense_oracle(dev, dtype, L, D, BLKQ, ratio):
+    g = torch.Generator().manual_seed(L + D)
+    q = torch.randn(1, 3, L, D, generator=g).to(dtype)
+    k = torch.randn(1, 3, L, D, generator=g).to(dtype)
+    v = torch.randn(1, 3, L, D, generator=g).to(dtype)
+    m, lut, T = O.get_block_map(q, k, ratio, BLKQ, 64)
+    o_ref, lse_ref = O.sparse_attn_fwd_dense(q, k, v, m, BLKQ, 64)
+    o = _run(q, k, v, lut, m, T, BLKQ, dev)
+    assert o.dtype == dtype
+    assert max_abs(o, o_ref) <= TOL_ABS
+    assert cos_sim(o, o_ref) >= TOL_COS
+
+
+def test_full_selection_equals_sdpa(dev):
+    g = torch.Generator().manual_seed(11)
+    q, k, v = (torch.randn(2, 2, 300, 128, generator=g).to(torch.bfloat16) for _ in range(3))
+    N = (300 + 63) // 64
+    lut = torch.arange(N).expand(2, 2, N, N).contiguous()
+    m = torch.ones(2, 2, N, N, dtype=torch.int8)
+    ref = torch.nn.functional.scaled_dot_product_attention(q.double(), k.double(), v.double())
+    o = _run(q, k, v, lut, m, N, 64, dev)
+    assert max_abs(o, ref) <= TOL_ABS and cos_sim(o, ref) >= TOL_COS
+
+
+def test_lut_order_and_int32(dev):
+    g = torch.Generator().manual_seed(12)
+    q, k, v = (torch.randn(1, 2, 1024, 128, generator=g).to(torch.bfloat16) for _ in range(3))
+    m, lut, T = O.get_block_map(q, k, 0.25, 64, 64)
+    o1 = _run(q, k, v, lut, m, T, 64, dev)
+    o2 = _run(q, k, v, lut.flip(-1).contiguous(), m, T, 64, dev, lut_dtype=torch.int32)
+    o_ref, _ = O.sparse_attn_fwd_dense(q, k, v, m, 64, 64)
+    assert max_abs(o1, o_ref) <= TOL_ABS and max_abs(o2, o_ref) <= TOL_ABS
+    assert max_abs(o1, o2) <= 1e-2
+
+
+def test_lse_and_determinism(dev):
+    from sla_amd.sparse_attn import sparse_attn_fwd
+    g = torch.Generator().manual_seed(13)
+    q, k, v = (torch.randn(1, 2, 1000, 128, generator=g).to(torch.bfloat16) for _ in range(3))
+    m, lut, T = O.get_block_map(q, k, 0.2, 64, 64)
+    _, lse_ref = O.sparse_attn_fwd_dense(q, k, v, m, 64, 64)
+    o1, lse1 = sparse_attn_fwd(q.to(dev), k.to(dev), v.to(dev), lut.to(dev), T, 64, 64, 128 ** -0.5)
+    o2, lse2 = sparse_attn_fwd(q.to(dev), k.to(dev), v.to(dev), lut.to(dev), T, 64, 64, 128 ** -0.5)
+    assert torch.equal(o1, o2) and torch.equal(lse1, lse2)
+    assert max_abs(lse1.cpu(), lse_ref) <= 1e-3
+    # lse * ln2 is the natural-log logsumexp of the scaled selected scores
+    s = (q.double() @ k.double().transpose(-1, -2)) * 128 ** -0.5
+    s = s.masked_fill(~O.expand_block_map(m, 1000, 64, 64), float("-inf"))
+    assert max_abs(lse1.cpu() * LN2, torch.logsumexp(s, -1)) <= 1e-3
+
+
+def test_cfg2_forward(dev):
+    cfg = CONFIGS["cfg2"]
+    d = make_inputs(cfg)
+    m, lut, T = O.get_block_map(d["q"], d["k"], cfg.topk, 64, 64)
+    o_ref, _ = O.sparse_attn_fwd_gather(d["q"], d["k"], d["v"], lut, 64, 64)
+    o = _run(d["q"], d["k"], d["v"], lut, m, T, 64, dev)
+    assert max_abs(o, o_ref) <= TOL_ABS and cos_sim(o, o_ref) >= TOL_COS
+
+
+def test_cfg3_two_heads_forward(dev):
+    cfg = CONFIGS["cfg3"]
+    d = make_inputs(cfg, H=2)
+    m, lut, T = O.get_block_map(d["q"], d["k"], cfg.topk, 64, 64)
+    o_ref, _ = O.sparse_attn_fwd_gather(d["q"], d["k"], d["v"], lut, 64, 64)
+    o = _run(d["q"], d["k"], d["v"], lut, m, T, 64, dev)
+    assert max_abs(o, o_ref) <= TOL_ABS and cos_sim(o, o_ref) >= TOL_COS
