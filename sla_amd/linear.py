@@ -1,0 +1,60 @@
+"""Host side of the linear-attention branch + projection + sum.
+
+Replaces the eager block of ``sparse_linear_attention/core.py:90-100`` (feature
+maps, ``calc_linear``, ``proj_l`` under autocast, ``o_s + o_l``) with one fused
+operator: ``out = residual + proj_l(calc_linear(phi(q), phi(k), v))``.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+
+
+def linear_fwd(q, k, v, weight, bias, residual, fmap: str):
+    _lib.require_gpu(q, k, v, weight, bias)
+    B, H, L, D = q.shape
+    dt = _lib.dtype_code(q.dtype)
+    ws = _lib.workspace(_lib.WS_LINEAR_FWD, dt, B, H, L, D, 64, 64, 0, q.device)
+    out = torch.empty_like(q)
+    rc = _lib.load().sla_linear_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), weight.data_ptr(), bias.data_ptr(),
+                                    0 if residual is None else residual.data_ptr(), out.data_ptr(), dt,
+                                    _lib.FMAP[fmap], B, H, L, D, ws.data_ptr(), ws.numel(), _lib.stream_ptr(q.device))
+    _lib.check(rc)
+    return out
+
+
+def linear_bwd(q, k, v, weight, bias, d_out, fmap: str):
+    B, H, L, D = q.shape
+    dt = _lib.dtype_code(q.dtype)
+    ws = _lib.workspace(_lib.WS_LINEAR_BWD, dt, B, H, L, D, 64, 64, 0, q.device)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    dw = torch.empty((D, D), dtype=torch.float32, device=q.device)
+    db = torch.empty((D,), dtype=torch.float32, device=q.device)
+    rc = _lib.load().sla_linear_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), weight.data_ptr(), bias.data_ptr(),
+                                    d_out.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), dw.data_ptr(),
+                                    db.data_ptr(), dt, _lib.FMAP[fmap], B, H, L, D, ws.data_ptr(), ws.numel(),
+                                    _lib.stream_ptr(q.device))
+    _lib.check(rc)
+    return dq, dk, dv, dw, db
+
+
+class _linear_proj_add(torch.autograd.Function):
+    """out = residual + proj(calc_linear(phi(q), phi(k), v)); weight/bias are the fp32 ``proj_l`` parameters."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, weight, bias, residual, fmap):
+        weight = weight.contiguous()
+        bias = bias.contiguous()
+        out = linear_fwd(q, k, v, weight, bias, residual, fmap)
+        ctx.save_for_backward(q, k, v, weight, bias)
+        ctx.fmap = fmap
+        ctx.has_residual = residual is not None
+        return out
+
+    @staticmethod
+    def backward(ctx, d_out):
+        q, k, v, weight, bias = ctx.saved_tensors
+        d_out = d_out.contiguous()
+        dq, dk, dv, dw, db = linear_bwd(q, k, v, weight, bias, d_out, ctx.fmap)
+        return dq, dk, dv, dw, db, (d_out if ctx.has_residual else None), None

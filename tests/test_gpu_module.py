@@ -1,0 +1,77 @@
+"""Whole-module forward (mask -> sparse -> linear -> proj -> sum) vs the CPU oracle."""
+import pytest
+import torch
+
+from conftest import cos_sim, max_abs
+from oracle import sla_oracle as O
+from sla_amd import SparseLinearAttention
+from sla_amd.inputs import CONFIGS, make_inputs, make_proj
+
+pytestmark = pytest.mark.gpu
+
+TOL_ABS = 2e-2
+TOL_COS = 0.999
+
+
+def _module(cfg, dev, seeded=True):
+    mod = SparseLinearAttention(cfg.D, cfg.topk, cfg.feature_map, cfg.BLKQ, cfg.BLKK).to(dev)
+    w, b = make_proj(cfg.D)
+    if seeded:
+        with torch.no_grad():
+            mod.proj_l.weight.copy_(w)
+            mod.proj_l.bias.copy_(b)
+    else:
+        w, b = torch.zeros_like(w), torch.zeros_like(b)
+    return mod, w, b
+
+
+def test_cfg1_fp32_inputs(dev):
+    cfg = CONFIGS["cfg1"]
+    d = make_inputs(cfg)
+    for seeded in (False, True):
+        mod, w, b = _module(cfg, dev, seeded)
+        o_ref, o_s, o_l, m, lut, T = O.sla_forward(d["q"], d["k"], d["v"], w, b, cfg.topk, cfg.feature_map,
+                                                   linear_dtype=torch.float32)
+        o, dens = mod(d["q"].to(dev), d["k"].to(dev), d["v"].to(dev), return_sparsity=True)
+        assert o.dtype == torch.float32 and dens == T / m.shape[-1] == 3 / 16
+        assert max_abs(o.cpu(), o_ref) <= TOL_ABS and cos_sim(o.cpu(), o_ref) >= TOL_COS
+
+
+def test_cfg2_forward(dev):
+    cfg = CONFIGS["cfg2"]
+    d = make_inputs(cfg)
+    mod, w, b = _module(cfg, dev)
+    o_ref, *_ = O.sla_forward(d["q"], d["k"], d["v"], w, b, cfg.topk, cfg.feature_map, linear_dtype=torch.float32)
+    o = mod(d["q"].to(dev), d["k"].to(dev), d["v"].to(dev)).cpu()
+    assert o.dtype == torch.bfloat16
+    assert max_abs(o, o_ref) <= TOL_ABS and cos_sim(o, o_ref) >= TOL_COS
+
+
+def test_zero_init_module_returns_sparse_branch(dev):
+    cfg = CONFIGS["cfg2"]
+    d = make_inputs(cfg)
+    mod, _, _ = _module(cfg, dev, seeded=False)
+    from sla_amd import _attention, get_block_map
+    q, k, v = (d[x].to(dev) for x in "qkv")
+    m, lut, T = get_block_map(q, k, cfg.topk)
+    o_s = _attention.apply(q, k, v, m, lut, T, 64, 64)
+    assert torch.equal(mod(q, k, v), o_s)
+
+
+def test_state_dict_layout_and_errors(dev):
+    mod = SparseLinearAttention(128, 0.2)
+    sd = mod.state_dict()
+    assert set(sd) == {"proj_l.weight", "proj_l.bias"}
+    assert sd["proj_l.weight"].shape == (128, 128) and sd["proj_l.weight"].dtype == torch.float32
+    assert float(sd["proj_l.weight"].abs().max()) == 0.0 and float(sd["proj_l.bias"].abs().max()) == 0.0
+    with pytest.raises(NotImplementedError):
+        SparseLinearAttention(128, 0.2, feature_map="hedgehog")
+
+
+def test_cfg3_three_heads_forward(dev):
+    cfg = CONFIGS["cfg3"]
+    d = make_inputs(cfg, H=3)
+    mod, w, b = _module(cfg, dev)
+    o_ref, *_ = O.sla_forward(d["q"], d["k"], d["v"], w, b, cfg.topk, cfg.feature_map, linear_dtype=torch.float32)
+    o = mod(d["q"].to(dev), d["k"].to(dev), d["v"].to(dev)).cpu()
+    assert max_abs(o, o_ref) <= TOL_ABS and cos_sim(o, o_ref) >= TOL_COS
