@@ -1,0 +1,485 @@
+// Block-sparse FlashAttention backward for gfx950.
+//
+// Stands in for _attn_bwd_preprocess, _attn_bwd_dq, _attn_bwd_dkdv and _attention.backward of
+// the reference (sparse_linear_attention/kernel.py:85-237, 277-320):
+//   delta = rowsum(o * do)
+//   P = exp2(S*c - lse) on the selected blocks, dP = dO V^T, dS = P * (dP - delta)
+//   dQ = scale * dS K ; dK = scale * dS^T Q ; dV = P^T dO
+//
+// Four kernels.
+//   delta      : one pass over o and do.
+//   col_lists  : the reference scans the dense int8 map column in the dK/dV kernel (about
+//                1/density wasted iterations); here the map is turned once into per-key-block
+//                lists of the query blocks that selected it.
+//   dq         : per query block over its look-up table, products formed transposed as in the
+//                forward (S^T = K Q^T, dP^T = V dO^T) so lse and delta are per-lane scalars and
+//                dS^T leaves the accumulator in B-operand layout for dQ^T += K^T dS^T (K^T is
+//                read from LDS with the transposing read).
+//   dkdv       : per key block over its list; S = Q K^T and dP = dO V^T with K^T/V^T resident
+//                in registers as B operands; P and dS leave the accumulators in B-operand layout
+//                for dV^T += dO^T P and dK^T += Q^T dS (Q^T, dO^T via transposing LDS reads).
+#include "common.h"
+
+namespace sla {
+
+int validate_attn_shape(int dtype, int B, int H, int L, int D, int BLKQ, int BLKK, int topk, int lut_elem_bytes);
+
+// ---- delta ------------------------------------------------------------------------------
+template <typename Tag, int D>
+__global__ __launch_bounds__(256) void bwd_delta_kernel(const uint16_t* __restrict__ o, const uint16_t* __restrict__ d_o,
+                                                        float* __restrict__ delta, size_t rows) {
+  using E = Elem<Tag>;
+  constexpr int CPR = D / 8;
+  const size_t row = (size_t)blockIdx.x * (256 / CPR) + threadIdx.x / CPR;
+  const int col = (threadIdx.x % CPR) * 8;
+  float s = 0.f;
+  if (row < rows) {
+    const i16x8_t a = *reinterpret_cast<const i16x8_t*>(o + row * D + col);
+    const i16x8_t b = *reinterpret_cast<const i16x8_t*>(d_o + row * D + col);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) s += E::to_float((uint16_t)a[e]) * E::to_float((uint16_t)b[e]);
+  }
+#pragma unroll
+  for (int sh = 1; sh < CPR; sh <<= 1) s += __shfl_xor(s, sh);
+  if (row < rows && col == 0) delta[row] = s;
+}
+
+// ---- per-key-block lists ------------------------------------------------------------------
+// One thread per key block n walks the rows of the map; list[bh][n][0..count) holds the
+// selecting query blocks in ascending order.  Capacity Mblk per list (only count entries are
+// ever touched).
+__global__ __launch_bounds__(64) void bwd_col_lists_kernel(const int8_t* __restrict__ sparse_map, int* __restrict__ list,
+                                                           int* __restrict__ count, int Mblk, int Nblk) {
+  const int bh = blockIdx.y;
+  const int n = blockIdx.x * 64 + threadIdx.x;
+  if (n >= Nblk) return;
+  const int8_t* col = sparse_map + (size_t)bh * Mblk * Nblk + n;
+  int* out = list + ((size_t)bh * Nblk + n) * Mblk;
+  int c = 0;
+#pragma unroll 8
+  for (int m = 0; m < Mblk; ++m) {
+    if (col[(size_t)m * Nblk] == 1) out[c++] = m;
+  }
+  count[(size_t)bh * Nblk + n] = c;
+}
+
+// ---- dQ ---------------------------------------------------------------------------------
+template <typename Tag, int D, int BLKQ>
+__global__ __launch_bounds__(BLKQ * 2) void bwd_dq_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ k,
+                                                          const uint16_t* __restrict__ v, const uint16_t* __restrict__ d_o,
+                                                          const float* __restrict__ lse, const float* __restrict__ delta,
+                                                          const void* __restrict__ lut, int lut64, uint16_t* __restrict__ dq,
+                                                          int L, int Mblk, int topk, float qk_scale, int total) {
+  using E = Elem<Tag>;
+  constexpr int BLKK = 64;
+  constexpr int NT = BLKQ * 2;
+  constexpr int DC = D / 16;
+  constexpr int DT = D / 32;
+  constexpr int KSTR = D + 16;   // K is read both row-wise and transposed
+  constexpr int VSTR = D + 8;
+  constexpr int CPR = D / 8;
+  constexpr int NLD = BLKK * CPR / NT;
+
+  __shared__ __attribute__((aligned(16))) uint16_t sK[BLKK * KSTR];
+  __shared__ __attribute__((aligned(16))) uint16_t sV[BLKK * VSTR];
+
+  const int logical = xcd_remap(blockIdx.x, gridDim.x, total);
+  if (logical < 0) return;
+  const int bh = logical / Mblk;
+  const int mb = logical - bh * Mblk;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int g = lane >> 5, r = lane & 31;
+  const float c_log2e = qk_scale * 1.4426950408889634f;
+
+  const size_t head_off = (size_t)bh * L * D;
+  const uint16_t* kh = k + head_off;
+  const uint16_t* vh = v + head_off;
+  const int qrow = mb * BLKQ + wave * 32 + r;
+  const bool qok = qrow < L;
+
+  i16x8_t qf[DC], dof[DC];
+#pragma unroll
+  for (int c = 0; c < DC; ++c) {
+    qf[c] = i16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+    dof[c] = i16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+    if (qok) {
+      qf[c] = *reinterpret_cast<const i16x8_t*>(q + head_off + (size_t)qrow * D + 16 * c + 8 * g);
+      dof[c] = *reinterpret_cast<const i16x8_t*>(d_o + head_off + (size_t)qrow * D + 16 * c + 8 * g);
+    }
+  }
+  // rows past L: lse = +inf makes every probability exactly 0 (the reference loads `other=inf`)
+  const float lse_q = qok ? lse[(size_t)bh * L + qrow] : INFINITY;
+  const float delta_q = qok ? delta[(size_t)bh * L + qrow] : 0.f;
+
+  const size_t lut_row = ((size_t)bh * Mblk + mb) * topk;
+  auto lut_at = [&](int i) -> int {
+    return lut64 ? (int)reinterpret_cast<const long long*>(lut)[lut_row + i]
+                 : reinterpret_cast<const int*>(lut)[lut_row + i];
+  };
+  i16x8_t kreg[NLD], vreg[NLD];
+  auto load_tile = [&](int nb) {
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) {
+      const int idx = tid + i * NT;
+      const int row = idx / CPR, col = (idx % CPR) * 8;
+      const int grow = nb * BLKK + row;
+      kreg[i] = i16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+      vreg[i] = i16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+      if (grow < L) {
+        kreg[i] = *reinterpret_cast<const i16x8_t*>(kh + (size_t)grow * D + col);
+        vreg[i] = *reinterpret_cast<const i16x8_t*>(vh + (size_t)grow * D + col);
+      }
+    }
+  };
+  auto store_tile = [&]() {
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) {
+      const int idx = tid + i * NT;
+      const int row = idx / CPR, col = (idx % CPR) * 8;
+      *reinterpret_cast<i16x8_t*>(&sK[row * KSTR + col]) = kreg[i];
+      *reinterpret_cast<i16x8_t*>(&sV[row * VSTR + col]) = vreg[i];
+    }
+  };
+
+  f32x16_t dqacc[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) dqacc[dt][i] = 0.f;
+
+  const int tr_row = (lane & 15) >> 2;
+  const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+
+  int nb = topk > 0 ? lut_at(0) : 0;
+  if (topk > 0) load_tile(nb);
+  for (int it = 0; it < topk; ++it) {
+    __syncthreads();
+    store_tile();
+    __syncthreads();
+    const int kv_valid = L - nb * BLKK;
+    if (it + 1 < topk) {
+      nb = lut_at(it + 1);
+      load_tile(nb);
+    }
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      f32x16_t s, dp;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        s[i] = 0.f;
+        dp[i] = 0.f;
+      }
+#pragma unroll
+      for (int c = 0; c < DC; ++c) {
+        const i16x8_t a = *reinterpret_cast<const i16x8_t*>(&sK[(32 * t + r) * KSTR + 16 * c + 8 * g]);
+        s = E::mfma32(a, qf[c], s);
+      }
+#pragma unroll
+      for (int c = 0; c < DC; ++c) {
+        const i16x8_t a = *reinterpret_cast<const i16x8_t*>(&sV[(32 * t + r) * VSTR + 16 * c + 8 * g]);
+        dp = E::mfma32(a, dof[c], dp);
+      }
+      // dS^T = P^T * (dP^T - delta), zero on key rows past L
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int key = 32 * t + 8 * (i >> 2) + 4 * g + (i & 3);
+        float p = fast_exp2(__builtin_fmaf(s[i], c_log2e, -lse_q));
+        if (key >= kv_valid) p = 0.f;
+        s[i] = p * (dp[i] - delta_q);
+      }
+#pragma unroll
+      for (int c2 = 0; c2 < 2; ++c2) {
+        i32x4_t pw;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) pw[j] = (int)E::pack2(s[8 * c2 + 2 * j], s[8 * c2 + 2 * j + 1]);
+        const i16x8_t dsb = __builtin_bit_cast(i16x8_t, pw);
+        const int key0 = 32 * t + 16 * c2 + 4 * g + tr_row;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          const uint16_t* p0 = &sK[key0 * KSTR + 32 * dt + tr_col];
+          dqacc[dt] = E::mfma32(concat4(lds_read_tr16(p0), lds_read_tr16(p0 + 8 * KSTR)), dsb, dqacc[dt]);
+        }
+      }
+    }
+  }
+  if (qok) {
+    uint16_t* orow = dq + head_off + (size_t)qrow * D;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; ++i4) {
+        i32x2_t w;
+        w[0] = (int)E::pack2(dqacc[dt][4 * i4 + 0] * qk_scale, dqacc[dt][4 * i4 + 1] * qk_scale);
+        w[1] = (int)E::pack2(dqacc[dt][4 * i4 + 2] * qk_scale, dqacc[dt][4 * i4 + 3] * qk_scale);
+        *reinterpret_cast<i32x2_t*>(orow + 32 * dt + 8 * i4 + 4 * g) = w;
+      }
+  }
+}
+
+// ---- dK, dV -----------------------------------------------------------------------------
+// One workgroup (2 waves) per key block; wave w owns keys 32w..32w+31 of it.
+template <typename Tag, int D, int BLKQ>
+__global__ __launch_bounds__(128) void bwd_dkdv_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ k,
+                                                       const uint16_t* __restrict__ v, const uint16_t* __restrict__ d_o,
+                                                       const float* __restrict__ lse, const float* __restrict__ delta,
+                                                       const int* __restrict__ list, const int* __restrict__ count,
+                                                       uint16_t* __restrict__ dk, uint16_t* __restrict__ dv, int L, int Mblk,
+                                                       int Nblk, float qk_scale, int total) {
+  using E = Elem<Tag>;
+  constexpr int TQ = 64;                  // query rows per LDS tile
+  constexpr int SUB = BLKQ / TQ;          // tiles per listed query block
+  constexpr int NT = 128;
+  constexpr int DC = D / 16;
+  constexpr int DT = D / 32;
+  constexpr int STR = D + 16;             // Q and dO are read row-wise and transposed
+  constexpr int CPR = D / 8;
+  constexpr int NLD = TQ * CPR / NT;
+
+  __shared__ __attribute__((aligned(16))) uint16_t sQ[TQ * STR];
+  __shared__ __attribute__((aligned(16))) uint16_t sDO[TQ * STR];
+  __shared__ __attribute__((aligned(16))) float sLse[TQ];
+  __shared__ __attribute__((aligned(16))) float sDelta[TQ];
+
+  const int logical = xcd_remap(blockIdx.x, gridDim.x, total);
+  if (logical < 0) return;
+  const int bh = logical / Nblk;
+  const int nb = logical - bh * Nblk;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int g = lane >> 5, r = lane & 31;
+  const float c_log2e = qk_scale * 1.4426950408889634f;
+
+  const size_t head_off = (size_t)bh * L * D;
+  const uint16_t* qh = q + head_off;
+  const uint16_t* doh = d_o + head_off;
+  const float* lseh = lse + (size_t)bh * L;
+  const float* deltah = delta + (size_t)bh * L;
+
+  // K^T and V^T fragments (B operands): this lane's key column, 8 adjacent d per chunk
+  const int krow = nb * 64 + wave * 32 + r;
+  const bool kok = krow < L;
+  i16x8_t kf[DC], vf[DC];
+#pragma unroll
+  for (int c = 0; c < DC; ++c) {
+    kf[c] = i16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+    vf[c] = i16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+    if (kok) {
+      kf[c] = *reinterpret_cast<const i16x8_t*>(k + head_off + (size_t)krow * D + 16 * c + 8 * g);
+      vf[c] = *reinterpret_cast<const i16x8_t*>(v + head_off + (size_t)krow * D + 16 * c + 8 * g);
+    }
+  }
+
+  f32x16_t dkacc[DT], dvacc[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      dkacc[dt][i] = 0.f;
+      dvacc[dt][i] = 0.f;
+    }
+
+  const int* mylist = list + ((size_t)bh * Nblk + nb) * Mblk;
+  const int ntile = count[(size_t)bh * Nblk + nb] * SUB;
+
+  i16x8_t qreg[NLD], doreg[NLD];
+  float lreg = 0.f, dreg = 0.f;
+  auto tile_row0 = [&](int ti) -> int { return mylist[ti / SUB] * BLKQ + (ti % SUB) * TQ; };
+  auto load_tile = [&](int row0) {
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) {
+      const int idx = tid + i * NT;
+      const int row = idx / CPR, col = (idx % CPR) * 8;
+      const int grow = row0 + row;
+      qreg[i] = i16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+      doreg[i] = i16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+      if (grow < L) {
+        qreg[i] = *reinterpret_cast<const i16x8_t*>(qh + (size_t)grow * D + col);
+        doreg[i] = *reinterpret_cast<const i16x8_t*>(doh + (size_t)grow * D + col);
+      }
+    }
+    if (tid < TQ) {
+      const int grow = row0 + tid;
+      lreg = grow < L ? lseh[grow] : INFINITY;     // +inf -> probability 0 for rows past L
+      dreg = grow < L ? deltah[grow] : 0.f;
+    }
+  };
+  auto store_tile = [&]() {
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) {
+      const int idx = tid + i * NT;
+      const int row = idx / CPR, col = (idx % CPR) * 8;
+      *reinterpret_cast<i16x8_t*>(&sQ[row * STR + col]) = qreg[i];
+      *reinterpret_cast<i16x8_t*>(&sDO[row * STR + col]) = doreg[i];
+    }
+    if (tid < TQ) {
+      sLse[tid] = lreg;
+      sDelta[tid] = dreg;
+    }
+  };
+
+  const int tr_row = (lane & 15) >> 2;
+  const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+
+  if (ntile > 0) load_tile(tile_row0(0));
+  for (int ti = 0; ti < ntile; ++ti) {
+    __syncthreads();
+    store_tile();
+    __syncthreads();
+    if (ti + 1 < ntile) load_tile(tile_row0(ti + 1));
+#pragma unroll
+    for (int t = 0; t < TQ / 32; ++t) {
+      f32x16_t s, dp;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        s[i] = 0.f;
+        dp[i] = 0.f;
+      }
+#pragma unroll
+      for (int c = 0; c < DC; ++c) {
+        const i16x8_t a = *reinterpret_cast<const i16x8_t*>(&sQ[(32 * t + r) * STR + 16 * c + 8 * g]);
+        s = E::mfma32(a, kf[c], s);
+      }
+#pragma unroll
+      for (int c = 0; c < DC; ++c) {
+        const i16x8_t a = *reinterpret_cast<const i16x8_t*>(&sDO[(32 * t + r) * STR + 16 * c + 8 * g]);
+        dp = E::mfma32(a, vf[c], dp);
+      }
+      // accumulator rows are queries 32t + 8*(i/4) + 4g + i%4; this lane's column is its key
+#pragma unroll
+      for (int i4 = 0; i4 < 4; ++i4) {
+        const f32x4_t l4 = *reinterpret_cast<const f32x4_t*>(&sLse[32 * t + 8 * i4 + 4 * g]);
+        const f32x4_t d4 = *reinterpret_cast<const f32x4_t*>(&sDelta[32 * t + 8 * i4 + 4 * g]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int i = 4 * i4 + j;
+          float p = fast_exp2(__builtin_fmaf(s[i], c_log2e, -l4[j]));
+          if (!kok) p = 0.f;
+          s[i] = p;
+          dp[i] = p * (dp[i] - d4[j]);
+        }
+      }
+#pragma unroll
+      for (int c2 = 0; c2 < 2; ++c2) {
+        i32x4_t pw, dw;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          pw[j] = (int)E::pack2(s[8 * c2 + 2 * j], s[8 * c2 + 2 * j + 1]);
+          dw[j] = (int)E::pack2(dp[8 * c2 + 2 * j], dp[8 * c2 + 2 * j + 1]);
+        }
+        const i16x8_t pb = __builtin_bit_cast(i16x8_t, pw);
+        const i16x8_t dsb = __builtin_bit_cast(i16x8_t, dw);
+        const int q0 = 32 * t + 16 * c2 + 4 * g + tr_row;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          const uint16_t* pdo = &sDO[q0 * STR + 32 * dt + tr_col];
+          dvacc[dt] = E::mfma32(concat4(lds_read_tr16(pdo), lds_read_tr16(pdo + 8 * STR)), pb, dvacc[dt]);
+          const uint16_t* pq = &sQ[q0 * STR + 32 * dt + tr_col];
+          dkacc[dt] = E::mfma32(concat4(lds_read_tr16(pq), lds_read_tr16(pq + 8 * STR)), dsb, dkacc[dt]);
+        }
+      }
+    }
+  }
+  if (kok) {
+    uint16_t* dkrow = dk + head_off + (size_t)krow * D;
+    uint16_t* dvrow = dv + head_off + (size_t)krow * D;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; ++i4) {
+        i32x2_t w;
+        w[0] = (int)E::pack2(dkacc[dt][4 * i4 + 0] * qk_scale, dkacc[dt][4 * i4 + 1] * qk_scale);
+        w[1] = (int)E::pack2(dkacc[dt][4 * i4 + 2] * qk_scale, dkacc[dt][4 * i4 + 3] * qk_scale);
+        *reinterpret_cast<i32x2_t*>(dkrow + 32 * dt + 8 * i4 + 4 * g) = w;
+        w[0] = (int)E::pack2(dvacc[dt][4 * i4 + 0], dvacc[dt][4 * i4 + 1]);
+        w[1] = (int)E::pack2(dvacc[dt][4 * i4 + 2], dvacc[dt][4 * i4 + 3]);
+        *reinterpret_cast<i32x2_t*>(dvrow + 32 * dt + 8 * i4 + 4 * g) = w;
+      }
+  }
+}
+
+// ---- host ---------------------------------------------------------------------------------
+struct BwdWs {
+  size_t delta, count, list, total;
+};
+static BwdWs bwd_ws(int BH, int L, int BLKQ, int BLKK) {
+  const int64_t M = cdiv(L, BLKQ), N = cdiv(L, BLKK);
+  BwdWs w;
+  size_t off = 0;
+  w.delta = off; off += align_up((int64_t)BH * L * 4, 256);
+  w.count = off; off += align_up((int64_t)BH * N * 4, 256);
+  w.list = off;  off += align_up((int64_t)BH * N * M * 4, 256);
+  w.total = off;
+  return w;
+}
+int64_t sparse_bwd_workspace_bytes(int BH, int L, int D, int BLKQ, int BLKK, int topk) {
+  (void)D;
+  (void)topk;
+  return (int64_t)bwd_ws(BH, L, BLKQ, BLKK).total;
+}
+
+template <typename Tag, int D, int BLKQ>
+static int bwd_impl(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
+                    const int8_t* sparse_map, const void* lut, int lut64, void* dq, void* dk, void* dv, int BH, int L,
+                    int topk, float qk_scale, char* ws, hipStream_t st) {
+  const BwdWs w = bwd_ws(BH, L, BLKQ, 64);
+  const int Mblk = cdiv(L, BLKQ), Nblk = cdiv(L, 64);
+  float* delta = (float*)(ws + w.delta);
+  int* count = (int*)(ws + w.count);
+  int* list = (int*)(ws + w.list);
+  const size_t rows = (size_t)BH * L;
+  constexpr int RPB = 256 / (D / 8);
+  hipLaunchKernelGGL((bwd_delta_kernel<Tag, D>), dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, st,
+                     (const uint16_t*)o, (const uint16_t*)d_o, delta, rows);
+  hipLaunchKernelGGL(bwd_col_lists_kernel, dim3(cdiv(Nblk, 64), BH), dim3(64), 0, st, sparse_map, list, count, Mblk, Nblk);
+  const int total_q = BH * Mblk;
+  hipLaunchKernelGGL((bwd_dq_kernel<Tag, D, BLKQ>), dim3(xcd_grid(total_q)), dim3(BLKQ * 2), 0, st, (const uint16_t*)q,
+                     (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse, delta, lut, lut64, (uint16_t*)dq, L,
+                     Mblk, topk, qk_scale, total_q);
+  const int total_k = BH * Nblk;
+  hipLaunchKernelGGL((bwd_dkdv_kernel<Tag, D, BLKQ>), dim3(xcd_grid(total_k)), dim3(128), 0, st, (const uint16_t*)q,
+                     (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse, delta, list, count, (uint16_t*)dk,
+                     (uint16_t*)dv, L, Mblk, Nblk, qk_scale, total_k);
+  return check_launch("sparse_attn_bwd");
+}
+
+}  // namespace sla
+
+using namespace sla;
+
+extern "C" int sla_sparse_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o,
+                                   const float* lse, const int8_t* sparse_map, const void* lut, int lut_elem_bytes,
+                                   void* dq, void* dk, void* dv, int dtype, int B, int H, int L, int D, int BLKQ, int BLKK,
+                                   int topk, float qk_scale, void* workspace, int64_t workspace_bytes, void* stream) {
+  int rc = validate_attn_shape(dtype, B, H, L, D, BLKQ, BLKK, topk, lut_elem_bytes);
+  if (rc) return rc;
+  SLA_REQUIRE(q && k && v && o && d_o && lse && sparse_map && dq && dk && dv && workspace && (lut || topk == 0),
+              SLA_ERR_BAD_ARG, "null pointer");
+  SLA_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)o | (uintptr_t)d_o | (uintptr_t)dq | (uintptr_t)dk |
+               (uintptr_t)dv | (uintptr_t)workspace) % 16 == 0,
+              SLA_ERR_BAD_ARG, "tensors must be 16-byte aligned");
+  SLA_REQUIRE((int64_t)B * H <= 65535, SLA_ERR_UNSUPPORTED, "B*H exceeds 65535");
+  const int BH = B * H;
+  const int64_t need = sparse_bwd_workspace_bytes(BH, L, D, BLKQ, BLKK, topk);
+  SLA_REQUIRE(workspace_bytes >= need, SLA_ERR_WORKSPACE, "workspace of %lld bytes, need %lld", (long long)workspace_bytes,
+              (long long)need);
+  SLA_REQUIRE((int64_t)BH * cdiv(L, 64) * cdiv(L, BLKQ) < (1ll << 40), SLA_ERR_UNSUPPORTED, "block map too large");
+  hipStream_t st = (hipStream_t)stream;
+  char* ws = (char*)workspace;
+  const int lut64 = lut_elem_bytes == 8;
+#define SLA_BWD_CASE(TAG, DD, BQ) \
+  if (D == DD && BLKQ == BQ)      \
+  return bwd_impl<TAG, DD, BQ>(q, k, v, o, d_o, lse, sparse_map, lut, lut64, dq, dk, dv, BH, L, topk, qk_scale, ws, st)
+  if (dtype == SLA_BF16) {
+    SLA_BWD_CASE(bf16_tag, 128, 64);
+    SLA_BWD_CASE(bf16_tag, 128, 128);
+    SLA_BWD_CASE(bf16_tag, 64, 64);
+    SLA_BWD_CASE(bf16_tag, 64, 128);
+  } else {
+    SLA_BWD_CASE(f16_tag, 128, 64);
+    SLA_BWD_CASE(f16_tag, 128, 128);
+    SLA_BWD_CASE(f16_tag, 64, 64);
+    SLA_BWD_CASE(f16_tag, 64, 128);
+  }
+#undef SLA_BWD_CASE
+  set_error("unsupported D=%d BLKQ=%d", D, BLKQ);
+  return SLA_ERR_UNSUPPORTED;
+}

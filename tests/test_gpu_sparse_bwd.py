@@ -1,0 +1,81 @@
+"""HIP block-sparse attention backward vs the CPU oracle (tolerance 2e-2 abs, cos >= 0.999)."""
+import pytest
+import torch
+
+from conftest import cos_sim, max_abs
+from oracle import sla_oracle as O
+from sla_amd import _attention
+from sla_amd.inputs import CONFIGS, make_inputs
+
+pytestmark = pytest.mark.gpu
+
+TOL_ABS = 2e-2
+TOL_COS = 0.999
+
+
+def _grads(q, k, v, do, m, lut, T, BLKQ, dev):
+    qd, kd, vd = (t.to(dev).requires_grad_(True) for t in (q, k, v))
+    o = _attention.apply(qd, kd, vd, m.to(dev), lut.to(dev), T, BLKQ, 64)
+    o.backward(do.to(dev))
+    torch.cuda.synchronize()
+    return o.detach().cpu(), qd.grad.cpu(), kd.grad.cpu(), vd.grad.cpu()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("L,D,BLKQ,ratio", [(512, 128, 64, 0.25), (1000, 128, 64, 0.3), (777, 128, 128, 0.4),
+                                            (640, 64, 64, 0.5), (333, 64, 128, 0.34), (50, 128, 64, 1.0)])
+def test_against_dense_oracle(dev, dtype, L, D, BLKQ, ratio):
+    g = torch.Generator().manual_seed(L + D)
+    q, k, v, do = (torch.randn(1, 3, L, D, generator=g).to(dtype) for _ in range(4))
+    m, lut, T = O.get_block_map(q, k, ratio, BLKQ, 64)
+    o_ref, lse_ref = O.sparse_attn_fwd_dense(q, k, v, m, BLKQ, 64)
+    refs = O.sparse_attn_bwd_dense(q, k, v, o_ref, do, lse_ref, m, BLKQ, 64)
+    o, dq, dk, dv = _grads(q, k, v, do, m, lut, T, BLKQ, dev)
+    for name, a, b in zip(("dq", "dk", "dv"), (dq, dk, dv), refs):
+        assert a.dtype == dtype
+        assert max_abs(a, b) <= TOL_ABS, name
+        assert cos_sim(a, b) >= TOL_COS, name
+
+
+def test_full_selection_equals_sdpa_autograd(dev):
+    g = torch.Generator().manual_seed(21)
+    q, k, v, do = (torch.randn(2, 2, 300, 128, generator=g).to(torch.bfloat16) for _ in range(4))
+    N = 5
+    lut = torch.arange(N).expand(2, 2, N, N).contiguous()
+    m = torch.ones(2, 2, N, N, dtype=torch.int8)
+    qr, kr, vr = (t.double().requires_grad_(True) for t in (q, k, v))
+    torch.nn.functional.scaled_dot_product_attention(qr, kr, vr).backward(do.double())
+    o, dq, dk, dv = _grads(q, k, v, do, m, lut, N, 64, dev)
+    for a, b in ((dq, qr.grad), (dk, kr.grad), (dv, vr.grad)):
+        assert max_abs(a, b) <= TOL_ABS and cos_sim(a, b) >= TOL_COS
+
+
+def test_cfg2_backward(dev):
+    cfg = CONFIGS["cfg2"]
+    d = make_inputs(cfg)
+    m, lut, T = O.get_block_map(d["q"], d["k"], cfg.topk, 64, 64)
+    o_ref, lse_ref = O.sparse_attn_fwd_gather(d["q"], d["k"], d["v"], lut, 64, 64)
+    refs = O.sparse_attn_bwd_gather(d["q"], d["k"], d["v"], o_ref, d["do"], lse_ref, lut, 64, 64)
+    o, dq, dk, dv = _grads(d["q"], d["k"], d["v"], d["do"], m, lut, T, 64, dev)
+    for name, a, b in zip(("dq", "dk", "dv"), (dq, dk, dv), refs):
+        assert max_abs(a, b) <= TOL_ABS, name
+        assert cos_sim(a, b) >= TOL_COS, name
+
+
+def test_cfg3_shape_invariants_and_two_heads(dev):
+    # long sequence with a partial last block: oracle on two heads + size-independent identities
+    cfg = CONFIGS["cfg3"]
+    d = make_inputs(cfg, H=2, with_do=True)
+    m, lut, T = O.get_block_map(d["q"], d["k"], cfg.topk, 64, 64)
+    o_ref, lse_ref = O.sparse_attn_fwd_gather(d["q"], d["k"], d["v"], lut, 64, 64)
+    refs = O.sparse_attn_bwd_gather(d["q"], d["k"], d["v"], o_ref, d["do"], lse_ref, lut, 64, 64)
+    o, dq, dk, dv = _grads(d["q"], d["k"], d["v"], d["do"], m, lut, T, 64, dev)
+    for name, a, b in zip(("dq", "dk", "dv"), (dq, dk, dv), refs):
+        assert max_abs(a, b) <= TOL_ABS, name
+        assert cos_sim(a, b) >= TOL_COS, name
+    # rows of P sum to one: sum_keys dV == sum_queries dO
+    assert max_abs(dv.double().sum(-2), d["do"].double().sum(-2)) <= 0.5
+    # q.k is invariant under (q*a, k/a): sum q.dq == sum k.dk
+    # (signed sums of bf16-rounded terms: the tolerance scales with the sum of magnitudes)
+    ta, tb = d["q"].double() * dq.double(), d["k"].double() * dk.double()
+    assert abs(ta.sum() - tb.sum()) <= 1e-3 * float(ta.abs().sum() + tb.abs().sum())
