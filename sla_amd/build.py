@@ -16,7 +16,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIBPATH = os.path.join(LIBDIR, "libsla_hip.so")
 
-SOURCES = ["capi.hip", "block_map.hip", "sparse_fwd.hip", "linear_fwd.hip", "sparse_bwd.hip", "stubs.hip"]
+SOURCES = ["capi.hip", "block_map.hip", "sparse_fwd.hip", "linear.hip", "linear_bwd.hip", "sparse_bwd.hip", "stubs.hip"]
 
 COMMON_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
@@ -38,7 +38,8 @@ def _hipcc() -> str:
 def _compile(src: str, force: bool) -> str:
     obj = os.path.join(LIBDIR, src.replace(".hip", ".o"))
     srcp = os.path.join(CSRC, src)
-    deps = [srcp, os.path.join(CSRC, "common.h"), os.path.join(HERE, "..", "include", "sla_hip.h"), __file__]
+    headers = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h")]
+    deps = [srcp, *headers, os.path.join(HERE, "..", "include", "sla_hip.h"), __file__]
     if not force and os.path.exists(obj) and all(os.path.getmtime(obj) >= os.path.getmtime(d) for d in deps):
         return obj
     flags = list(COMMON_FLAGS)

@@ -1,0 +1,197 @@
+// phi(K)^T V and sum phi(K) state kernels of the linear branch (used by forward and backward).
+#pragma once
+#include "linear_common.h"
+
+namespace sla {
+
+// ---- kernel 1: partial states -----------------------------------------------------------
+// grid (nsplit, BH), 256 threads.  Thread t moves 16-byte chunk (t%CPR) of rows t/CPR + i*RPP.
+template <typename Tag, int D>
+__global__ __launch_bounds__(256) void linear_state_partial_kernel(const uint16_t* __restrict__ k,
+                                                                   const uint16_t* __restrict__ v, float* __restrict__ kv_part,
+                                                                   float* __restrict__ z_part, int L, int rows_per_split,
+                                                                   int fmap) {
+  using E = Elem<Tag>;
+  constexpr int TR = 64;                 // rows per LDS tile
+  constexpr int STR = D + 16;            // LDS row stride: transposed reads of 4 rows hit disjoint banks
+  constexpr int CPR = D / 8;             // 16-byte chunks per row
+  constexpr int RPP = 256 / CPR;         // rows covered by one pass of the 256 threads
+  constexpr int NP = TR / RPP;           // passes per tile
+  constexpr int DT = D / 32;             // 32-wide tiles along either state dimension
+  constexpr int WPT = (DT * DT) / 4;     // output tiles per wave (4 waves)
+  static_assert(DT * DT % 4 == 0, "state tiles must divide among 4 waves");
+
+  __shared__ __attribute__((aligned(16))) uint16_t sK[TR * STR];
+  __shared__ __attribute__((aligned(16))) uint16_t sV[TR * STR];
+  __shared__ float sZ[RPP][D];
+
+  const int split = blockIdx.x, bh = blockIdx.y, nsplit = gridDim.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int g = lane >> 5;
+  const int row_begin = split * rows_per_split;
+  const int row_end = min(L, row_begin + rows_per_split);
+  const uint16_t* kh = k + (size_t)bh * L * D;
+  const uint16_t* vh = v + (size_t)bh * L * D;
+
+  const int lrow = tid / CPR, lcol = (tid % CPR) * 8;
+
+  // wave w owns output tiles w*WPT .. w*WPT+WPT-1; tile id = d1tile*DT + d2tile
+  f32x16_t acc[WPT];
+#pragma unroll
+  for (int t = 0; t < WPT; ++t)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[t][i] = 0.f;
+  float zacc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) zacc[e] = 0.f;
+
+  const int tr_row = (lane & 15) >> 2;
+  const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+
+  for (int r0 = row_begin; r0 < row_end; r0 += TR) {
+    __syncthreads();
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
+      const int row = lrow + p * RPP;
+      const int grow = r0 + row;
+      i16x8_t kk = {0, 0, 0, 0, 0, 0, 0, 0}, vv = {0, 0, 0, 0, 0, 0, 0, 0};
+      const bool ok = grow < row_end;
+      if (ok) {
+        kk = *reinterpret_cast<const i16x8_t*>(kh + (size_t)grow * D + lcol);
+        vv = *reinterpret_cast<const i16x8_t*>(vh + (size_t)grow * D + lcol);
+      }
+      float f[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) f[e] = E::to_float((uint16_t)kk[e]);
+      if (fmap == SLA_FMAP_SOFTMAX) {
+        // the CPR lanes that share this row are adjacent: reduce max and sum across them
+        float mx = f[0];
+#pragma unroll
+        for (int e = 1; e < 8; ++e) mx = fmaxf(mx, f[e]);
+#pragma unroll
+        for (int s = 1; s < CPR; s <<= 1) mx = fmaxf(mx, __shfl_xor(mx, s));
+        float sum = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          f[e] = __expf(f[e] - mx);
+          sum += f[e];
+        }
+#pragma unroll
+        for (int s = 1; s < CPR; s <<= 1) sum += __shfl_xor(sum, s);
+        const float inv = 1.0f / sum;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) f[e] = round16<Tag>(f[e] * inv);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) f[e] = fmap_pointwise<Tag>(fmap, f[e]);
+      }
+      i16x8_t fk;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        if (!ok) f[e] = 0.f;              // rows past the end take no part (phi(0) is not 0 for elu/softmax)
+        zacc[e] += f[e];
+        fk[e] = (short)E::from_float(f[e]);
+      }
+      *reinterpret_cast<i16x8_t*>(&sK[row * STR + lcol]) = fk;
+      *reinterpret_cast<i16x8_t*>(&sV[row * STR + lcol]) = vv;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int c = 0; c < TR / 16; ++c) {
+      const int l0 = 16 * c + 8 * g + tr_row;
+#pragma unroll
+      for (int t = 0; t < WPT; ++t) {
+        const int tile = wave * WPT + t;
+        const int d1t = tile / DT, d2t = tile % DT;
+        const uint16_t* pa = &sK[l0 * STR + 32 * d1t + tr_col];
+        const uint16_t* pb = &sV[l0 * STR + 32 * d2t + tr_col];
+        const i16x8_t a = concat4(lds_read_tr16(pa), lds_read_tr16(pa + 4 * STR));
+        const i16x8_t b = concat4(lds_read_tr16(pb), lds_read_tr16(pb + 4 * STR));
+        acc[t] = E::mfma32(a, b, acc[t]);
+      }
+    }
+  }
+
+  // partial KV, stored transposed: kv_part[bh][split][d2][d1]
+  float* out = kv_part + ((size_t)bh * nsplit + split) * D * D;
+#pragma unroll
+  for (int t = 0; t < WPT; ++t) {
+    const int tile = wave * WPT + t;
+    const int d1t = tile / DT, d2t = tile % DT;
+    const int d2 = 32 * d2t + (lane & 31);
+#pragma unroll
+    for (int i4 = 0; i4 < 4; ++i4) {
+      f32x4_t w = {acc[t][4 * i4], acc[t][4 * i4 + 1], acc[t][4 * i4 + 2], acc[t][4 * i4 + 3]};
+      *reinterpret_cast<f32x4_t*>(out + (size_t)d2 * D + 32 * d1t + 8 * i4 + 4 * g) = w;
+    }
+  }
+  // partial z: reduce the RPP row groups through LDS
+  __syncthreads();
+#pragma unroll
+  for (int e = 0; e < 8; ++e) sZ[lrow][lcol + e] = zacc[e];
+  __syncthreads();
+  if (tid < D) {
+    float s = 0.f;
+#pragma unroll
+    for (int r = 0; r < RPP; ++r) s += sZ[r][tid];
+    z_part[((size_t)bh * nsplit + split) * D + tid] = s;
+  }
+}
+
+// ---- kernel 2: reduce partials, round to 16 bit -------------------------------------------
+template <typename Tag>
+__global__ void linear_state_reduce_kernel(const float* __restrict__ kv_part, const float* __restrict__ z_part,
+                                           uint16_t* __restrict__ kvt, uint16_t* __restrict__ z, int nsplit, int DD, int D) {
+  using E = Elem<Tag>;
+  const int bh = blockIdx.y;
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < DD) {
+    const float* p = kv_part + (size_t)bh * nsplit * DD + i;
+    float s = 0.f;
+    for (int sp = 0; sp < nsplit; ++sp) s += p[(size_t)sp * DD];
+    kvt[(size_t)bh * DD + i] = E::from_float(s);
+  }
+  if (i < D) {
+    const float* p = z_part + (size_t)bh * nsplit * D + i;
+    float s = 0.f;
+    for (int sp = 0; sp < nsplit; ++sp) s += p[(size_t)sp * D];
+    z[(size_t)bh * D + i] = E::from_float(s);
+  }
+}
+
+// ---- workspace layout of the state build -----------------------------------------------------
+struct LinWs {
+  int nsplit, rows_per_split;
+  size_t kv_part, z_part, kvt, z, total;
+};
+
+static inline LinWs lin_ws(int BH, int L, int D) {
+  LinWs w;
+  const LinSplit sp = lin_split(BH, L);
+  w.nsplit = sp.nsplit;
+  w.rows_per_split = sp.rows_per_split;
+  size_t off = 0;
+  w.kv_part = off; off += align_up((int64_t)BH * w.nsplit * D * D * 4, 256);
+  w.z_part = off;  off += align_up((int64_t)BH * w.nsplit * D * 4, 256);
+  w.kvt = off;     off += align_up((int64_t)BH * D * D * 2, 256);
+  w.z = off;       off += align_up((int64_t)BH * D * 2, 256);
+  w.total = off;
+  return w;
+}
+
+
+// Streams K and V once and leaves KVT (16 bit, [d2][d1]) and z (16 bit) in the workspace.
+template <typename Tag, int D>
+static inline void launch_state_build(const void* k, const void* v, int fmap, int BH, int L, char* ws, const LinWs& w,
+                                      hipStream_t st) {
+  float* kv_part = (float*)(ws + w.kv_part);
+  float* z_part = (float*)(ws + w.z_part);
+  uint16_t* kvt = (uint16_t*)(ws + w.kvt);
+  uint16_t* z = (uint16_t*)(ws + w.z);
+  hipLaunchKernelGGL((linear_state_partial_kernel<Tag, D>), dim3(w.nsplit, BH), dim3(256), 0, st, (const uint16_t*)k,
+                     (const uint16_t*)v, kv_part, z_part, L, w.rows_per_split, fmap);
+  hipLaunchKernelGGL((linear_state_reduce_kernel<Tag>), dim3(cdiv(D * D, 256), BH), dim3(256), 0, st, kv_part, z_part, kvt, z,
+                     w.nsplit, D * D, D);
+}
+
+}  // namespace sla

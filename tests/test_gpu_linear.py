@@ -51,3 +51,33 @@ def test_cfg3_shape_two_heads(dev):
     ref = O.linear_branch(d["q"], d["k"], d["v"], w, b, cfg.feature_map, torch.float32)
     out = linear_fwd(d["q"].to(dev), d["k"].to(dev), d["v"].to(dev), w.to(dev), b.to(dev), None, cfg.feature_map).cpu()
     assert max_abs(out, ref) <= TOL_ABS and cos_sim(out, ref) >= TOL_COS
+
+
+def _oracle_linear_grads(q, k, v, w, b, g, fmap):
+    qd, kd, vd = (t.double().requires_grad_(True) for t in (q, k, v))
+    wd, bd = w.double().requires_grad_(True), b.double().requires_grad_(True)
+    out = O.linear_branch(qd, kd, vd, wd, bd, fmap, torch.float64)
+    out.backward(g.double())
+    return qd.grad, kd.grad, vd.grad, wd.grad, bd.grad
+
+
+@pytest.mark.parametrize("fmap", ["elu", "relu", "softmax"])
+@pytest.mark.parametrize("L,D", [(512, 128), (1000, 128), (333, 64)])
+def test_linear_branch_backward_vs_autograd_oracle(dev, fmap, L, D):
+    from sla_amd.linear import _linear_proj_add
+    gen = torch.Generator().manual_seed(L + 7)
+    q, k, v, res, g = (torch.randn(2, 2, L, D, generator=gen).to(torch.bfloat16) for _ in range(5))
+    w, b = make_proj(D)
+    refs = _oracle_linear_grads(q, k, v, w, b, g, fmap)
+    qd, kd, vd, rd = (t.to(dev).requires_grad_(True) for t in (q, k, v, res))
+    wd, bd = w.to(dev).requires_grad_(True), b.to(dev).requires_grad_(True)
+    out = _linear_proj_add.apply(qd, kd, vd, wd, bd, rd, fmap)
+    out.backward(g.to(dev))
+    torch.cuda.synchronize()
+    assert torch.equal(rd.grad.cpu(), g)
+    names = ("dq", "dk", "dv", "dW", "db")
+    for name, a, r in zip(names, (qd.grad, kd.grad, vd.grad, wd.grad, bd.grad), refs):
+        a = a.cpu()
+        scale = max(1.0, float(r.abs().max()))          # dW/db are sums over B*H*L rows
+        assert max_abs(a, r) <= TOL_ABS * scale, (name, max_abs(a, r), scale)
+        assert cos_sim(a, r) >= TOL_COS, (name, cos_sim(a, r))

@@ -1,0 +1,52 @@
+"""Whole-module forward+backward (cfg2, README shape) vs autograd of the fp64 dense oracle."""
+import pytest
+import torch
+
+from conftest import cos_sim, max_abs
+from oracle import sla_oracle as O
+from sla_amd import SparseLinearAttention
+from sla_amd.inputs import CONFIGS, make_inputs, make_proj
+
+pytestmark = pytest.mark.gpu
+
+TOL_ABS = 2e-2
+TOL_COS = 0.999
+
+
+@pytest.mark.parametrize("fmap", ["softmax", "elu", "relu"])
+def test_cfg2_gradients(dev, fmap):
+    cfg = CONFIGS["cfg2"]
+    d = make_inputs(cfg)
+    w, b = make_proj(cfg.D)
+    mod = SparseLinearAttention(cfg.D, cfg.topk, fmap, cfg.BLKQ, cfg.BLKK).to(dev)
+    with torch.no_grad():
+        mod.proj_l.weight.copy_(w)
+        mod.proj_l.bias.copy_(b)
+    qd, kd, vd = (d[x].to(dev).requires_grad_(True) for x in "qkv")
+    o = mod(qd, kd, vd)
+    o.backward(d["do"].to(dev))
+    torch.cuda.synchronize()
+
+    m, lut, T = O.get_block_map(d["q"], d["k"], cfg.topk, cfg.BLKQ, cfg.BLKK)
+    grads = {}
+    # the dense oracle needs L^2 scores per head: one (b,h) at a time
+    dw_ref = torch.zeros(cfg.D, cfg.D, dtype=torch.float64)
+    db_ref = torch.zeros(cfg.D, dtype=torch.float64)
+    for bi in range(cfg.B):
+        for hi in range(cfg.H):
+            sl = (slice(bi, bi + 1), slice(hi, hi + 1))
+            qr, kr, vr = (d[x][sl].double().requires_grad_(True) for x in "qkv")
+            wr, br = w.double().requires_grad_(True), b.double().requires_grad_(True)
+            out, _, _ = O.sla_forward_autograd(qr, kr, vr, wr, br, m[sl], fmap, cfg.BLKQ, cfg.BLKK)
+            out.backward(d["do"][sl].double())
+            dw_ref += wr.grad
+            db_ref += br.grad
+            for name, a, r in (("dq", qd.grad[sl], qr.grad), ("dk", kd.grad[sl], kr.grad), ("dv", vd.grad[sl], vr.grad)):
+                assert max_abs(a.cpu(), r) <= TOL_ABS, (name, bi, hi, max_abs(a.cpu(), r))
+                assert cos_sim(a.cpu(), r) >= TOL_COS, (name, bi, hi)
+            if bi == 0 and hi == 0:
+                assert max_abs(o[sl].detach().cpu(), out.detach()) <= TOL_ABS
+    for name, a, r in (("dW", mod.proj_l.weight.grad, dw_ref), ("db", mod.proj_l.bias.grad, db_ref)):
+        scale = max(1.0, float(r.abs().max()))
+        assert max_abs(a.cpu(), r) <= TOL_ABS * scale, (name, max_abs(a.cpu(), r), scale)
+        assert cos_sim(a.cpu(), r) >= TOL_COS, name
