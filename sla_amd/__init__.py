@@ -2,3 +2,4 @@
 from .block_map import get_block_map, mean_pool  # noqa: F401
 from .sparse_attn import _attention  # noqa: F401
 from .module import SparseLinearAttention  # noqa: F401
+from .sage import SageSparseLinearAttention  # noqa: F401

@@ -290,6 +290,23 @@ static int block_map_impl(const void* q, const void* k, int dtype, int BH, int L
   return check_launch("block map");
 }
 
+// Column mean of k over L in the fixed order (chunk sums, then chunks), rounded to `dtype`.
+// chunk_sums: fp32 (BH, ceil(L/64), D) scratch; colmean: (BH, D) in `dtype`.
+void launch_k_colmean(const void* k, int dtype, int BH, int L, int D, float* chunk_sums, void* colmean, hipStream_t st) {
+  const int nchunk = cdiv(L, KMEAN_CHUNK);
+  const dim3 grid(cdiv(D, 128), BH);
+  if (dtype == SLA_F32) {
+    launch_pool<IoF32, 0>(k, nullptr, chunk_sums, BH, L, D, KMEAN_CHUNK, st);
+    hipLaunchKernelGGL((colmean_kernel<IoF32>), grid, dim3(128), 0, st, chunk_sums, (float*)colmean, nchunk, D, L);
+  } else if (dtype == SLA_BF16) {
+    launch_pool<IoBf16, 0>(k, nullptr, chunk_sums, BH, L, D, KMEAN_CHUNK, st);
+    hipLaunchKernelGGL((colmean_kernel<IoBf16>), grid, dim3(128), 0, st, chunk_sums, (uint16_t*)colmean, nchunk, D, L);
+  } else {
+    launch_pool<IoF16, 0>(k, nullptr, chunk_sums, BH, L, D, KMEAN_CHUNK, st);
+    hipLaunchKernelGGL((colmean_kernel<IoF16>), grid, dim3(128), 0, st, chunk_sums, (uint16_t*)colmean, nchunk, D, L);
+  }
+}
+
 }  // namespace sla
 
 using namespace sla;

@@ -1,0 +1,444 @@
+// SageSLA quantised forward for gfx950: INT8 QK^T and FP8 (e4m3) PV on the matrix cores.
+//
+// Stands in for the third-party calls of SageSLA/core.py:102-144 of the reference
+// (spas_sage_attn get_vanilla_qk_quant, block_map_lut_triton, transpose_pad_permute_cuda,
+// scale_fuse_quant_cuda, qk_int8_sv_f8_*): that extension is not part of the reference tree,
+// so the scheme below follows its published description, not its code:
+//   q_int8 = rint(q / sq), sq = max|q| / 127 over each block of BLKQ rows;
+//   k_int8 = rint((k - mean_L k) / sk), sk per block of BLKK rows;
+//   v_fp8  = e4m3(v / sv), sv[d] = max_L |v[:, d]| / 448;
+//   S = (q_int8 . k_int8) * sq * sk * scale ; P = softmax over the selected blocks ;
+//   O = (e4m3(448 P) . v_fp8) * sv / (448 l).
+// The look-up table of the bf16 path is used as is (no delta encoding is needed here).
+#include "common.h"
+
+namespace sla {
+
+void launch_k_colmean(const void* k, int dtype, int BH, int L, int D, float* chunk_sums, void* colmean, hipStream_t st);
+
+// ---- INT8 block quantisation ----------------------------------------------------------------
+// One workgroup per (block, bh).  SUB_MEAN: subtract the per-head column mean first.
+template <typename Tag, int D, int BLK, bool SUB_MEAN>
+__global__ __launch_bounds__(256) void quant_int8_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ colmean,
+                                                         int8_t* __restrict__ xq, float* __restrict__ scale, int L, int nblk) {
+  using E = Elem<Tag>;
+  constexpr int CPR = D / 8;
+  constexpr int RPP = 256 / CPR;
+  constexpr int NP = BLK / RPP;
+  __shared__ float sred[4];
+  const int blk = blockIdx.x, bh = blockIdx.y;
+  const int tid = threadIdx.x;
+  const int lrow = tid / CPR, lcol = (tid % CPR) * 8;
+  float cm[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) cm[e] = 0.f;
+  if (SUB_MEAN) {
+    const i16x8_t m = *reinterpret_cast<const i16x8_t*>(colmean + (size_t)bh * D + lcol);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) cm[e] = E::to_float((uint16_t)m[e]);
+  }
+  float val[NP][8];
+  float amax = 0.f;
+#pragma unroll
+  for (int p = 0; p < NP; ++p) {
+    const int grow = blk * BLK + lrow + p * RPP;
+    i16x8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
+    const bool ok = grow < L;
+    if (ok) v = *reinterpret_cast<const i16x8_t*>(x + ((size_t)bh * L + grow) * D + lcol);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      val[p][e] = ok ? E::to_float((uint16_t)v[e]) - cm[e] : 0.f;
+      amax = fmaxf(amax, fabsf(val[p][e]));
+    }
+  }
+#pragma unroll
+  for (int s = 1; s < 64; s <<= 1) amax = fmaxf(amax, __shfl_xor(amax, s));
+  if ((tid & 63) == 0) sred[tid >> 6] = amax;
+  __syncthreads();
+  amax = fmaxf(fmaxf(sred[0], sred[1]), fmaxf(sred[2], sred[3]));
+  const float sc = fmaxf(amax, 1e-30f) / 127.0f;
+  if (tid == 0) scale[(size_t)bh * nblk + blk] = sc;
+#pragma unroll
+  for (int p = 0; p < NP; ++p) {
+    const int grow = blk * BLK + lrow + p * RPP;
+    if (grow >= L) continue;
+    i32x2_t w;
+    int8_t* b = reinterpret_cast<int8_t*>(&w);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      float r = rintf(val[p][e] / sc);
+      r = fminf(fmaxf(r, -127.f), 127.f);
+      b[e] = (int8_t)(int)r;
+    }
+    *reinterpret_cast<i32x2_t*>(xq + ((size_t)bh * L + grow) * D + lcol) = w;
+  }
+}
+
+// ---- FP8 per-channel quantisation of V ------------------------------------------------------
+// pass 1: per (chunk of 256 rows, bh) column abs-max -> partial; pass 2: reduce partials;
+// pass 3: v_fp8 = e4m3(v / scale).
+template <typename Tag, int D>
+__global__ __launch_bounds__(256) void v_amax_partial_kernel(const uint16_t* __restrict__ v, float* __restrict__ part, int L,
+                                                             int rows_per_chunk) {
+  using E = Elem<Tag>;
+  constexpr int CPR = D / 8;
+  constexpr int RPP = 256 / CPR;
+  __shared__ float sm[RPP][D];
+  const int chunk = blockIdx.x, bh = blockIdx.y, nchunk = gridDim.x;
+  const int tid = threadIdx.x;
+  const int lrow = tid / CPR, lcol = (tid % CPR) * 8;
+  const int r_end = min(L, (chunk + 1) * rows_per_chunk);
+  float am[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) am[e] = 0.f;
+  for (int row = chunk * rows_per_chunk + lrow; row < r_end; row += RPP) {
+    const i16x8_t x = *reinterpret_cast<const i16x8_t*>(v + ((size_t)bh * L + row) * D + lcol);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) am[e] = fmaxf(am[e], fabsf(E::to_float((uint16_t)x[e])));
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) sm[lrow][lcol + e] = am[e];
+  __syncthreads();
+  if (tid < D) {
+    float a = 0.f;
+#pragma unroll
+    for (int r = 0; r < RPP; ++r) a = fmaxf(a, sm[r][tid]);
+    part[((size_t)bh * nchunk + chunk) * D + tid] = a;
+  }
+}
+
+__global__ void v_scale_kernel(const float* __restrict__ part, float* __restrict__ v_scale, int nchunk, int D) {
+  const int bh = blockIdx.x, d = threadIdx.x;
+  if (d >= D) return;
+  float a = 0.f;
+  for (int c = 0; c < nchunk; ++c) a = fmaxf(a, part[((size_t)bh * nchunk + c) * D + d]);
+  v_scale[(size_t)bh * D + d] = fmaxf(a, 1e-30f) / 448.0f;
+}
+
+static __device__ __forceinline__ uint32_t cvt4_fp8(float a, float b, float c, float d) {
+  int w = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
+  w = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, w, true);
+  return (uint32_t)w;
+}
+
+template <typename Tag, int D>
+__global__ __launch_bounds__(256) void v_quant_fp8_kernel(const uint16_t* __restrict__ v, const float* __restrict__ v_scale,
+                                                          uint8_t* __restrict__ v8, int L) {
+  using E = Elem<Tag>;
+  constexpr int CPR = D / 8;
+  constexpr int RPP = 256 / CPR;
+  const int bh = blockIdx.y;
+  const int row = blockIdx.x * RPP + threadIdx.x / CPR;
+  const int lcol = (threadIdx.x % CPR) * 8;
+  if (row >= L) return;
+  const i16x8_t x = *reinterpret_cast<const i16x8_t*>(v + ((size_t)bh * L + row) * D + lcol);
+  float f[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) f[e] = E::to_float((uint16_t)x[e]) / v_scale[(size_t)bh * D + lcol + e];
+  i32x2_t w;
+  w[0] = (int)cvt4_fp8(f[0], f[1], f[2], f[3]);
+  w[1] = (int)cvt4_fp8(f[4], f[5], f[6], f[7]);
+  *reinterpret_cast<i32x2_t*>(v8 + ((size_t)bh * L + row) * D + lcol) = w;
+}
+
+// ---- quantised block-sparse attention ----------------------------------------------------------
+typedef __attribute__((address_space(3))) i32x2_t lds_i32x2_t;
+
+template <typename OutTag, int D, int BLKQ>
+__global__ __launch_bounds__(BLKQ * 2) void sage_fwd_kernel(const int8_t* __restrict__ q8, const float* __restrict__ q_scale,
+                                                            const int8_t* __restrict__ k8, const float* __restrict__ k_scale,
+                                                            const uint8_t* __restrict__ v8, const float* __restrict__ v_scale,
+                                                            const void* __restrict__ lut, int lut64, uint16_t* __restrict__ o,
+                                                            int L, int Mblk, int Nblk, int topk, float scale_log2e, int total) {
+  using EO = Elem<OutTag>;
+  constexpr int BLKK = 64;
+  constexpr int NT = BLKQ * 2;
+  constexpr int QC = D / 32;                // 32-wide int8 contraction chunks
+  constexpr int DT = D / 32;                // 32-row tiles of O^T
+  constexpr int STR = D + 16;               // bytes per LDS row
+  constexpr int CPR = D / 16;               // 16-byte chunks per row
+  constexpr int NLD = (BLKK * CPR + NT - 1) / NT;
+
+  __shared__ __attribute__((aligned(16))) uint8_t sK[BLKK * STR];
+  __shared__ __attribute__((aligned(16))) uint8_t sV[BLKK * STR];
+
+  const int logical = xcd_remap(blockIdx.x, gridDim.x, total);
+  if (logical < 0) return;
+  const int bh = logical / Mblk;
+  const int mb = logical - bh * Mblk;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int g = lane >> 5, r = lane & 31;
+
+  const size_t head_off = (size_t)bh * L * D;
+  const int qrow = mb * BLKQ + wave * 32 + r;
+  i32x4_t qf[QC];
+#pragma unroll
+  for (int c = 0; c < QC; ++c) {
+    qf[c] = i32x4_t{0, 0, 0, 0};
+    if (qrow < L) qf[c] = *reinterpret_cast<const i32x4_t*>(q8 + head_off + (size_t)qrow * D + 32 * c + 16 * g);
+  }
+  const float qs = q_scale[(size_t)bh * Mblk + mb] * scale_log2e;
+  const float* ksc = k_scale + (size_t)bh * Nblk;
+
+  const size_t lut_row = ((size_t)bh * Mblk + mb) * topk;
+  auto lut_at = [&](int i) -> int {
+    return lut64 ? (int)reinterpret_cast<const long long*>(lut)[lut_row + i]
+                 : reinterpret_cast<const int*>(lut)[lut_row + i];
+  };
+  i32x4_t kreg[NLD], vreg[NLD];
+  auto load_tile = [&](int nb) {
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) {
+      const int idx = tid + i * NT;
+      const int row = idx / CPR, col = (idx % CPR) * 16;
+      const int grow = nb * BLKK + row;
+      kreg[i] = i32x4_t{0, 0, 0, 0};
+      vreg[i] = i32x4_t{0, 0, 0, 0};
+      if (idx < BLKK * CPR && grow < L) {
+        kreg[i] = *reinterpret_cast<const i32x4_t*>(k8 + head_off + (size_t)grow * D + col);
+        vreg[i] = *reinterpret_cast<const i32x4_t*>(v8 + head_off + (size_t)grow * D + col);
+      }
+    }
+  };
+  auto store_tile = [&]() {
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) {
+      const int idx = tid + i * NT;
+      if (idx < BLKK * CPR) {
+        const int row = idx / CPR, col = (idx % CPR) * 16;
+        *reinterpret_cast<i32x4_t*>(&sK[row * STR + col]) = kreg[i];
+        *reinterpret_cast<i32x4_t*>(&sV[row * STR + col]) = vreg[i];
+      }
+    }
+  };
+
+  f32x16_t oacc[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) oacc[dt][i] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+
+  // transposed 8-bit read: lane i of a 16-lane group passes the address of (row i/2, 8 bytes at
+  // column 8*(i%2)) and receives column i of the 8x16 tile.  Row i/2 is mapped to the key that
+  // accumulator slot i/2 of the probabilities holds: keys 4g+{0..3} and 8+4g+{0..3} of a 16-key chunk.
+  const int li = lane & 15;
+  const int slot = li >> 1;
+  const int tr_key = 8 * (slot >> 2) + 4 * g + (slot & 3);
+  const int tr_col = 16 * ((lane >> 4) & 1) + 8 * (li & 1);
+
+  int nb = topk > 0 ? lut_at(0) : 0;
+  if (topk > 0) load_tile(nb);
+  for (int it = 0; it < topk; ++it) {
+    __syncthreads();
+    store_tile();
+    __syncthreads();
+    const int kv_valid = L - nb * BLKK;
+    const float sc = qs * ksc[nb];
+    if (it + 1 < topk) {
+      nb = lut_at(it + 1);
+      load_tile(nb);
+    }
+    float s[2][16];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      i32x16_t acc;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[i] = 0;
+#pragma unroll
+      for (int c = 0; c < QC; ++c) {
+        const i32x4_t a = *reinterpret_cast<const i32x4_t*>(&sK[(32 * t + r) * STR + 32 * c + 16 * g]);
+        acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, qf[c], acc, 0, 0, 0);
+      }
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int key = 32 * t + 8 * (i >> 2) + 4 * g + (i & 3);
+        s[t][i] = key < kv_valid ? (float)acc[i] * sc : -INFINITY;
+      }
+    }
+    float mx = s[0][0];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[t][i]);
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    const float m_new = fmaxf(m_run, mx);
+    const float alpha = fast_exp2(m_run - m_new);
+    float psum = 0.f;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const float p = fast_exp2(s[t][i] - m_new);
+        psum += p;
+        s[t][i] = p * 448.0f;
+      }
+    l_run = l_run * alpha + psum;
+    m_run = m_new;
+    if (__any(alpha != 1.0f)) {
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) oacc[dt][i] *= alpha;
+    }
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int c2 = 0; c2 < 2; ++c2) {
+        i32x2_t pw;
+        pw[0] = (int)cvt4_fp8(s[t][8 * c2 + 0], s[t][8 * c2 + 1], s[t][8 * c2 + 2], s[t][8 * c2 + 3]);
+        pw[1] = (int)cvt4_fp8(s[t][8 * c2 + 4], s[t][8 * c2 + 5], s[t][8 * c2 + 6], s[t][8 * c2 + 7]);
+        const long pb = __builtin_bit_cast(long, pw);
+        const int key = 32 * t + 16 * c2 + tr_key;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          const i32x2_t a = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_i32x2_t*)&sV[key * STR + 32 * dt + tr_col]);
+          oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(__builtin_bit_cast(long, a), pb, oacc[dt], 0, 0, 0);
+        }
+      }
+  }
+  const float l_tot = l_run + __shfl_xor(l_run, 32);
+  const float inv = 1.0f / (448.0f * l_tot);
+  if (qrow < L) {
+    uint16_t* orow = o + head_off + (size_t)qrow * D;
+    const float* vs = v_scale + (size_t)bh * D;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; ++i4) {
+        const int d0 = 32 * dt + 8 * i4 + 4 * g;
+        const f32x4_t sv = *reinterpret_cast<const f32x4_t*>(vs + d0);
+        i32x2_t w;
+        w[0] = (int)EO::pack2(oacc[dt][4 * i4 + 0] * inv * sv[0], oacc[dt][4 * i4 + 1] * inv * sv[1]);
+        w[1] = (int)EO::pack2(oacc[dt][4 * i4 + 2] * inv * sv[2], oacc[dt][4 * i4 + 3] * inv * sv[3]);
+        *reinterpret_cast<i32x2_t*>(orow + d0) = w;
+      }
+  }
+}
+
+// ---- host -------------------------------------------------------------------------------------
+struct SageWs {
+  int nchunk_v, rows_per_chunk_v;
+  size_t chunk_sums, colmean, v_part, total;
+};
+static SageWs sage_ws(int BH, int L, int D) {
+  SageWs w;
+  w.rows_per_chunk_v = 256;
+  w.nchunk_v = cdiv(L, w.rows_per_chunk_v);
+  size_t off = 0;
+  w.chunk_sums = off; off += align_up((int64_t)BH * cdiv(L, 64) * D * 4, 256);
+  w.colmean = off;    off += align_up((int64_t)BH * D * 2, 256);
+  w.v_part = off;     off += align_up((int64_t)BH * w.nchunk_v * D * 4, 256);
+  w.total = off;
+  return w;
+}
+int64_t sage_quant_workspace_bytes(int BH, int L, int D) { return (int64_t)sage_ws(BH, L, D).total; }
+
+static int validate_sage(int dtype, int B, int H, int L, int D, int BLKQ, int BLKK) {
+  SLA_REQUIRE(B > 0 && H > 0 && L > 0, SLA_ERR_BAD_ARG, "non-positive size (B=%d H=%d L=%d)", B, H, L);
+  SLA_REQUIRE((int64_t)B * H <= 65535, SLA_ERR_UNSUPPORTED, "B*H exceeds 65535");
+  SLA_REQUIRE(dtype == SLA_BF16 || dtype == SLA_F16, SLA_ERR_UNSUPPORTED, "SageSLA takes bf16 or f16, got dtype %d", dtype);
+  SLA_REQUIRE(D == 64 || D == 128, SLA_ERR_UNSUPPORTED, "headdim should be in [64, 128], got %d", D);
+  SLA_REQUIRE(BLKQ == 128 && BLKK == 64, SLA_ERR_UNSUPPORTED, "SageSLA only supports BLKQ=128 and BLKK=64, got %d/%d", BLKQ,
+              BLKK);
+  return SLA_OK;
+}
+
+template <typename Tag, int D>
+static int quant_qk_impl(const void* q, const void* k, int dtype, int BH, int L, int8_t* q8, float* qs, int8_t* k8,
+                         float* ks, char* ws, hipStream_t st) {
+  const SageWs w = sage_ws(BH, L, D);
+  const int M = cdiv(L, 128), N = cdiv(L, 64);
+  launch_k_colmean(k, dtype, BH, L, D, (float*)(ws + w.chunk_sums), ws + w.colmean, st);
+  hipLaunchKernelGGL((quant_int8_kernel<Tag, D, 128, false>), dim3(M, BH), dim3(256), 0, st, (const uint16_t*)q, nullptr, q8,
+                     qs, L, M);
+  hipLaunchKernelGGL((quant_int8_kernel<Tag, D, 64, true>), dim3(N, BH), dim3(256), 0, st, (const uint16_t*)k,
+                     (const uint16_t*)(ws + w.colmean), k8, ks, L, N);
+  return check_launch("sage_quant_qk");
+}
+
+template <typename Tag, int D>
+static int quant_v_impl(const void* v, int BH, int L, uint8_t* v8, float* vs, char* ws, hipStream_t st) {
+  const SageWs w = sage_ws(BH, L, D);
+  float* part = (float*)(ws + w.v_part);
+  hipLaunchKernelGGL((v_amax_partial_kernel<Tag, D>), dim3(w.nchunk_v, BH), dim3(256), 0, st, (const uint16_t*)v, part, L,
+                     w.rows_per_chunk_v);
+  hipLaunchKernelGGL(v_scale_kernel, dim3(BH), dim3(D), 0, st, part, vs, w.nchunk_v, D);
+  constexpr int RPP = 256 / (D / 8);
+  hipLaunchKernelGGL((v_quant_fp8_kernel<Tag, D>), dim3(cdiv(L, RPP), BH), dim3(256), 0, st, (const uint16_t*)v, vs, v8, L);
+  return check_launch("sage_quant_v");
+}
+
+}  // namespace sla
+
+using namespace sla;
+
+extern "C" int sage_quant_qk(const void* q, const void* k, int dtype, int B, int H, int L, int D, int BLKQ, int BLKK,
+                             int8_t* q_int8, float* q_scale, int8_t* k_int8, float* k_scale, void* workspace,
+                             int64_t workspace_bytes, void* stream) {
+  int rc = validate_sage(dtype, B, H, L, D, BLKQ, BLKK);
+  if (rc) return rc;
+  SLA_REQUIRE(q && k && q_int8 && q_scale && k_int8 && k_scale && workspace, SLA_ERR_BAD_ARG, "null pointer");
+  SLA_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)q_int8 | (uintptr_t)k_int8 | (uintptr_t)workspace) % 16 == 0,
+              SLA_ERR_BAD_ARG, "pointers must be 16-byte aligned");
+  const int BH = B * H;
+  SLA_REQUIRE(workspace_bytes >= sage_quant_workspace_bytes(BH, L, D), SLA_ERR_WORKSPACE, "workspace too small");
+  hipStream_t st = (hipStream_t)stream;
+  char* ws = (char*)workspace;
+  if (dtype == SLA_BF16) {
+    if (D == 128) return quant_qk_impl<bf16_tag, 128>(q, k, dtype, BH, L, q_int8, q_scale, k_int8, k_scale, ws, st);
+    return quant_qk_impl<bf16_tag, 64>(q, k, dtype, BH, L, q_int8, q_scale, k_int8, k_scale, ws, st);
+  }
+  if (D == 128) return quant_qk_impl<f16_tag, 128>(q, k, dtype, BH, L, q_int8, q_scale, k_int8, k_scale, ws, st);
+  return quant_qk_impl<f16_tag, 64>(q, k, dtype, BH, L, q_int8, q_scale, k_int8, k_scale, ws, st);
+}
+
+extern "C" int sage_quant_v(const void* v, int dtype, int B, int H, int L, int D, uint8_t* v_fp8, float* v_scale,
+                            void* workspace, int64_t workspace_bytes, void* stream) {
+  int rc = validate_sage(dtype, B, H, L, D, 128, 64);
+  if (rc) return rc;
+  SLA_REQUIRE(v && v_fp8 && v_scale && workspace, SLA_ERR_BAD_ARG, "null pointer");
+  SLA_REQUIRE(((uintptr_t)v | (uintptr_t)v_fp8 | (uintptr_t)workspace) % 16 == 0, SLA_ERR_BAD_ARG,
+              "pointers must be 16-byte aligned");
+  const int BH = B * H;
+  SLA_REQUIRE(workspace_bytes >= sage_quant_workspace_bytes(BH, L, D), SLA_ERR_WORKSPACE, "workspace too small");
+  hipStream_t st = (hipStream_t)stream;
+  char* ws = (char*)workspace;
+  if (dtype == SLA_BF16) {
+    if (D == 128) return quant_v_impl<bf16_tag, 128>(v, BH, L, v_fp8, v_scale, ws, st);
+    return quant_v_impl<bf16_tag, 64>(v, BH, L, v_fp8, v_scale, ws, st);
+  }
+  if (D == 128) return quant_v_impl<f16_tag, 128>(v, BH, L, v_fp8, v_scale, ws, st);
+  return quant_v_impl<f16_tag, 64>(v, BH, L, v_fp8, v_scale, ws, st);
+}
+
+extern "C" int sage_sparse_attn_fwd(const int8_t* q_int8, const float* q_scale, const int8_t* k_int8,
+                                    const float* k_scale, const uint8_t* v_fp8, const float* v_scale, const void* lut,
+                                    int lut_elem_bytes, void* o, int out_dtype, int B, int H, int L, int D, int BLKQ,
+                                    int BLKK, int topk, float qk_scale, void* stream) {
+  int rc = validate_sage(out_dtype, B, H, L, D, BLKQ, BLKK);
+  if (rc) return rc;
+  const int Mblk = cdiv(L, BLKQ), Nblk = cdiv(L, BLKK);
+  SLA_REQUIRE(topk >= 0 && topk <= Nblk, SLA_ERR_BAD_ARG, "topk=%d outside [0, %d]", topk, Nblk);
+  SLA_REQUIRE(lut_elem_bytes == 4 || lut_elem_bytes == 8, SLA_ERR_BAD_ARG, "lut_elem_bytes must be 4 or 8");
+  SLA_REQUIRE(q_int8 && q_scale && k_int8 && k_scale && v_fp8 && v_scale && o && (lut || topk == 0), SLA_ERR_BAD_ARG,
+              "null pointer");
+  SLA_REQUIRE(((uintptr_t)q_int8 | (uintptr_t)k_int8 | (uintptr_t)v_fp8 | (uintptr_t)o | (uintptr_t)v_scale) % 16 == 0,
+              SLA_ERR_BAD_ARG, "pointers must be 16-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+  const int BH = B * H;
+  const int total = BH * Mblk;
+  const float c = qk_scale * 1.4426950408889634f;
+  const int lut64 = lut_elem_bytes == 8;
+#define SAGE_CASE(TAG, DD)                                                                                              \
+  hipLaunchKernelGGL((sage_fwd_kernel<TAG, DD, 128>), dim3(xcd_grid(total)), dim3(256), 0, st, q_int8, q_scale, k_int8, \
+                     k_scale, v_fp8, v_scale, lut, lut64, (uint16_t*)o, L, Mblk, Nblk, topk, c, total);                 \
+  return check_launch("sage_sparse_attn_fwd")
+  if (out_dtype == SLA_BF16) {
+    if (D == 128) { SAGE_CASE(bf16_tag, 128); }
+    SAGE_CASE(bf16_tag, 64);
+  }
+  if (D == 128) { SAGE_CASE(f16_tag, 128); }
+  SAGE_CASE(f16_tag, 64);
+#undef SAGE_CASE
+}

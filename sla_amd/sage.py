@@ -1,0 +1,111 @@
+"""SageSLA: quantised forward of Sparse-Linear Attention (INT8 QK^T, FP8 PV).
+
+Mirrors ``SageSparseLinearAttention`` of ``SageSLA/core.py:33-163``: same constructor,
+parameters and forward; inference only.  The reference picks block sizes from the CUDA
+architecture (``SageSLA/core.py:90-94``); gfx950 has one path, BLKQ=128 / BLKK=64.
+"""
+from __future__ import annotations
+
+import torch
+import torch.nn as nn
+
+from . import _lib
+from .block_map import get_block_map
+from .linear import linear_fwd
+from .module import FEATURE_MAPS
+
+SAGE_BLKQ, SAGE_BLKK = 128, 64
+
+
+def quant_qk(q, k):
+    """Per-block INT8 q and mean-smoothed k.  Returns (q_int8, q_scale, k_int8, k_scale)."""
+    _lib.require_gpu(q, k)
+    B, H, L, D = q.shape
+    dt = _lib.dtype_code(q.dtype)
+    M, N = (L + SAGE_BLKQ - 1) // SAGE_BLKQ, (L + SAGE_BLKK - 1) // SAGE_BLKK
+    ws = _lib.workspace(_lib.WS_SAGE_QUANT, dt, B, H, L, D, SAGE_BLKQ, SAGE_BLKK, 0, q.device)
+    q8 = torch.empty((B, H, L, D), dtype=torch.int8, device=q.device)
+    k8 = torch.empty((B, H, L, D), dtype=torch.int8, device=q.device)
+    qs = torch.empty((B, H, M), dtype=torch.float32, device=q.device)
+    ks = torch.empty((B, H, N), dtype=torch.float32, device=q.device)
+    rc = _lib.load().sage_quant_qk(q.data_ptr(), k.data_ptr(), dt, B, H, L, D, SAGE_BLKQ, SAGE_BLKK, q8.data_ptr(),
+                                   qs.data_ptr(), k8.data_ptr(), ks.data_ptr(), ws.data_ptr(), ws.numel(),
+                                   _lib.stream_ptr(q.device))
+    _lib.check(rc)
+    return q8, qs, k8, ks
+
+
+def quant_v(v):
+    """Per-channel FP8 e4m3 v.  Returns (v_fp8 (B,H,L,D) float8_e4m3fn, v_scale (B,H,D) fp32)."""
+    _lib.require_gpu(v)
+    B, H, L, D = v.shape
+    dt = _lib.dtype_code(v.dtype)
+    ws = _lib.workspace(_lib.WS_SAGE_QUANT, dt, B, H, L, D, SAGE_BLKQ, SAGE_BLKK, 0, v.device)
+    v8 = torch.empty((B, H, L, D), dtype=torch.float8_e4m3fn, device=v.device)
+    vs = torch.empty((B, H, D), dtype=torch.float32, device=v.device)
+    rc = _lib.load().sage_quant_v(v.data_ptr(), dt, B, H, L, D, v8.data_ptr(), vs.data_ptr(), ws.data_ptr(), ws.numel(),
+                                  _lib.stream_ptr(v.device))
+    _lib.check(rc)
+    return v8, vs
+
+
+def sage_attn_fwd(q8, qs, k8, ks, v8, vs, lut, topk, out_dtype, qk_scale=None):
+    B, H, L, D = q8.shape
+    if qk_scale is None:
+        qk_scale = D ** -0.5
+    o = torch.empty((B, H, L, D), dtype=out_dtype, device=q8.device)
+    lut_bytes = 8 if lut.dtype == torch.int64 else 4
+    rc = _lib.load().sage_sparse_attn_fwd(q8.data_ptr(), qs.data_ptr(), k8.data_ptr(), ks.data_ptr(), v8.data_ptr(),
+                                          vs.data_ptr(), lut.data_ptr(), lut_bytes, o.data_ptr(),
+                                          _lib.dtype_code(out_dtype), B, H, L, D, SAGE_BLKQ, SAGE_BLKK, topk,
+                                          float(qk_scale), _lib.stream_ptr(q8.device))
+    _lib.check(rc)
+    return o
+
+
+class SageSparseLinearAttention(nn.Module):
+    def __init__(self, head_dim, topk, feature_map="softmax", use_bf16=True, tie_feature_map_qk=True, BLKQ=SAGE_BLKQ,
+                 BLKK=SAGE_BLKK):
+        r"""
+        Args:
+            head_dim: dimension of each head (64 or 128).
+            topk: ratio of keys selected for sparse attention, shared across all queries.
+            feature_map: feature map for linear attention, one of ['elu', 'relu', 'softmax'].
+            use_bf16: bfloat16 (default) or float16 compute.
+            tie_feature_map_qk: kept for signature compatibility.
+            BLKQ, BLKK: accepted because the reference's README passes them; only 128 / 64 exist.
+        """
+        super().__init__()
+        assert BLKQ == SAGE_BLKQ and BLKK == SAGE_BLKK, "SageSLA only supports BLKQ=128 and BLKK=64"
+        self.dtype = torch.bfloat16 if use_bf16 else torch.float16
+        self.topk = topk
+        self.proj_l = nn.Linear(head_dim, head_dim, dtype=torch.float32)
+        if feature_map not in FEATURE_MAPS:
+            raise NotImplementedError(f"Not supported feature map {feature_map}.")
+        self.feature_map = feature_map
+        self.init_weights_()
+
+    def init_weights_(self):
+        with torch.no_grad():
+            nn.init.zeros_(self.proj_l.weight)
+            nn.init.zeros_(self.proj_l.bias)
+
+    @torch.no_grad()
+    def forward(self, q, k, v, return_sparsity=False):
+        dtype = q.dtype
+        q = q.contiguous()
+        k = k.contiguous()
+        v = v.contiguous()
+        sparse_map, lut, real_topk = get_block_map(q, k, topk_ratio=self.topk, BLKQ=SAGE_BLKQ, BLKK=SAGE_BLKK)
+        q = q.to(self.dtype)
+        k = k.to(self.dtype)
+        v = v.to(self.dtype)
+        headdim = q.size(-1)
+        assert headdim in [64, 128], "headdim should be in [64, 128]. For other headdim, you can use padding and specify the softmax scale."
+        q8, qs, k8, ks = quant_qk(q, k)
+        v8, vs = quant_v(v)
+        o_s = sage_attn_fwd(q8, qs, k8, ks, v8, vs, lut, real_topk, self.dtype)
+        o = linear_fwd(q, k, v, self.proj_l.weight, self.proj_l.bias, o_s, self.feature_map).to(dtype)
+        if return_sparsity:
+            return o, real_topk / sparse_map.shape[-1]
+        return o
