@@ -76,6 +76,9 @@ def main():
               "forward); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
 
+    from sla_amd import build as _build
+    if not os.path.exists(_build.LIBPATH):
+        _build.build(force=True)
     import torch
     from sla_amd import SparseLinearAttention, get_block_map
     from sla_amd.inputs import CONFIGS, make_inputs, make_proj

@@ -11,6 +11,10 @@ if ROOT not in sys.path:
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+    # the kernels are loaded from the in-tree build; compile only when nothing has been built yet
+    from sla_amd import build as _build
+    if not os.path.exists(_build.LIBPATH):
+        _build.build(force=True)
 
 
 def pytest_collection_modifyitems(config, items):

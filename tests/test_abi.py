@@ -1,0 +1,117 @@
+"""CPU-only checks of the C ABI: the library loads, exports every symbol the header declares,
+and validates arguments before touching the device (so error paths need no GPU)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from sla_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "sla_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(sla_\w+|sage_\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    names = _declared_symbols()
+    assert len(names) >= 12
+    for n in names:
+        assert hasattr(lib, n), n
+    assert set(names) == set(_lib.SIGNATURES), "python binding and header disagree"
+    assert lib.sla_version() >= 1
+
+
+def test_workspace_sizes():
+    lib = _lib.load()
+    n = lib.sla_workspace_bytes(_lib.WS_BLOCK_MAP, _lib.SLA_BF16, 1, 12, 32760, 128, 64, 64, 25)
+    # chunk sums + column mean + pooled q/k + scores for cfg3
+    assert n >= 12 * (512 * 128 * 4 + 2 * 512 * 128 * 2 + 512 * 512 * 2)
+    assert lib.sla_workspace_bytes(_lib.WS_BLOCK_MAP, 7, 1, 1, 64, 64, 64, 64, 1) == _lib.ERR_BAD_ARG
+    assert lib.sla_workspace_bytes(99, 1, 1, 1, 64, 64, 64, 64, 1) == _lib.ERR_BAD_ARG
+    assert lib.sla_workspace_bytes(_lib.WS_SPARSE_BWD, 1, 0, 1, 64, 64, 64, 64, 1) == _lib.ERR_BAD_ARG
+    for op in (_lib.WS_SPARSE_BWD, _lib.WS_LINEAR_FWD, _lib.WS_LINEAR_BWD, _lib.WS_SAGE_QUANT):
+        assert lib.sla_workspace_bytes(op, 1, 2, 4, 4096, 128, 64, 64, 12) > 0
+
+
+FAKE = 0x1000  # non-null, 16-byte aligned; never dereferenced because validation fails first
+
+
+def test_attention_rejects_bad_shapes_before_launch():
+    lib = _lib.load()
+    args = dict(q=FAKE, k=FAKE, v=FAKE, lut=FAKE, lb=8, o=FAKE, lse=FAKE)
+
+    def call(dtype=1, B=1, H=1, L=128, D=128, BLKQ=64, BLKK=64, topk=1, **kw):
+        a = {**args, **kw}
+        return lib.sla_sparse_attn_fwd(a["q"], a["k"], a["v"], a["lut"], a["lb"], a["o"], a["lse"], dtype, B, H, L, D,
+                                       BLKQ, BLKK, topk, 0.1, None)
+    assert call(BLKQ=32) == _lib.ERR_UNSUPPORTED and "BLOCK_M" in _lib.last_error()
+    assert call(BLKK=128) == _lib.ERR_UNSUPPORTED and "BLOCK_N" in _lib.last_error()
+    assert call(D=96) == _lib.ERR_UNSUPPORTED
+    assert call(dtype=0) == _lib.ERR_UNSUPPORTED
+    assert call(topk=3) == _lib.ERR_BAD_ARG
+    assert call(L=0) == _lib.ERR_BAD_ARG
+    assert call(lb=2) == _lib.ERR_BAD_ARG
+    assert call(q=None) == _lib.ERR_BAD_ARG and "null" in _lib.last_error()
+    assert call(q=FAKE + 2) == _lib.ERR_BAD_ARG and "aligned" in _lib.last_error()
+    with pytest.raises(AssertionError):
+        _lib.check(call(BLKQ=32))
+    with pytest.raises(ValueError):
+        _lib.check(call(q=None))
+
+
+def test_other_entry_points_validate():
+    lib = _lib.load()
+    assert lib.sla_mean_pool(None, FAKE, 1, 1, 64, 64, 64, None) == _lib.ERR_BAD_ARG
+    assert lib.sla_mean_pool(FAKE, FAKE, 1, 1, 64, 60, 64, None) == _lib.ERR_UNSUPPORTED
+    assert lib.sla_block_map_fwd(FAKE, FAKE, 1, 1, 1, 128, 64, 64, 64, 5, FAKE, 1 << 30, FAKE, FAKE, 8, None) == _lib.ERR_BAD_ARG
+    assert lib.sla_block_map_fwd(FAKE, FAKE, 1, 1, 1, 128, 64, 64, 64, 1, FAKE, 16, FAKE, FAKE, 8, None) == _lib.ERR_WORKSPACE
+    assert lib.sla_linear_fwd(FAKE, FAKE, FAKE, FAKE, FAKE, None, FAKE, 1, 9, 1, 1, 64, 128, FAKE, 1 << 30, None) == _lib.ERR_BAD_ARG
+    assert lib.sla_linear_fwd(FAKE, FAKE, FAKE, FAKE, FAKE, None, FAKE, 1, 0, 1, 1, 64, 96, FAKE, 1 << 30, None) == _lib.ERR_UNSUPPORTED
+    assert lib.sla_linear_bwd(FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, 1, 0, 1, 1, 64, 128, FAKE, 8,
+                              None) == _lib.ERR_WORKSPACE
+    assert lib.sla_sparse_attn_bwd(FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, 8, FAKE, FAKE, FAKE, 1, 1, 1, 128, 128, 64,
+                                   64, 1, 0.1, FAKE, 8, None) == _lib.ERR_WORKSPACE
+    assert lib.sage_quant_qk(FAKE, FAKE, 1, 1, 1, 128, 128, 64, 64, FAKE, FAKE, FAKE, FAKE, FAKE, 1 << 30, None) == _lib.ERR_UNSUPPORTED
+    assert "BLKQ=128" in _lib.last_error()
+    assert lib.sage_quant_v(FAKE, 1, 1, 1, 128, 32, FAKE, FAKE, FAKE, 1 << 30, None) == _lib.ERR_UNSUPPORTED
+    assert "headdim" in _lib.last_error()
+    assert lib.sage_sparse_attn_fwd(FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, 8, FAKE, 1, 1, 1, 128, 128, 128, 64, 9, 0.1,
+                                    None) == _lib.ERR_BAD_ARG
+
+
+def test_host_api_mirrors_reference_names_and_errors():
+    import torch
+
+    import SageSLA
+    import sparse_linear_attention as sla
+    from sparse_linear_attention.kernel import _attention
+    from sparse_linear_attention.utils import get_block_map, mean_pool  # noqa: F401
+    mod = sla.SparseLinearAttention(head_dim=128, topk=0.2, feature_map="softmax", BLKQ=64, BLKK=64)
+    assert set(mod.state_dict()) == {"proj_l.weight", "proj_l.bias"}
+    assert mod.dtype == torch.bfloat16 and sla.SparseLinearAttention(64, 0.1, use_bf16=False).dtype == torch.float16
+    with pytest.raises(NotImplementedError):
+        sla.SparseLinearAttention(128, 0.2, feature_map="hedgehog")
+    sage = SageSLA.SageSparseLinearAttention(head_dim=128, topk=0.2, feature_map="softmax", BLKQ=128, BLKK=64)
+    assert set(sage.state_dict()) == {"proj_l.weight", "proj_l.bias"}
+    x = torch.zeros(1, 1, 128, 128, dtype=torch.bfloat16)
+    with pytest.raises(AssertionError):          # reference asserts contiguity first (kernel.py:243)
+        _attention.apply(x.transpose(-1, -2), x, x, torch.zeros(1, 1, 2, 2, dtype=torch.int8),
+                         torch.zeros(1, 1, 2, 1, dtype=torch.int64), 1, 64, 64)
+    with pytest.raises(AssertionError):          # BLOCK_M must be 64 or 128 (kernel.py:247)
+        _attention.apply(x, x, x, torch.zeros(1, 1, 2, 2, dtype=torch.int8), torch.zeros(1, 1, 2, 1, dtype=torch.int64),
+                         1, 32, 64)
+    with pytest.raises(RuntimeError):            # no CPU fallback: CPU tensors are refused loudly
+        mod(x, x, x)
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libsla_hip.so")
+    with pytest.raises(ImportError):
+        _lib.load()
