@@ -102,6 +102,15 @@ static __device__ __forceinline__ i16x8_t concat4(i16x4_t lo, i16x4_t hi) {
   return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
+// Buffer-addressed loads: offsets past `bytes` return zero, so ragged tails need no branches.
+typedef __attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned u32x4_t;
+static __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)bytes, 0x00020000);
+}
+static __device__ __forceinline__ i16x8_t buf_load_b128(__amdgpu_buffer_rsrc_t r, uint32_t byte_off) {
+  return __builtin_bit_cast(i16x8_t, __builtin_amdgcn_raw_buffer_load_b128(r, (int)byte_off, 0, 0));
+}
+
 static __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 static __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 

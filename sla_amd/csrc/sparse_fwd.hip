@@ -9,14 +9,15 @@
 // are then per-lane loops plus one exchange with lane^32, and the probabilities, once
 // packed to 16 bit, already sit in the B-operand layout of the second product
 // O^T = V^T P^T.  V^T fragments come out of LDS with the transposing 64-bit read.
-// K/V tiles go global -> registers -> LDS; the next tile's global loads are in flight
-// while the current tile is multiplied.
+// K/V tiles go global -> registers -> LDS; the next tile's K is in flight during QK^T and
+// softmax, its V during PV.  Register use is held to 256 so two waves share a SIMD and one
+// wave's softmax (vector ALU) overlaps the other's MFMAs.
 #include "common.h"
 
 namespace sla {
 
 template <typename Tag, int D, int BLKQ>
-__global__ __launch_bounds__(BLKQ * 2) void sparse_fwd_kernel(const uint16_t* __restrict__ q,
+__global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))) void sparse_fwd_kernel(const uint16_t* __restrict__ q,
                                                               const uint16_t* __restrict__ k,
                                                               const uint16_t* __restrict__ v,
                                                               const void* __restrict__ lut, int lut64,
@@ -48,20 +49,16 @@ __global__ __launch_bounds__(BLKQ * 2) void sparse_fwd_kernel(const uint16_t* __
   const int r = lane & 31;                  // query column (S^T, O^T) / key row (A operand)
 
   const size_t head_off = (size_t)bh * L * D;
-  const uint16_t* qh = q + head_off;
-  const uint16_t* kh = k + head_off;
-  const uint16_t* vh = v + head_off;
+  const uint32_t head_bytes = (uint32_t)L * D * 2;
+  const __amdgpu_buffer_rsrc_t qh = make_rsrc(q + head_off, head_bytes);
+  const __amdgpu_buffer_rsrc_t kh = make_rsrc(k + head_off, head_bytes);
+  const __amdgpu_buffer_rsrc_t vh = make_rsrc(v + head_off, head_bytes);
 
   // Q^T fragments (B operand), resident for the whole loop.
   const int qrow = mb * BLKQ + wave * 32 + r;
   i16x8_t qf[DC];
 #pragma unroll
-  for (int c = 0; c < DC; ++c) {
-    if (qrow < L)
-      qf[c] = *reinterpret_cast<const i16x8_t*>(qh + (size_t)qrow * D + 16 * c + 8 * g);
-    else
-      qf[c] = i16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
-  }
+  for (int c = 0; c < DC; ++c) qf[c] = buf_load_b128(qh, ((uint32_t)qrow * D + 16 * c + 8 * g) * 2);   // rows past L: 0
 
   const size_t lut_row = ((size_t)bh * Mblk + mb) * topk;
   auto lut_at = [&](int i) -> int {
@@ -69,29 +66,24 @@ __global__ __launch_bounds__(BLKQ * 2) void sparse_fwd_kernel(const uint16_t* __
                  : reinterpret_cast<const int*>(lut)[lut_row + i];
   };
 
-  i16x8_t kreg[NLD], vreg[NLD];
-  auto load_tile = [&](int nb) {
+  // One set of staging registers carries K of the next tile during the QK^T phase and V of the
+  // next tile during the PV phase (each LDS buffer is free while the other one is being read).
+  i16x8_t stg[NLD];
+  auto load_rows = [&](const __amdgpu_buffer_rsrc_t& base, int nb) {
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
       const int idx = tid + i * NT;
       const int row = idx / CPR, col = (idx % CPR) * 8;
-      const int grow = nb * BLKK + row;
-      if (grow < L) {
-        kreg[i] = *reinterpret_cast<const i16x8_t*>(kh + (size_t)grow * D + col);
-        vreg[i] = *reinterpret_cast<const i16x8_t*>(vh + (size_t)grow * D + col);
-      } else {
-        kreg[i] = i16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
-        vreg[i] = i16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
-      }
+      // rows past L lie beyond the buffer range and read as zero (0 * garbage could be NaN)
+      stg[i] = buf_load_b128(base, ((uint32_t)(nb * BLKK + row) * D + col) * 2);
     }
   };
-  auto store_tile = [&]() {
+  auto store_rows = [&](uint16_t* dst, int stride) {
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
       const int idx = tid + i * NT;
       const int row = idx / CPR, col = (idx % CPR) * 8;
-      *reinterpret_cast<i16x8_t*>(&sK[row * KSTR + col]) = kreg[i];
-      *reinterpret_cast<i16x8_t*>(&sV[row * VSTR + col]) = vreg[i];
+      *reinterpret_cast<i16x8_t*>(&dst[row * stride + col]) = stg[i];
     }
   };
 
@@ -107,39 +99,58 @@ __global__ __launch_bounds__(BLKQ * 2) void sparse_fwd_kernel(const uint16_t* __
   const int tr_row = (lane & 15) >> 2;
   const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
 
+  // look-up-table entries are fetched two tiles ahead so their latency never sits in front of
+  // the address computation of the K/V loads
   int nb = topk > 0 ? lut_at(0) : 0;
-  if (topk > 0) load_tile(nb);
+  int nb_next = topk > 1 ? lut_at(1) : 0;
+  if (topk > 0) {
+    load_rows(kh, nb);
+    store_rows(sK, KSTR);
+    load_rows(vh, nb);
+  }
+  __syncthreads();
 
   for (int it = 0; it < topk; ++it) {
-    __syncthreads();                       // previous tile fully consumed
-    store_tile();
-    __syncthreads();
+    // here: sK holds K of this tile, the staging registers hold V of this tile, sV is free
+    store_rows(sV, VSTR);
     const int kv_valid = L - nb * BLKK;    // rows of this tile that exist
-    if (it + 1 < topk) {
-      nb = lut_at(it + 1);
-      load_tile(nb);                       // in flight during the math below
+    const bool more = it + 1 < topk;
+    if (more) {
+      nb = nb_next;
+      nb_next = it + 2 < topk ? lut_at(it + 2) : 0;
+      load_rows(kh, nb);                   // K of the next tile, in flight during QK^T and softmax
     }
 
-    // ---- S^T = K Q^T : two 32-key sub-tiles ----
+    // ---- S^T = K Q^T : two 32-key sub-tiles, their MFMA chains interleaved ----
     f32x16_t s[2];
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
+    for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int i = 0; i < 16; ++i) s[t][i] = 0.f;
+    {
+      const uint16_t* k0 = &sK[r * KSTR + 8 * g];
+      i16x8_t ka[DC], kb[DC];
+#pragma unroll
+      for (int c = 0; c < DC; ++c) ka[c] = *reinterpret_cast<const i16x8_t*>(k0 + 16 * c);
+      __builtin_amdgcn_sched_barrier(0);   // keep all first-half fragments in flight before the first MFMA
 #pragma unroll
       for (int c = 0; c < DC; ++c) {
-        const i16x8_t a = *reinterpret_cast<const i16x8_t*>(&sK[(32 * t + r) * KSTR + 16 * c + 8 * g]);
-        s[t] = E::mfma32(a, qf[c], s[t]);
+        kb[c] = *reinterpret_cast<const i16x8_t*>(k0 + 32 * KSTR + 16 * c);
+        s[0] = E::mfma32(ka[c], qf[c], s[0]);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read ...
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // ... then one MFMA
       }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int c = 0; c < DC; ++c) s[1] = E::mfma32(kb[c], qf[c], s[1]);
     }
     if (kv_valid < BLKK) {                 // partial last key block: rows past L never take part
+      const int lim = kv_valid - 4 * g;    // key index of register i is 32t + 8(i/4) + i%4 + 4g
 #pragma unroll
       for (int t = 0; t < 2; ++t)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int key = 32 * t + 8 * (i >> 2) + 4 * g + (i & 3);
-          if (key >= kv_valid) s[t][i] = -INFINITY;
-        }
+        for (int i = 0; i < 16; ++i)
+          if (32 * t + 8 * (i >> 2) + (i & 3) >= lim) s[t][i] = -INFINITY;
     }
 
     // ---- online softmax (base 2) ----
@@ -169,24 +180,42 @@ __global__ __launch_bounds__(BLKQ * 2) void sparse_fwd_kernel(const uint16_t* __
         for (int i = 0; i < 16; ++i) oacc[dt][i] *= alpha;
     }
 
-    // ---- O^T += V^T P^T ----
+    __syncthreads();                       // sK fully consumed; sV stores visible
+    if (more) {
+      store_rows(sK, KSTR);
+      load_rows(vh, nb);                   // V of the next tile, in flight during PV
+    }
+
+    // ---- O^T += V^T P^T : four 16-key groups; the V^T fragments of the next group are read
+    //      (two transposing reads per fragment) while the current group's MFMAs run ----
+    {
+      auto read_group = [&](int gi, i16x8_t (&vf)[DT]) {
+        const int key0 = 16 * gi + 4 * g + tr_row;      // gi = 2t + c2
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+        for (int dt = 0; dt < DT; ++dt) {
+          const uint16_t* p0 = &sV[key0 * VSTR + 32 * dt + tr_col];
+          vf[dt] = concat4(lds_read_tr16(p0), lds_read_tr16(p0 + 8 * VSTR));
+        }
+      };
+      i16x8_t vf[2][DT];
+      read_group(0, vf[0]);
 #pragma unroll
-      for (int c2 = 0; c2 < 2; ++c2) {
+      for (int gi = 0; gi < 4; ++gi) {
+        const int t = gi >> 1, c2 = gi & 1;
         i32x4_t pw;
 #pragma unroll
         for (int j = 0; j < 4; ++j) pw[j] = (int)E::pack2(s[t][8 * c2 + 2 * j], s[t][8 * c2 + 2 * j + 1]);
         const i16x8_t pb = __builtin_bit_cast(i16x8_t, pw);
-        const int key0 = 32 * t + 16 * c2 + 4 * g + tr_row;
+        if (gi < 3) read_group(gi + 1, vf[(gi + 1) & 1]);
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
-          const uint16_t* p0 = &sV[key0 * VSTR + 32 * dt + tr_col];
-          const i16x4_t lo = lds_read_tr16(p0);
-          const i16x4_t hi = lds_read_tr16(p0 + 8 * VSTR);
-          oacc[dt] = E::mfma32(concat4(lo, hi), pb, oacc[dt]);
+          oacc[dt] = E::mfma32(vf[gi & 1][dt], pb, oacc[dt]);
+          if (gi < 3) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         }
       }
+    }
+    __syncthreads();                       // sV fully consumed; sK stores visible
   }
 
   // ---- epilogue ----
@@ -242,6 +271,7 @@ int validate_attn_shape(int dtype, int B, int H, int L, int D, int BLKQ, int BLK
   SLA_REQUIRE(lut_elem_bytes == 4 || lut_elem_bytes == 8, SLA_ERR_BAD_ARG, "lut_elem_bytes must be 4 or 8, got %d",
               lut_elem_bytes);
   SLA_REQUIRE((int64_t)B * H * cdiv(L, 64) < (1ll << 31) - 8, SLA_ERR_UNSUPPORTED, "too many blocks");
+  SLA_REQUIRE((int64_t)(L + 128) * D * 2 < (1ll << 32), SLA_ERR_UNSUPPORTED, "one head exceeds 4 GiB");
   return SLA_OK;
 }
 
