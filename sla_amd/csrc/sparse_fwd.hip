@@ -92,8 +92,6 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
   for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
     for (int i = 0; i < 16; ++i) oacc[dt][i] = 0.f;
-  float m_run = -INFINITY;   // running maximum of the scaled scores of this lane's query
-  float l_run = 0.f;         // this lane's share of the running sum (its 32 of the 64 key rows)
 
   // transposed-read addressing of V: lane i of a 16-lane group points at row i/4, cols 4*(i%4)
   const int tr_row = (lane & 15) >> 2;
@@ -110,113 +108,171 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
   }
   __syncthreads();
 
+  // Reference maximum of the online softmax.  It is only moved when a sub-tile's maximum exceeds it
+  // by more than TAU (in log2 units): probabilities are then at most 2^TAU, exact in fp32 and bf16,
+  // and the final 1/l normalisation is unchanged.  Without a per-tile maximum on the critical path
+  // the exponentials of one 32-key sub-tile can be issued in the shadow of the other sub-tile's MFMAs.
+  constexpr float TAU = 8.0f;
+  float m_used = -INFINITY;
+  float l_run = 0.f;         // this lane's share of the running sum (its 32 of the 64 key rows)
+  i16x8_t pb[2][2];          // packed probabilities of the two sub-tiles, B operands of the PV product
+
+  // moves the reference maximum to at least `mx` (this lane's raw maximum of the sub-tile) and rescales
+  // everything accumulated so far; `done` = number of sub-tiles of this tile already exponentiated
+  auto raise_reference = [&](float mx, int done) {
+    mx = fmaxf(mx, __shfl_xor(mx, 32)) * scale_log2e;
+    const float m_new = fmaxf(m_used, mx);
+    const float f = fast_exp2(m_used - m_new);     // 0 on the first tile (m_used = -inf)
+    m_used = m_new;
+    l_run *= f;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) oacc[dt][i] *= f;
+    if (done > 0) {
+#pragma unroll
+      for (int c2 = 0; c2 < 2; ++c2) {
+        i32x4_t w = __builtin_bit_cast(i32x4_t, pb[0][c2]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const uint32_t u = (uint32_t)w[j];
+          w[j] = (int)E::pack2(E::to_float((uint16_t)(u & 0xffff)) * f, E::to_float((uint16_t)(u >> 16)) * f);
+        }
+        pb[0][c2] = __builtin_bit_cast(i16x8_t, w);
+      }
+    }
+  };
+  // exp2 of one sub-tile against the current reference; adds to l_run; packs into pb[t]
+  auto softmax_subtile = [&](f32x16_t& sv, int t) {
+    float psum = 0.f;
+#pragma unroll
+    for (int c2 = 0; c2 < 2; ++c2) {
+      i32x4_t pw;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float p0 = fast_exp2(__builtin_fmaf(sv[8 * c2 + 2 * j], scale_log2e, -m_used));
+        const float p1 = fast_exp2(__builtin_fmaf(sv[8 * c2 + 2 * j + 1], scale_log2e, -m_used));
+        psum += p0 + p1;
+        pw[j] = (int)E::pack2(p0, p1);
+      }
+      pb[t][c2] = __builtin_bit_cast(i16x8_t, pw);
+    }
+    l_run += psum;
+  };
+  auto row_max = [&](const f32x16_t& sv) {
+    float mx = sv[0];
+#pragma unroll
+    for (int i = 1; i < 16; ++i) mx = fmaxf(mx, sv[i]);
+    return mx;
+  };
+  auto mask_tail = [&](f32x16_t& sv, int t, int kv_valid) {
+    const int lim = kv_valid - 4 * g;      // key index of register i is 32t + 8(i/4) + i%4 + 4g
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+      if (32 * t + 8 * (i >> 2) + (i & 3) >= lim) sv[i] = -INFINITY;
+  };
+  auto read_vgroup = [&](int gi, i16x8_t (&vf)[DT]) {   // V^T fragments of 16-key group gi = 2t + c2
+    const int key0 = 16 * gi + 4 * g + tr_row;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      const uint16_t* p0 = &sV[key0 * VSTR + 32 * dt + tr_col];
+      vf[dt] = concat4(lds_read_tr16(p0), lds_read_tr16(p0 + 8 * VSTR));
+    }
+  };
+
   for (int it = 0; it < topk; ++it) {
     // here: sK holds K of this tile, the staging registers hold V of this tile, sV is free
+    const uint16_t* k0 = &sK[r * KSTR + 8 * g];
+    i16x8_t ka[DC], kb[DC];
+#pragma unroll
+    for (int c = 0; c < DC; ++c) ka[c] = *reinterpret_cast<const i16x8_t*>(k0 + 16 * c);
     store_rows(sV, VSTR);
     const int kv_valid = L - nb * BLKK;    // rows of this tile that exist
+    const bool tail = kv_valid < BLKK;
     const bool more = it + 1 < topk;
     if (more) {
       nb = nb_next;
       nb_next = it + 2 < topk ? lut_at(it + 2) : 0;
-      load_rows(kh, nb);                   // K of the next tile, in flight during QK^T and softmax
+      load_rows(kh, nb);                   // K of the next tile, in flight until the middle of this one
     }
 
-    // ---- S^T = K Q^T : two 32-key sub-tiles, their MFMA chains interleaved ----
-    f32x16_t s[2];
+    // ---- A: S0^T = K[0:32] Q^T, with the fragments of K[32:64] fetched in its shadow ----
+    f32x16_t s0, s1;
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) s[t][i] = 0.f;
-    {
-      const uint16_t* k0 = &sK[r * KSTR + 8 * g];
-      i16x8_t ka[DC], kb[DC];
-#pragma unroll
-      for (int c = 0; c < DC; ++c) ka[c] = *reinterpret_cast<const i16x8_t*>(k0 + 16 * c);
-      __builtin_amdgcn_sched_barrier(0);   // keep all first-half fragments in flight before the first MFMA
-#pragma unroll
-      for (int c = 0; c < DC; ++c) {
-        kb[c] = *reinterpret_cast<const i16x8_t*>(k0 + 32 * KSTR + 16 * c);
-        s[0] = E::mfma32(ka[c], qf[c], s[0]);
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read ...
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // ... then one MFMA
-      }
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int c = 0; c < DC; ++c) s[1] = E::mfma32(kb[c], qf[c], s[1]);
+    for (int i = 0; i < 16; ++i) {
+      s0[i] = 0.f;
+      s1[i] = 0.f;
     }
-    if (kv_valid < BLKK) {                 // partial last key block: rows past L never take part
-      const int lim = kv_valid - 4 * g;    // key index of register i is 32t + 8(i/4) + i%4 + 4g
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int i = 0; i < 16; ++i)
-          if (32 * t + 8 * (i >> 2) + (i & 3) >= lim) s[t][i] = -INFINITY;
+    for (int c = 0; c < DC; ++c) {
+      kb[c] = *reinterpret_cast<const i16x8_t*>(k0 + 32 * KSTR + 16 * c);
+      s0 = E::mfma32(ka[c], qf[c], s0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
     }
-
-    // ---- online softmax (base 2) ----
-    float mx = s[0][0];
-#pragma unroll
-    for (int t = 0; t < 2; ++t)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[t][i]);
-    mx = fmaxf(mx, __shfl_xor(mx, 32));
-    const float m_new = fmaxf(m_run, mx * scale_log2e);
-    const float alpha = fast_exp2(m_run - m_new);
-    float psum = 0.f;
-#pragma unroll
-    for (int t = 0; t < 2; ++t)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const float p = fast_exp2(__builtin_fmaf(s[t][i], scale_log2e, -m_new));
-        s[t][i] = p;
-        psum += p;
-      }
-    l_run = l_run * alpha + psum;
-    m_run = m_new;
-    if (__any(alpha != 1.0f)) {
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) oacc[dt][i] *= alpha;
+    __builtin_amdgcn_sched_barrier(0);
+    // rare path (one branch, so the common path stays a straight line): the reference maximum has
+    // to move, or this is the partial last key block whose missing rows are masked out first
+    if (tail || __any(row_max(s0) * scale_log2e > m_used + TAU)) {
+      if (tail) mask_tail(s0, 0, kv_valid);
+      raise_reference(row_max(s0), 0);
     }
-
-    __syncthreads();                       // sK fully consumed; sV stores visible
+    __syncthreads();                       // every wave has its K fragments: sK is free; sV stores visible
     if (more) {
       store_rows(sK, KSTR);
-      load_rows(vh, nb);                   // V of the next tile, in flight during PV
+      load_rows(vh, nb);                   // V of the next tile, in flight until the top of the next one
     }
 
-    // ---- O^T += V^T P^T : four 16-key groups; the V^T fragments of the next group are read
-    //      (two transposing reads per fragment) while the current group's MFMAs run ----
-    {
-      auto read_group = [&](int gi, i16x8_t (&vf)[DT]) {
-        const int key0 = 16 * gi + 4 * g + tr_row;      // gi = 2t + c2
+    // ---- B: S1^T = K[32:64] Q^T  ||  exponentials of S0 ; V^T fragments of keys 0..31 fetched ----
+    // (the group barriers fix the issue order: after every MFMA two LDS reads and seven vector-ALU
+    //  instructions, two of them exponentials, are issued while the matrix core works)
+    i16x8_t vf0[DT], vf1[DT];
+    __builtin_amdgcn_sched_barrier(0);
+    read_vgroup(0, vf0);
+    read_vgroup(1, vf1);
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-          const uint16_t* p0 = &sV[key0 * VSTR + 32 * dt + tr_col];
-          vf[dt] = concat4(lds_read_tr16(p0), lds_read_tr16(p0 + 8 * VSTR));
-        }
-      };
-      i16x8_t vf[2][DT];
-      read_group(0, vf[0]);
+    for (int c = 0; c < DC; ++c) s1 = E::mfma32(kb[c], qf[c], s1);
+    softmax_subtile(s0, 0);
 #pragma unroll
-      for (int gi = 0; gi < 4; ++gi) {
-        const int t = gi >> 1, c2 = gi & 1;
-        i32x4_t pw;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) pw[j] = (int)E::pack2(s[t][8 * c2 + 2 * j], s[t][8 * c2 + 2 * j + 1]);
-        const i16x8_t pb = __builtin_bit_cast(i16x8_t, pw);
-        if (gi < 3) read_group(gi + 1, vf[(gi + 1) & 1]);
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-          oacc[dt] = E::mfma32(vf[gi & 1][dt], pb, oacc[dt]);
-          if (gi < 3) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        }
-      }
+    for (int c = 0; c < DC; ++c) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);
+      __builtin_amdgcn_sched_group_barrier(0x400, 2, 0);
     }
+    __builtin_amdgcn_sched_barrier(0);
+    if (tail || __any(row_max(s1) * scale_log2e > m_used + TAU)) {
+      if (tail) mask_tail(s1, 1, kv_valid);
+      raise_reference(row_max(s1), 1);
+    }
+
+    // ---- C: O^T += V[0:32]^T P0^T  ||  exponentials of S1 ; V^T fragments of keys 32..63 fetched ----
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) oacc[dt] = E::mfma32(vf0[dt], pb[0][0], oacc[dt]);
+    read_vgroup(2, vf0);
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) oacc[dt] = E::mfma32(vf1[dt], pb[0][1], oacc[dt]);
+    read_vgroup(3, vf1);
+    softmax_subtile(s1, 1);
+#pragma unroll
+    for (int c = 0; c < 2 * DT; ++c) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);
+      __builtin_amdgcn_sched_group_barrier(0x400, 2, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- D: O^T += V[32:64]^T P1^T ----
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) oacc[dt] = E::mfma32(vf0[dt], pb[1][0], oacc[dt]);
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) oacc[dt] = E::mfma32(vf1[dt], pb[1][1], oacc[dt]);
     __syncthreads();                       // sV fully consumed; sK stores visible
   }
+  const float m_run = m_used;
 
   // ---- epilogue ----
   const float l_tot = l_run + __shfl_xor(l_run, 32);
