@@ -34,8 +34,9 @@ Two things are fixed here that the reference leaves open, because without them
     - block mean: rows of the block added one by one in ascending row order,
       then one IEEE division by the real row count;
     - column mean of K: rows added one by one inside chunks of
-      ``KMEAN_CHUNK`` rows, the chunk sums added one by one in ascending chunk
-      order, one IEEE division by L;
+      ``KMEAN_CHUNK`` rows; the chunk sums added one by one inside groups of
+      ``KMEAN_GROUP`` consecutive chunks; the group sums added one by one in
+      ascending order; one IEEE division by L;
     - pooled score: ``acc = acc + (a_d * b_d)`` for d ascending, product and sum
       rounded separately (no fused multiply-add).
   All results are then rounded to the input dtype exactly where the reference
@@ -59,7 +60,8 @@ import math
 import torch
 import torch.nn.functional as F
 
-KMEAN_CHUNK = 64
+KMEAN_CHUNK = 64      # rows per level-1 sum of the K column mean
+KMEAN_GROUP = 32      # level-1 sums per level-2 sum
 LOG2E = 1.4426950408889634
 
 
@@ -104,7 +106,8 @@ def k_column_mean(k: torch.Tensor) -> torch.Tensor:
     """``torch.mean(k, dim=-2, keepdim=True)`` (utils.py:56) in the fixed order."""
     B, H, L, D = k.shape
     chunk_sums = _seq_sum_rows(_blocked(k, KMEAN_CHUNK))    # (B,H,nchunk,D)
-    total = _seq_sum_rows(chunk_sums)                       # (B,H,D)
+    group_sums = _seq_sum_rows(_blocked(chunk_sums, KMEAN_GROUP))
+    total = _seq_sum_rows(group_sums)                       # (B,H,D)
     return (total / float(L)).to(k.dtype).unsqueeze(-2)
 
 

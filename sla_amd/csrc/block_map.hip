@@ -7,8 +7,8 @@
 // All of this is HBM-bound streaming or tiny, so it runs on the vector ALUs with a
 // FIXED fp32 summation order that a CPU checker can follow bit for bit:
 //   block mean : rows added one at a time in ascending order, one IEEE division;
-//   column mean: 64-row chunk sums (same order), chunk sums added in ascending order,
-//                one IEEE division by L;
+//   column mean: 64-row chunk sums (same order); groups of 32 consecutive chunk sums added in
+//                ascending order; group sums added in ascending order; one IEEE division by L;
 //   score      : acc = acc + (a_d * b_d), d ascending, no fused multiply-add.
 // Selection is by (score descending, index ascending); -0.0 == +0.0.
 #include "common.h"
@@ -17,23 +17,28 @@
 
 namespace sla {
 
-constexpr int KMEAN_CHUNK = 64;
+constexpr int KMEAN_CHUNK = 64;   // rows per level-1 sum
+constexpr int KMEAN_GROUP = 32;   // level-1 sums per level-2 sum
 
+// KEY_LOW_BIT: lowest bit of the fp32 image of a value of this type that can be non-zero.
 struct IoF32 {
   typedef float raw;
   static constexpr int VEC = 4;
+  static constexpr int KEY_LOW_BIT = 0;
   static __device__ __forceinline__ float ld(raw x) { return x; }
   static __device__ __forceinline__ raw st(float x) { return x; }
 };
 struct IoBf16 {
   typedef uint16_t raw;
   static constexpr int VEC = 8;
+  static constexpr int KEY_LOW_BIT = 16;
   static __device__ __forceinline__ float ld(raw x) { return Elem<bf16_tag>::to_float(x); }
   static __device__ __forceinline__ raw st(float x) { return Elem<bf16_tag>::from_float(x); }
 };
 struct IoF16 {
   typedef uint16_t raw;
   static constexpr int VEC = 8;
+  static constexpr int KEY_LOW_BIT = 13;
   static __device__ __forceinline__ float ld(raw x) { return Elem<f16_tag>::to_float(x); }
   static __device__ __forceinline__ raw st(float x) { return Elem<f16_tag>::from_float(x); }
 };
@@ -95,17 +100,33 @@ __global__ __launch_bounds__(256) void pool_kernel(const typename IO::raw* __res
   }
 }
 
-// colmean[bh][d] = (sum over chunks, ascending) / L, rounded to the input dtype.
+// Column mean of K, levels 2 and 3 of the fixed summation order:
+//   group_sums[bh][g][d] = chunk sums of group g (KMEAN_GROUP consecutive chunks) added in ascending order;
+//   colmean[bh][d]       = (group sums added in ascending order) / L, rounded to the input dtype.
+__global__ __launch_bounds__(128) void colmean_group_kernel(const float* __restrict__ chunk_sums,
+                                                            float* __restrict__ group_sums, int nchunk, int ngroup, int D) {
+  const int g = blockIdx.x, bh = blockIdx.y;
+  const int c0 = g * KMEAN_GROUP;
+  const int n = min(KMEAN_GROUP, nchunk - c0);
+  for (int d = threadIdx.x; d < D; d += 128) {
+    const float* p = chunk_sums + ((size_t)bh * nchunk + c0) * D + d;
+    float acc = 0.f;
+#pragma unroll 8
+    for (int i = 0; i < n; ++i) acc = acc + p[(size_t)i * D];
+    group_sums[((size_t)bh * ngroup + g) * D + d] = acc;
+  }
+}
+
 template <typename IO>
-__global__ void colmean_kernel(const float* __restrict__ chunk_sums, typename IO::raw* __restrict__ colmean, int nchunk,
-                               int D, int L) {
+__global__ __launch_bounds__(128) void colmean_kernel(const float* __restrict__ group_sums,
+                                                      typename IO::raw* __restrict__ colmean, int ngroup, int D, int L) {
   const int bh = blockIdx.y;
   const int d = blockIdx.x * blockDim.x + threadIdx.x;
   if (d >= D) return;
-  const float* p = chunk_sums + (size_t)bh * nchunk * D + d;
+  const float* p = group_sums + (size_t)bh * ngroup * D + d;
   float acc = 0.f;
 #pragma unroll 8
-  for (int i = 0; i < nchunk; ++i) acc = acc + p[(size_t)i * D];
+  for (int i = 0; i < ngroup; ++i) acc = acc + p[(size_t)i * D];
   colmean[(size_t)bh * D + d] = IO::st(acc / (float)L);
 }
 
@@ -164,50 +185,77 @@ __global__ __launch_bounds__(256) void score_kernel(const typename IO::raw* __re
   }
 }
 
-// Monotone map float -> uint32 (larger float = larger key); -0.0 is folded onto +0.0.
+// Monotone map float -> uint32 (larger float = larger key); -0.0 is folded onto +0.0.  The LOW_BIT
+// low bits (zero in the fp32 image of every value of the score dtype) are cleared, also for negative
+// values where the complement would set them, so the radix select can stop at LOW_BIT.
+template <int LOW_BIT>
 static __device__ __forceinline__ uint32_t order_key(float f) {
   uint32_t u = __float_as_uint(f);
   if (u == 0x80000000u) u = 0u;
-  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+  u = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+  return u & ~((1u << LOW_BIT) - 1u);
 }
 
-// One wavefront per (bh, m) row: radix-select the T-th largest key bit by bit with ballot
-// counts, then emit winners in ascending index order (ties at the threshold value go to
-// the lowest indices).  Writes the int8 map row and the look-up-table row.
-template <typename IO>
-__global__ __launch_bounds__(64) void topk_kernel(const typename IO::raw* __restrict__ score,
-                                                  int8_t* __restrict__ sparse_map, void* __restrict__ lut, int lut64, int N,
-                                                  int T) {
-  extern __shared__ uint32_t keys[];
-  const size_t row = blockIdx.x;
-  const int lane = threadIdx.x;
+// One wavefront per (bh, m) row (four rows per workgroup): radix-select the T-th largest key bit
+// by bit with ballot counts, then emit winners in ascending index order (ties at the threshold
+// value go to the lowest indices).  Writes the int8 map row and the look-up-table row.
+// EPL > 0: the row's keys live in EPL registers per lane (N <= 64*EPL); EPL == 0: keys in LDS.
+// LOW_BIT: lowest key bit that can differ (16 for 16-bit score dtypes, whose low bits are zero).
+template <typename IO, int EPL, int LOW_BIT>
+__global__ __launch_bounds__(256) void topk_kernel(const typename IO::raw* __restrict__ score,
+                                                   int8_t* __restrict__ sparse_map, void* __restrict__ lut, int lut64, int N,
+                                                   int T, size_t nrows) {
+  extern __shared__ uint32_t lds_keys[];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const size_t row = (size_t)blockIdx.x * 4 + wave;
+  if (row >= nrows) return;
   const typename IO::raw* s = score + row * N;
-  for (int i = lane; i < N; i += 64) keys[i] = order_key(IO::ld(s[i]));
-  __syncthreads();
+  constexpr int NR = EPL > 0 ? EPL : 1;
+  uint32_t kreg[NR];
+  uint32_t* keys = lds_keys + (size_t)wave * (EPL > 0 ? 0 : N);
+  const int nit = EPL > 0 ? EPL : (N + 63) / 64;
+  // out-of-range slots hold key 0, below every real key (a real key has bit 31 set or is > 0 ... except
+  // the most negative NaN pattern); they are excluded explicitly by the index test below.
+  if (EPL > 0) {
+#pragma unroll
+    for (int e = 0; e < NR; ++e) {
+      const int i = e * 64 + lane;
+      kreg[e] = i < N ? order_key<LOW_BIT>(IO::ld(s[i])) : 0u;
+    }
+  } else {
+    for (int i = lane; i < N; i += 64) keys[i] = order_key<LOW_BIT>(IO::ld(s[i]));
+  }
+  auto key_at = [&](int e) -> uint32_t {
+    if (EPL > 0) return kreg[e < NR ? e : 0];
+    const int i = e * 64 + lane;
+    return i < N ? keys[i] : 0u;
+  };
   uint32_t thr = 0;
-  for (int bit = 31; bit >= 0; --bit) {
+  for (int bit = 31; bit >= LOW_BIT; --bit) {
     const uint32_t cand = thr | (1u << bit);
     int cnt = 0;
-    for (int i0 = 0; i0 < N; i0 += 64) {
-      const int i = i0 + lane;
-      const bool ge = (i < N) && (keys[i] >= cand);
-      cnt += __popcll(__ballot(ge));
+    if (EPL > 0) {
+#pragma unroll
+      for (int e = 0; e < NR; ++e) cnt += __popcll(__ballot((e * 64 + lane < N) && kreg[e] >= cand));
+    } else {
+      for (int e = 0; e < nit; ++e) cnt += __popcll(__ballot((e * 64 + lane < N) && key_at(e) >= cand));
     }
     if (cnt >= T) thr = cand;
   }
   int n_gt = 0;
-  for (int i0 = 0; i0 < N; i0 += 64) {
-    const int i = i0 + lane;
-    n_gt += __popcll(__ballot((i < N) && (keys[i] > thr)));
+  if (EPL > 0) {
+#pragma unroll
+    for (int e = 0; e < NR; ++e) n_gt += __popcll(__ballot((e * 64 + lane < N) && kreg[e] > thr));
+  } else {
+    for (int e = 0; e < nit; ++e) n_gt += __popcll(__ballot((e * 64 + lane < N) && key_at(e) > thr));
   }
   const int need_eq = T - n_gt;
   int run_eq = 0, run_sel = 0;
   const unsigned long long lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
   int8_t* mrow = sparse_map + row * N;
-  for (int i0 = 0; i0 < N; i0 += 64) {
-    const int i = i0 + lane;
+  auto emit = [&](int e, uint32_t kv) {
+    const int i = e * 64 + lane;
     const bool in = i < N;
-    const uint32_t kv = in ? keys[i] : 0u;
     const bool gt = in && kv > thr;
     const bool eq = in && kv == thr;
     const unsigned long long beq = __ballot(eq);
@@ -224,11 +272,33 @@ __global__ __launch_bounds__(64) void topk_kernel(const typename IO::raw* __rest
     }
     run_eq += __popcll(beq);
     run_sel += __popcll(bsel);
+  };
+  if (EPL > 0) {
+#pragma unroll
+    for (int e = 0; e < NR; ++e)
+      if (e * 64 < N) emit(e, kreg[e]);
+  } else {
+    for (int e = 0; e < nit; ++e) emit(e, key_at(e));
   }
 }
 
+template <typename IO>
+static void launch_topk(const typename IO::raw* score, int8_t* sparse_map, void* lut, int lut64, int N, int T, size_t nrows,
+                        hipStream_t st) {
+  constexpr int LOW = IO::KEY_LOW_BIT;
+  const dim3 grid((unsigned)((nrows + 3) / 4)), block(256);
+  if (N <= 512)
+    hipLaunchKernelGGL((topk_kernel<IO, 8, LOW>), grid, block, 0, st, score, sparse_map, lut, lut64, N, T, nrows);
+  else if (N <= 1280)
+    hipLaunchKernelGGL((topk_kernel<IO, 20, LOW>), grid, block, 0, st, score, sparse_map, lut, lut64, N, T, nrows);
+  else if (N <= 2048)
+    hipLaunchKernelGGL((topk_kernel<IO, 32, LOW>), grid, block, 0, st, score, sparse_map, lut, lut64, N, T, nrows);
+  else
+    hipLaunchKernelGGL((topk_kernel<IO, 0, LOW>), grid, block, (size_t)N * 16, st, score, sparse_map, lut, lut64, N, T, nrows);
+}
+
 struct MapWs {
-  size_t chunk_sums, colmean, pq, pk, score, total;
+  size_t chunk_sums, group_sums, colmean, pq, pk, score, total;
 };
 
 static MapWs map_ws(int dtype, int BH, int L, int D, int BLKQ, int BLKK) {
@@ -237,6 +307,7 @@ static MapWs map_ws(int dtype, int BH, int L, int D, int BLKQ, int BLKK) {
   MapWs w;
   size_t off = 0;
   w.chunk_sums = off; off += align_up((int64_t)BH * nchunk * D * 4, 256);
+  w.group_sums = off; off += align_up((int64_t)BH * cdiv((int)nchunk, KMEAN_GROUP) * D * 4, 256);
   w.colmean = off;    off += align_up((int64_t)BH * D * eb, 256);
   w.pq = off;         off += align_up((int64_t)BH * M * D * eb, 256);
   w.pk = off;         off += align_up((int64_t)BH * N * D * eb, 256);
@@ -270,41 +341,49 @@ static void launch_pool(const void* x, const void* colmean, void* out, int BH, i
 }
 
 template <typename IO>
+static void launch_k_colmean_t(const void* k, int BH, int L, int D, float* chunk_sums, float* group_sums,
+                               typename IO::raw* colmean, hipStream_t st) {
+  const int nchunk = cdiv(L, KMEAN_CHUNK), ngroup = cdiv(nchunk, KMEAN_GROUP);
+  launch_pool<IO, 0>(k, nullptr, chunk_sums, BH, L, D, KMEAN_CHUNK, st);
+  hipLaunchKernelGGL(colmean_group_kernel, dim3(ngroup, BH), dim3(128), 0, st, chunk_sums, group_sums, nchunk, ngroup, D);
+  hipLaunchKernelGGL((colmean_kernel<IO>), dim3(cdiv(D, 128), BH), dim3(128), 0, st, group_sums, colmean, ngroup, D, L);
+}
+
+template <typename IO>
 static int block_map_impl(const void* q, const void* k, int dtype, int BH, int L, int D, int BLKQ, int BLKK, int topk,
                           char* ws, int8_t* sparse_map, void* lut, int lut64, hipStream_t st) {
   const MapWs w = map_ws(dtype, BH, L, D, BLKQ, BLKK);
-  const int M = cdiv(L, BLKQ), N = cdiv(L, BLKK), nchunk = cdiv(L, KMEAN_CHUNK);
+  const int M = cdiv(L, BLKQ), N = cdiv(L, BLKK);
   float* chunk_sums = (float*)(ws + w.chunk_sums);
   typename IO::raw* colmean = (typename IO::raw*)(ws + w.colmean);
   typename IO::raw* pq = (typename IO::raw*)(ws + w.pq);
   typename IO::raw* pk = (typename IO::raw*)(ws + w.pk);
   typename IO::raw* score = (typename IO::raw*)(ws + w.score);
-  launch_pool<IO, 0>(k, nullptr, chunk_sums, BH, L, D, KMEAN_CHUNK, st);
-  hipLaunchKernelGGL((colmean_kernel<IO>), dim3(cdiv(D, 128), BH), dim3(128), 0, st, chunk_sums, colmean, nchunk, D, L);
+  launch_k_colmean_t<IO>(k, BH, L, D, chunk_sums, (float*)(ws + w.group_sums), colmean, st);
   launch_pool<IO, 1>(q, nullptr, pq, BH, L, D, BLKQ, st);
   launch_pool<IO, 2>(k, colmean, pk, BH, L, D, BLKK, st);
   hipLaunchKernelGGL((score_kernel<IO>), dim3(cdiv(N, 64), cdiv(M, 64), BH), dim3(256), 0, st, pq, pk, score, M, N, D);
   // topk == 0 selects nothing: the kernel then only clears the map row.
-  hipLaunchKernelGGL((topk_kernel<IO>), dim3((unsigned)((size_t)BH * M)), dim3(64), (size_t)N * 4, st, score, sparse_map,
-                     lut, lut64, N, topk);
+  launch_topk<IO>(score, sparse_map, lut, lut64, N, topk, (size_t)BH * M, st);
   return check_launch("block map");
 }
 
-// Column mean of k over L in the fixed order (chunk sums, then chunks), rounded to `dtype`.
-// chunk_sums: fp32 (BH, ceil(L/64), D) scratch; colmean: (BH, D) in `dtype`.
-void launch_k_colmean(const void* k, int dtype, int BH, int L, int D, float* chunk_sums, void* colmean, hipStream_t st) {
-  const int nchunk = cdiv(L, KMEAN_CHUNK);
-  const dim3 grid(cdiv(D, 128), BH);
-  if (dtype == SLA_F32) {
-    launch_pool<IoF32, 0>(k, nullptr, chunk_sums, BH, L, D, KMEAN_CHUNK, st);
-    hipLaunchKernelGGL((colmean_kernel<IoF32>), grid, dim3(128), 0, st, chunk_sums, (float*)colmean, nchunk, D, L);
-  } else if (dtype == SLA_BF16) {
-    launch_pool<IoBf16, 0>(k, nullptr, chunk_sums, BH, L, D, KMEAN_CHUNK, st);
-    hipLaunchKernelGGL((colmean_kernel<IoBf16>), grid, dim3(128), 0, st, chunk_sums, (uint16_t*)colmean, nchunk, D, L);
-  } else {
-    launch_pool<IoF16, 0>(k, nullptr, chunk_sums, BH, L, D, KMEAN_CHUNK, st);
-    hipLaunchKernelGGL((colmean_kernel<IoF16>), grid, dim3(128), 0, st, chunk_sums, (uint16_t*)colmean, nchunk, D, L);
-  }
+// Column mean of k over L in the fixed order, rounded to `dtype`.  scratch: fp32, at least
+// k_colmean_scratch_floats(BH, L, D) elements; colmean: (BH, D) in `dtype`.
+int64_t k_colmean_scratch_floats(int BH, int L, int D) {
+  const int64_t nchunk = cdiv(L, KMEAN_CHUNK), ngroup = cdiv((int)nchunk, KMEAN_GROUP);
+  return (int64_t)BH * (nchunk + ngroup) * D;
+}
+void launch_k_colmean(const void* k, int dtype, int BH, int L, int D, float* scratch, void* colmean, hipStream_t st) {
+  const int64_t nchunk = cdiv(L, KMEAN_CHUNK);
+  float* chunk_sums = scratch;
+  float* group_sums = scratch + (int64_t)BH * nchunk * D;
+  if (dtype == SLA_F32)
+    launch_k_colmean_t<IoF32>(k, BH, L, D, chunk_sums, group_sums, (float*)colmean, st);
+  else if (dtype == SLA_BF16)
+    launch_k_colmean_t<IoBf16>(k, BH, L, D, chunk_sums, group_sums, (uint16_t*)colmean, st);
+  else
+    launch_k_colmean_t<IoF16>(k, BH, L, D, chunk_sums, group_sums, (uint16_t*)colmean, st);
 }
 
 }  // namespace sla
@@ -336,7 +415,7 @@ extern "C" int sla_block_map_fwd(const void* q, const void* k, int dtype, int B,
   if (rc) return rc;
   const int M = cdiv(L, BLKQ), N = cdiv(L, BLKK);
   SLA_REQUIRE(topk >= 0 && topk <= N, SLA_ERR_BAD_ARG, "topk=%d outside [0, %d]", topk, N);
-  SLA_REQUIRE(N <= 32768, SLA_ERR_UNSUPPORTED, "more than 32768 key blocks (%d)", N);
+  SLA_REQUIRE(N <= 8192, SLA_ERR_UNSUPPORTED, "more than 8192 key blocks (%d)", N);
   SLA_REQUIRE((int64_t)BH * M < (1ll << 31), SLA_ERR_UNSUPPORTED, "too many query-block rows");
   SLA_REQUIRE(lut_elem_bytes == 4 || lut_elem_bytes == 8, SLA_ERR_BAD_ARG, "lut_elem_bytes must be 4 or 8, got %d",
               lut_elem_bytes);

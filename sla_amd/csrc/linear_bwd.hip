@@ -13,7 +13,8 @@
 //            scalars stay per-lane), writes dq and the row-wise temporaries dn, y (16 bit) and dden
 //   states : streams q, dn, G, y once; dS and dW on the MFMA (operands read transposed from LDS),
 //            dz and db on the vector ALU; fp32 partials
-//   reduce : fixed-order sums of the partials -> dS (16 bit, both orientations), dz, dW, db
+//   reduce : fixed-order sums of the partials -> dS (16 bit, both orientations), dz, per-head dW, db;
+//            a second small kernel adds the heads
 //   kv     : per 32 keys on one wave: dc^T = dS v^T + dz, dv^T = dS^T c^T, dk = phi'(k) dc
 #include "linear_state.h"
 
@@ -351,48 +352,66 @@ __global__ __launch_bounds__(256) void linear_bwd_states_kernel(
 }
 
 // ---- reduce -------------------------------------------------------------------------------
-// grid (cdiv(D*D,256), BH + 1): blocks y < BH reduce one head's dS/dz; block y == BH reduces dW/db
-// over every (head, split) partial in ascending order.
+// Stage 1, grid (cdiv(D*D,256), BH): per head, add the split partials in ascending order:
+//   dS (16 bit, both orientations), dz, and this head's dW^T / db (fp32).
+// Stage 2, grid (cdiv(D*D,256)): add the per-head dW^T / db in ascending head order.
 template <typename Tag>
-__global__ void linear_bwd_reduce_kernel(const float* __restrict__ ds_part, const float* __restrict__ dw_part,
-                                         const float* __restrict__ dz_part, const float* __restrict__ db_part,
-                                         uint16_t* __restrict__ ds, uint16_t* __restrict__ dst, float* __restrict__ dz,
-                                         float* __restrict__ d_weight, float* __restrict__ d_bias, int nsplit, int BH, int D) {
+__global__ __launch_bounds__(256) void linear_bwd_reduce_kernel(const float* __restrict__ ds_part,
+                                                                const float* __restrict__ dw_part,
+                                                                const float* __restrict__ dz_part,
+                                                                const float* __restrict__ db_part, uint16_t* __restrict__ ds,
+                                                                uint16_t* __restrict__ dst, float* __restrict__ dz,
+                                                                float* __restrict__ dw_head, float* __restrict__ db_head,
+                                                                int nsplit, int D) {
   using E = Elem<Tag>;
   const int DD = D * D;
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   const int bh = blockIdx.y;
-  if (bh < BH) {
-    if (i < DD) {
-      const float* p = ds_part + (size_t)bh * nsplit * DD + i;
-      float s = 0.f;
-      for (int sp = 0; sp < nsplit; ++sp) s += p[(size_t)sp * DD];
-      const int d2 = i / D, d1 = i % D;   // partial layout [d2][d1]
-      const uint16_t h = E::from_float(s);
-      dst[(size_t)bh * DD + i] = h;                 // dS^T [d2][d1]
-      ds[(size_t)bh * DD + d1 * D + d2] = h;        // dS   [d1][d2]
+  if (i < DD) {
+    const float* p = ds_part + (size_t)bh * nsplit * DD + i;
+    const float* pw = dw_part + (size_t)bh * nsplit * DD + i;
+    float s = 0.f, sw = 0.f;
+#pragma unroll 4
+    for (int sp = 0; sp < nsplit; ++sp) {
+      s += p[(size_t)sp * DD];
+      sw += pw[(size_t)sp * DD];
     }
-    if (i < D) {
-      const float* p = dz_part + (size_t)bh * nsplit * D + i;
-      float s = 0.f;
-      for (int sp = 0; sp < nsplit; ++sp) s += p[(size_t)sp * D];
-      dz[(size_t)bh * D + i] = s;
+    const int d2 = i / D, d1 = i % D;   // partial layout [d2][d1]
+    const uint16_t h = E::from_float(s);
+    dst[(size_t)bh * DD + i] = h;                 // dS^T [d2][d1]
+    ds[(size_t)bh * DD + d1 * D + d2] = h;        // dS   [d1][d2]
+    dw_head[(size_t)bh * DD + i] = sw;            // dW^T [d][e] of this head
+  }
+  if (i < D) {
+    const float* p = dz_part + (size_t)bh * nsplit * D + i;
+    const float* pb = db_part + (size_t)bh * nsplit * D + i;
+    float s = 0.f, sb = 0.f;
+    for (int sp = 0; sp < nsplit; ++sp) {
+      s += p[(size_t)sp * D];
+      sb += pb[(size_t)sp * D];
     }
-  } else {
-    const int np = BH * nsplit;
-    if (i < DD) {
-      const float* p = dw_part + i;
-      float s = 0.f;
-      for (int sp = 0; sp < np; ++sp) s += p[(size_t)sp * DD];
-      const int d = i / D, e = i % D;      // partial layout [d][e]
-      d_weight[e * D + d] = s;
-    }
-    if (i < D) {
-      const float* p = db_part + i;
-      float s = 0.f;
-      for (int sp = 0; sp < np; ++sp) s += p[(size_t)sp * D];
-      d_bias[i] = s;
-    }
+    dz[(size_t)bh * D + i] = s;
+    db_head[(size_t)bh * D + i] = sb;
+  }
+}
+
+__global__ __launch_bounds__(256) void linear_bwd_reduce_heads_kernel(const float* __restrict__ dw_head,
+                                                                      const float* __restrict__ db_head,
+                                                                      float* __restrict__ d_weight, float* __restrict__ d_bias,
+                                                                      int BH, int D) {
+  const int DD = D * D;
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < DD) {
+    float s = 0.f;
+#pragma unroll 4
+    for (int h = 0; h < BH; ++h) s += dw_head[(size_t)h * DD + i];
+    const int d = i / D, e = i % D;      // layout [d][e]
+    d_weight[e * D + d] = s;
+  }
+  if (i < D) {
+    float s = 0.f;
+    for (int h = 0; h < BH; ++h) s += db_head[(size_t)h * D + i];
+    d_bias[i] = s;
   }
 }
 
@@ -507,7 +526,7 @@ __global__ __launch_bounds__(256) void linear_bwd_kv_kernel(const uint16_t* __re
 // ---- host ---------------------------------------------------------------------------------
 struct LinBwdWs {
   LinWs fwd;
-  size_t dn, y, dden, ds_part, dw_part, dz_part, db_part, ds, dst, dz, total;
+  size_t dn, y, dden, ds_part, dw_part, dz_part, db_part, ds, dst, dz, dw_head, db_head, total;
 };
 static LinBwdWs lin_bwd_ws(int BH, int L, int D) {
   LinBwdWs w;
@@ -524,6 +543,8 @@ static LinBwdWs lin_bwd_ws(int BH, int L, int D) {
   w.ds = off;      off += align_up((int64_t)BH * D * D * 2, 256);
   w.dst = off;     off += align_up((int64_t)BH * D * D * 2, 256);
   w.dz = off;      off += align_up((int64_t)BH * D * 4, 256);
+  w.dw_head = off; off += align_up((int64_t)BH * D * D * 4, 256);
+  w.db_head = off; off += align_up((int64_t)BH * D * 4, 256);
   w.total = off;
   return w;
 }
@@ -547,10 +568,12 @@ static int linear_bwd_impl(const void* q, const void* k, const void* v, const fl
   hipLaunchKernelGGL((linear_bwd_states_kernel<Tag, D>), dim3(w.fwd.nsplit, BH), dim3(256), 0, st, (const uint16_t*)q, dn,
                      (const uint16_t*)d_out, y, dden, (float*)(ws + w.ds_part), (float*)(ws + w.dw_part),
                      (float*)(ws + w.dz_part), (float*)(ws + w.db_part), L, w.fwd.rows_per_split, fmap);
-  hipLaunchKernelGGL((linear_bwd_reduce_kernel<Tag>), dim3(cdiv(D * D, 256), BH + 1), dim3(256), 0, st,
+  hipLaunchKernelGGL((linear_bwd_reduce_kernel<Tag>), dim3(cdiv(D * D, 256), BH), dim3(256), 0, st,
                      (const float*)(ws + w.ds_part), (const float*)(ws + w.dw_part), (const float*)(ws + w.dz_part),
                      (const float*)(ws + w.db_part), (uint16_t*)(ws + w.ds), (uint16_t*)(ws + w.dst), (float*)(ws + w.dz),
-                     d_weight, d_bias, w.fwd.nsplit, BH, D);
+                     (float*)(ws + w.dw_head), (float*)(ws + w.db_head), w.fwd.nsplit, D);
+  hipLaunchKernelGGL(linear_bwd_reduce_heads_kernel, dim3(cdiv(D * D, 256)), dim3(256), 0, st,
+                     (const float*)(ws + w.dw_head), (const float*)(ws + w.db_head), d_weight, d_bias, BH, D);
   hipLaunchKernelGGL((linear_bwd_kv_kernel<Tag, D>), row_grid, dim3(256), 0, st, (const uint16_t*)k, (const uint16_t*)v,
                      (const uint16_t*)(ws + w.ds), (const uint16_t*)(ws + w.dst), (const float*)(ws + w.dz), (uint16_t*)dk,
                      (uint16_t*)dv, L, fmap, tiles);

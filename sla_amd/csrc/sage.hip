@@ -14,7 +14,8 @@
 
 namespace sla {
 
-void launch_k_colmean(const void* k, int dtype, int BH, int L, int D, float* chunk_sums, void* colmean, hipStream_t st);
+int64_t k_colmean_scratch_floats(int BH, int L, int D);
+void launch_k_colmean(const void* k, int dtype, int BH, int L, int D, float* scratch, void* colmean, hipStream_t st);
 
 // ---- INT8 block quantisation ----------------------------------------------------------------
 // One workgroup per (block, bh).  SUB_MEAN: subtract the per-head column mean first.
@@ -326,7 +327,7 @@ static SageWs sage_ws(int BH, int L, int D) {
   w.rows_per_chunk_v = 256;
   w.nchunk_v = cdiv(L, w.rows_per_chunk_v);
   size_t off = 0;
-  w.chunk_sums = off; off += align_up((int64_t)BH * cdiv(L, 64) * D * 4, 256);
+  w.chunk_sums = off; off += align_up(k_colmean_scratch_floats(BH, L, D) * 4, 256);
   w.colmean = off;    off += align_up((int64_t)BH * D * 2, 256);
   w.v_part = off;     off += align_up((int64_t)BH * w.nchunk_v * D * 4, 256);
   w.total = off;

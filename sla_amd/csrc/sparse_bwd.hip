@@ -45,22 +45,55 @@ __global__ __launch_bounds__(256) void bwd_delta_kernel(const uint16_t* __restri
 }
 
 // ---- per-key-block lists ------------------------------------------------------------------
-// One thread per key block n walks the rows of the map; list[bh][n][0..count) holds the
-// selecting query blocks in ascending order.  Capacity Mblk per list (only count entries are
-// ever touched).
+// One wavefront per strip of 64 key blocks.  The map is read 64 rows at a time with coalesced
+// 16-byte loads (the next tile's loads are in flight while this one is scanned) and transposed
+// through LDS; lane c then walks the 64 bytes of its column in order, so list[bh][n][0..count)
+// holds the selecting query blocks in ascending order.  Capacity Mblk per list (only `count`
+// entries are ever touched).
 __global__ __launch_bounds__(64) void bwd_col_lists_kernel(const int8_t* __restrict__ sparse_map, int* __restrict__ list,
-                                                           int* __restrict__ count, int Mblk, int Nblk) {
+                                                           int* __restrict__ count, int Mblk, int Nblk, int vec_ok) {
+  __shared__ __attribute__((aligned(16))) int8_t tile[64][80];
   const int bh = blockIdx.y;
-  const int n = blockIdx.x * 64 + threadIdx.x;
-  if (n >= Nblk) return;
-  const int8_t* col = sparse_map + (size_t)bh * Mblk * Nblk + n;
-  int* out = list + ((size_t)bh * Nblk + n) * Mblk;
+  const int n0 = blockIdx.x * 64;
+  const int lane = threadIdx.x;
+  const int n = n0 + lane;
+  const int8_t* base = sparse_map + (size_t)bh * Mblk * Nblk;
+  int* out = list + ((size_t)bh * Nblk + (n < Nblk ? n : 0)) * Mblk;
+  // lane -> (row lr + 16j, 16-byte chunk lc) of the tile
+  const int lr = lane >> 2, lc = (lane & 3) * 16;
+  i32x4_t pre[4];
+  auto fetch = [&](int m0) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int m = m0 + lr + 16 * j;
+      pre[j] = i32x4_t{0, 0, 0, 0};
+      if (m < Mblk) {
+        if (vec_ok && n0 + lc + 16 <= Nblk) {
+          pre[j] = *reinterpret_cast<const i32x4_t*>(base + (size_t)m * Nblk + n0 + lc);
+        } else {
+          int8_t* b = reinterpret_cast<int8_t*>(&pre[j]);
+          for (int e = 0; e < 16; ++e)
+            if (n0 + lc + e < Nblk) b[e] = base[(size_t)m * Nblk + n0 + lc + e];
+        }
+      }
+    }
+  };
   int c = 0;
-#pragma unroll 8
-  for (int m = 0; m < Mblk; ++m) {
-    if (col[(size_t)m * Nblk] == 1) out[c++] = m;
+  fetch(0);
+  for (int m0 = 0; m0 < Mblk; m0 += 64) {
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < 4; ++j) *reinterpret_cast<i32x4_t*>(&tile[lr + 16 * j][lc]) = pre[j];
+    __syncthreads();
+    if (m0 + 64 < Mblk) fetch(m0 + 64);
+    if (n < Nblk) {
+#pragma unroll 16
+      for (int r = 0; r < 64; ++r) {
+        if (tile[r][lane] == 1) out[c++] = m0 + r;
+      }
+    }
   }
-  count[(size_t)bh * Nblk + n] = c;
+  if (n < Nblk) count[(size_t)bh * Nblk + n] = c;
 }
 
 // ---- dQ ---------------------------------------------------------------------------------
@@ -429,7 +462,10 @@ static int bwd_impl(const void* q, const void* k, const void* v, const void* o, 
   constexpr int RPB = 256 / (D / 8);
   hipLaunchKernelGGL((bwd_delta_kernel<Tag, D>), dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, st,
                      (const uint16_t*)o, (const uint16_t*)d_o, delta, rows);
-  hipLaunchKernelGGL(bwd_col_lists_kernel, dim3(cdiv(Nblk, 64), BH), dim3(64), 0, st, sparse_map, list, count, Mblk, Nblk);
+  // 16-byte loads of map rows need 16-byte aligned rows
+  const int vec_ok = (Nblk % 16 == 0) && ((uintptr_t)sparse_map % 16 == 0);
+  hipLaunchKernelGGL(bwd_col_lists_kernel, dim3(cdiv(Nblk, 64), BH), dim3(64), 0, st, sparse_map, list, count, Mblk, Nblk,
+                     vec_ok);
   const int total_q = BH * Mblk;
   hipLaunchKernelGGL((bwd_dq_kernel<Tag, D, BLKQ>), dim3(xcd_grid(total_q)), dim3(BLKQ * 2), 0, st, (const uint16_t*)q,
                      (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse, delta, lut, lut64, (uint16_t*)dq, L,

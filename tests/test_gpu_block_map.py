@@ -88,3 +88,13 @@ def test_full_size_invariants(dev):
     m1, lut1, _ = get_block_map(q.to(dev), k.to(dev), 0.1, 64, 64)
     m2, lut2, _ = get_block_map(q.to(dev), (k.float() + 8.0).to(k.dtype).to(dev), 0.1, 64, 64)
     assert torch.equal(lut1, lut2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_negative_scores_and_wide_rows(dev, dtype):
+    # all pooled scores negative (threshold key is a negative number) and N beyond 512 / 1280 / 2048
+    g = torch.Generator().manual_seed(77)
+    for L, ratio in ((64 * 70, 0.1), (64 * 600, 0.05), (64 * 1300, 0.02), (64 * 2100, 0.01)):
+        q = (torch.rand(1, 1, L, 32, generator=g) + 0.5).to(dtype)
+        k = -(torch.rand(1, 1, L, 32, generator=g) * torch.linspace(0.5, 2.0, L).view(1, 1, L, 1) + 0.5).to(dtype)
+        _compare(q, k, ratio, 64, 64, dev)

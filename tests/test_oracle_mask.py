@@ -121,12 +121,14 @@ def test_block_map_ignores_constant_key_offset():
 
 def test_block_map_selects_blocks_with_highest_exact_scores():
     # independent float64 restatement on tie-free data: the chosen set is the true top-T
-    q, k = torch.randn(1, 1, 640, 16, dtype=torch.float64), torch.randn(1, 1, 640, 16, dtype=torch.float64)
+    g = torch.Generator().manual_seed(2)
+    q = torch.randn(1, 1, 640, 16, dtype=torch.float64, generator=g)
+    k = torch.randn(1, 1, 640, 16, dtype=torch.float64, generator=g)
     pq = q.view(1, 1, 10, 64, 16).mean(-2)
     pk = (k - k.mean(-2, keepdim=True)).view(1, 1, 10, 64, 16).mean(-2)
     score = pq @ pk.transpose(-1, -2)
     lib = torch.topk(score, 3, dim=-1).indices.sort(-1).values
     gap = (score.sort(-1, descending=True).values[..., 2] - score.sort(-1, descending=True).values[..., 3]).min()
-    assert gap > 1e-4
+    assert gap > 1e-5
     _, lut, _ = O.get_block_map(q.float(), k.float(), 0.3)
     assert torch.equal(lut, lib)
