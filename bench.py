@@ -26,13 +26,31 @@ if ROOT not in sys.path:
 PEAK_BF16_TFLOPS = 2500.0     # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0
 
+# HBM bytes per launch of the dominant kernel, from two `rocprofv3 --pmc` runs of this script
+# (FETCH_SIZE, then WRITE_SIZE; summaries under profiles/), each scaled by what the same counter reads for
+# the 1 GiB-read / 1 GiB-write elementwise kernel of --pmc-calibration (FETCH_SIZE x2.0, WRITE_SIZE x1.0).
+# It is a property of the kernel and the workload, not re-measured by a plain bench run.
+MEASURED_TRAFFIC_BYTES = {
+    "cfg3": {"kernel": "sparse_fwd_kernel", "fetch": 201962.4 * 1024 * 2.0, "write": 100071.1 * 1024 * 1.0},
+}
+
 
 def _events(torch):
     return torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
 
 
-def time_region(torch, fn, steps, warmup):
-    """Average milliseconds per call over exactly `steps` calls, on the current stream."""
+def time_region(torch, fn, steps, warmup, preheat_s=0.15):
+    """Average milliseconds per call over exactly `steps` calls, on the current stream.
+
+    Before the `warmup` untimed calls the same call is repeated for `preheat_s` seconds (untimed as well):
+    the GPU needs that long under load to leave its idle clocks, and a handful of sub-millisecond
+    warm-up calls does not get it there.
+    """
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < preheat_s:
+        for _ in range(10):
+            fn()
+        torch.cuda.synchronize()
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
@@ -68,8 +86,11 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="cfg3")
-    ap.add_argument("--cpu-heads", type=int, default=2, help="heads of the workload timed on the CPU oracle (0 = skip)")
+    ap.add_argument("--cpu-heads", type=int, default=12, help="heads of the workload timed on the CPU oracle (0 = skip)")
     ap.add_argument("--no-extras", action="store_true", help="skip the per-kernel, backward and SageSLA timings")
+    ap.add_argument("--pmc-calibration", action="store_true",
+                    help="also run one plain 1 GiB read + 1 GiB write elementwise kernel, the known-size reference for "
+                         "scaling the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (heads shard with no collective in "
@@ -121,7 +142,10 @@ def main():
                                f"topk{cfg.topk} (T={T} of N={N}) feature_map={cfg.feature_map}, structured q/k",
                    "B": B, "H": H, "L": L, "D": D, "topk": cfg.topk, "T": T},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None, "kernel": "sparse_fwd_kernel",
+                     "frac": achieved / PEAK_BF16_TFLOPS,
+                     "traffic": (sum(v for k_, v in MEASURED_TRAFFIC_BYTES[cfg.name].items() if k_ != "kernel")
+                                 if cfg.name in MEASURED_TRAFFIC_BYTES else None),
+                     "traffic_unit": "HBM bytes per launch (fetch + write)", "kernel": "sparse_fwd_kernel",
                      "flops_per_launch": sparse_flops, "ms_per_launch": ms_sparse},
     }
     extra = {"sla_fwd_ms": ms_fwd, "sparse_fwd_ms": ms_sparse}
@@ -156,6 +180,12 @@ def main():
         except (ImportError, AssertionError, RuntimeError) as e:
             extra["sage_fwd_ms"] = None
             extra["sage_note"] = str(e)[:200]
+    if args.pmc_calibration:
+        x = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+        y = torch.empty_like(x)
+        torch.add(x, 1.0, out=y)          # 1 GiB read + 1 GiB written by one elementwise kernel
+        torch.cuda.synchronize()
+        extra["pmc_calibration"] = "torch.add on 2^28 fp32: 1 GiB read, 1 GiB written"
     out["extra"] = extra
     if args.cpu_heads > 0:
         out["cpu_baseline"] = cpu_baseline(cfg, min(args.cpu_heads, cfg.H), torch)
