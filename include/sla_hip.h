@@ -98,11 +98,12 @@ int sla_linear_fwd(const void* q, const void* k, const void* v, const float* wei
 
 /* Linear branch backward.  d_out is the gradient of `out` above.  Writes dq, dk, dv in `dtype`
  * (gradients of the linear branch only; the residual's gradient is d_out itself) and the
- * fp32 gradients of weight (D,D) and bias (D).
+ * fp32 gradients of weight (D,D) and bias (D).  With accumulate != 0, dq/dk/dv already hold
+ * the gradients of the sparse branch and the linear ones are added to them (in fp32, one rounding).
  * Replaces torch autograd through sparse_linear_attention/core.py:90-99. */
 int sla_linear_bwd(const void* q, const void* k, const void* v, const float* weight, const float* bias,
                    const void* d_out, void* dq, void* dk, void* dv, float* d_weight, float* d_bias,
-                   int dtype, int fmap, int B, int H, int L, int D, void* workspace,
+                   int dtype, int fmap, int B, int H, int L, int D, int accumulate, void* workspace,
                    int64_t workspace_bytes, void* stream);
 
 /* SageSLA: per-block INT8 quantisation of q (BLKQ rows) and of k - mean_L(k) (BLKK rows).

@@ -25,7 +25,7 @@ template <typename Tag, int D>
 __global__ __launch_bounds__(256) void linear_bwd_rows_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ gout, const uint16_t* __restrict__ kvt,
     const uint16_t* __restrict__ z, const float* __restrict__ weight, uint16_t* __restrict__ dq, uint16_t* __restrict__ dn_out,
-    uint16_t* __restrict__ y_out, float* __restrict__ dden_out, int L, int fmap, int tiles_per_wg) {
+    uint16_t* __restrict__ y_out, float* __restrict__ dden_out, int L, int fmap, int tiles_per_wg, int accumulate) {
   using E = Elem<Tag>;
   constexpr int DC = D / 16;
   constexpr int DT = D / 32;
@@ -185,10 +185,17 @@ __global__ __launch_bounds__(256) void linear_bwd_rows_kernel(
       for (int t1 = 0; t1 < DT; ++t1)
 #pragma unroll
         for (int i4 = 0; i4 < 4; ++i4) {
+          uint16_t* dst = dq + roff + 32 * t1 + 8 * i4 + 4 * g;
+          if (accumulate) {
+            const i32x2_t old = *reinterpret_cast<const i32x2_t*>(dst);
+            const uint16_t* op = reinterpret_cast<const uint16_t*>(&old);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) da[t1][4 * i4 + j] += E::to_float(op[j]);
+          }
           i32x2_t w;
           w[0] = (int)E::pack2(da[t1][4 * i4 + 0], da[t1][4 * i4 + 1]);
           w[1] = (int)E::pack2(da[t1][4 * i4 + 2], da[t1][4 * i4 + 3]);
-          *reinterpret_cast<i32x2_t*>(dq + roff + 32 * t1 + 8 * i4 + 4 * g) = w;
+          *reinterpret_cast<i32x2_t*>(dst) = w;
         }
     }
   }
@@ -420,7 +427,8 @@ template <typename Tag, int D>
 __global__ __launch_bounds__(256) void linear_bwd_kv_kernel(const uint16_t* __restrict__ k, const uint16_t* __restrict__ v,
                                                             const uint16_t* __restrict__ ds, const uint16_t* __restrict__ dst,
                                                             const float* __restrict__ dz, uint16_t* __restrict__ dk,
-                                                            uint16_t* __restrict__ dv, int L, int fmap, int tiles_per_wg) {
+                                                            uint16_t* __restrict__ dv, int L, int fmap, int tiles_per_wg,
+                                                            int accumulate) {
   using E = Elem<Tag>;
   constexpr int DC = D / 16;
   constexpr int DT = D / 32;
@@ -501,9 +509,16 @@ __global__ __launch_bounds__(256) void linear_bwd_kv_kernel(const uint16_t* __re
           xk[t][4 * i4 + j] = E::to_float(xp[j]);
         }
         if (ok) {
+          float dvv[4] = {vacc[4 * i4 + 0], vacc[4 * i4 + 1], vacc[4 * i4 + 2], vacc[4 * i4 + 3]};
+          if (accumulate) {
+            const i32x2_t old = *reinterpret_cast<const i32x2_t*>(dv + roff + d0);
+            const uint16_t* op = reinterpret_cast<const uint16_t*>(&old);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) dvv[j] += E::to_float(op[j]);
+          }
           i32x2_t w;
-          w[0] = (int)E::pack2(vacc[4 * i4 + 0], vacc[4 * i4 + 1]);
-          w[1] = (int)E::pack2(vacc[4 * i4 + 2], vacc[4 * i4 + 3]);
+          w[0] = (int)E::pack2(dvv[0], dvv[1]);
+          w[1] = (int)E::pack2(dvv[2], dvv[3]);
           *reinterpret_cast<i32x2_t*>(dv + roff + d0) = w;
         }
       }
@@ -514,10 +529,17 @@ __global__ __launch_bounds__(256) void linear_bwd_kv_kernel(const uint16_t* __re
       for (int t = 0; t < DT; ++t)
 #pragma unroll
         for (int i4 = 0; i4 < 4; ++i4) {
+          uint16_t* dst = dk + roff + 32 * t + 8 * i4 + 4 * g;
+          if (accumulate) {
+            const i32x2_t old = *reinterpret_cast<const i32x2_t*>(dst);
+            const uint16_t* op = reinterpret_cast<const uint16_t*>(&old);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) dc[t][4 * i4 + j] += E::to_float(op[j]);
+          }
           i32x2_t w;
           w[0] = (int)E::pack2(dc[t][4 * i4 + 0], dc[t][4 * i4 + 1]);
           w[1] = (int)E::pack2(dc[t][4 * i4 + 2], dc[t][4 * i4 + 3]);
-          *reinterpret_cast<i32x2_t*>(dk + roff + 32 * t + 8 * i4 + 4 * g) = w;
+          *reinterpret_cast<i32x2_t*>(dst) = w;
         }
     }
   }
@@ -552,8 +574,8 @@ int64_t linear_bwd_workspace_bytes(int BH, int L, int D) { return (int64_t)lin_b
 
 template <typename Tag, int D>
 static int linear_bwd_impl(const void* q, const void* k, const void* v, const float* weight, const void* d_out, void* dq,
-                           void* dk, void* dv, float* d_weight, float* d_bias, int fmap, int BH, int L, char* ws,
-                           hipStream_t st) {
+                           void* dk, void* dv, float* d_weight, float* d_bias, int fmap, int BH, int L, int accumulate,
+                           char* ws, hipStream_t st) {
   const LinBwdWs w = lin_bwd_ws(BH, L, D);
   launch_state_build<Tag, D>(k, v, fmap, BH, L, ws, w.fwd, st);
   uint16_t* kvt = (uint16_t*)(ws + w.fwd.kvt);
@@ -564,7 +586,7 @@ static int linear_bwd_impl(const void* q, const void* k, const void* v, const fl
   const int tiles = 4;
   const dim3 row_grid(cdiv(L, 128 * tiles), BH);
   hipLaunchKernelGGL((linear_bwd_rows_kernel<Tag, D>), row_grid, dim3(256), 0, st, (const uint16_t*)q,
-                     (const uint16_t*)d_out, kvt, z, weight, (uint16_t*)dq, dn, y, dden, L, fmap, tiles);
+                     (const uint16_t*)d_out, kvt, z, weight, (uint16_t*)dq, dn, y, dden, L, fmap, tiles, accumulate);
   hipLaunchKernelGGL((linear_bwd_states_kernel<Tag, D>), dim3(w.fwd.nsplit, BH), dim3(256), 0, st, (const uint16_t*)q, dn,
                      (const uint16_t*)d_out, y, dden, (float*)(ws + w.ds_part), (float*)(ws + w.dw_part),
                      (float*)(ws + w.dz_part), (float*)(ws + w.db_part), L, w.fwd.rows_per_split, fmap);
@@ -576,7 +598,7 @@ static int linear_bwd_impl(const void* q, const void* k, const void* v, const fl
                      (const float*)(ws + w.dw_head), (const float*)(ws + w.db_head), d_weight, d_bias, BH, D);
   hipLaunchKernelGGL((linear_bwd_kv_kernel<Tag, D>), row_grid, dim3(256), 0, st, (const uint16_t*)k, (const uint16_t*)v,
                      (const uint16_t*)(ws + w.ds), (const uint16_t*)(ws + w.dst), (const float*)(ws + w.dz), (uint16_t*)dk,
-                     (uint16_t*)dv, L, fmap, tiles);
+                     (uint16_t*)dv, L, fmap, tiles, accumulate);
   return check_launch("linear_bwd");
 }
 
@@ -586,7 +608,8 @@ using namespace sla;
 
 extern "C" int sla_linear_bwd(const void* q, const void* k, const void* v, const float* weight, const float* bias,
                               const void* d_out, void* dq, void* dk, void* dv, float* d_weight, float* d_bias, int dtype,
-                              int fmap, int B, int H, int L, int D, void* workspace, int64_t workspace_bytes, void* stream) {
+                              int fmap, int B, int H, int L, int D, int accumulate, void* workspace,
+                              int64_t workspace_bytes, void* stream) {
   int rc = validate_linear(dtype, fmap, B, H, L, D);
   if (rc) return rc;
   (void)bias;  // the bias does not enter any gradient
@@ -602,7 +625,7 @@ extern "C" int sla_linear_bwd(const void* q, const void* k, const void* v, const
   hipStream_t st = (hipStream_t)stream;
   char* ws = (char*)workspace;
 #define SLA_LINB_CASE(TAG, DD) \
-  return linear_bwd_impl<TAG, DD>(q, k, v, weight, d_out, dq, dk, dv, d_weight, d_bias, fmap, BH, L, ws, st)
+  return linear_bwd_impl<TAG, DD>(q, k, v, weight, d_out, dq, dk, dv, d_weight, d_bias, fmap, BH, L, accumulate, ws, st)
   if (dtype == SLA_BF16) {
     if (D == 128) SLA_LINB_CASE(bf16_tag, 128);
     SLA_LINB_CASE(bf16_tag, 64);

@@ -24,16 +24,22 @@ def linear_fwd(q, k, v, weight, bias, residual, fmap: str):
     return out
 
 
-def linear_bwd(q, k, v, weight, bias, d_out, fmap: str):
+def linear_bwd(q, k, v, weight, bias, d_out, fmap: str, accumulate_into=None):
+    """Gradients of the linear branch.  ``accumulate_into=(dq, dk, dv)`` adds them to existing
+    gradient tensors (those of the sparse branch) instead of allocating new ones."""
     B, H, L, D = q.shape
     dt = _lib.dtype_code(q.dtype)
     ws = _lib.workspace(_lib.WS_LINEAR_BWD, dt, B, H, L, D, 64, 64, 0, q.device)
-    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    if accumulate_into is None:
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    else:
+        dq, dk, dv = accumulate_into
     dw = torch.empty((D, D), dtype=torch.float32, device=q.device)
     db = torch.empty((D,), dtype=torch.float32, device=q.device)
     rc = _lib.load().sla_linear_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), weight.data_ptr(), bias.data_ptr(),
                                     d_out.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), dw.data_ptr(),
-                                    db.data_ptr(), dt, _lib.FMAP[fmap], B, H, L, D, ws.data_ptr(), ws.numel(),
+                                    db.data_ptr(), dt, _lib.FMAP[fmap], B, H, L, D,
+                                    0 if accumulate_into is None else 1, ws.data_ptr(), ws.numel(),
                                     _lib.stream_ptr(q.device))
     _lib.check(rc)
     return dq, dk, dv, dw, db

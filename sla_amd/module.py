@@ -6,10 +6,42 @@ import torch
 import torch.nn as nn
 
 from .block_map import get_block_map
-from .linear import _linear_proj_add
-from .sparse_attn import _attention
+from .linear import linear_bwd, linear_fwd
+from .sparse_attn import sparse_attn_bwd, sparse_attn_fwd
 
 FEATURE_MAPS = ("elu", "relu", "softmax")
+
+
+class _sla_core(torch.autograd.Function):
+    """Sparse branch + linear branch + projection + sum as one differentiable operator.
+
+    Same function as ``_attention`` followed by ``_linear_proj_add`` (reference core.py:88-100); fusing
+    them lets the backward add the linear-branch gradients into the sparse-branch ones in place.
+    """
+
+    @staticmethod
+    def forward(ctx, q, k, v, weight, bias, sparse_map, lut, topk, BLKQ, BLKK, fmap):
+        assert q.is_contiguous() and k.is_contiguous() and v.is_contiguous()
+        assert sparse_map.is_contiguous() and lut.is_contiguous()
+        assert BLKQ == 64 or BLKQ == 128
+        assert BLKK == 64
+        qk_scale = q.shape[-1] ** -0.5
+        weight = weight.contiguous()
+        bias = bias.contiguous()
+        o_s, lse = sparse_attn_fwd(q, k, v, lut, topk, BLKQ, BLKK, qk_scale)
+        out = linear_fwd(q, k, v, weight, bias, o_s, fmap)
+        ctx.save_for_backward(q, k, v, weight, bias, sparse_map, lut, lse, o_s)
+        ctx.cfg = (topk, BLKQ, BLKK, fmap, qk_scale)
+        return out
+
+    @staticmethod
+    def backward(ctx, d_out):
+        q, k, v, weight, bias, sparse_map, lut, lse, o_s = ctx.saved_tensors
+        topk, BLKQ, BLKK, fmap, qk_scale = ctx.cfg
+        d_out = d_out.contiguous()
+        dq, dk, dv = sparse_attn_bwd(q, k, v, o_s, d_out, lse, sparse_map, lut, topk, BLKQ, BLKK, qk_scale)
+        _, _, _, dw, db = linear_bwd(q, k, v, weight, bias, d_out, fmap, accumulate_into=(dq, dk, dv))
+        return dq, dk, dv, dw, db, None, None, None, None, None, None
 
 
 class SparseLinearAttention(nn.Module):
@@ -60,8 +92,8 @@ class SparseLinearAttention(nn.Module):
         q = q.to(self.dtype)
         k = k.to(self.dtype)
         v = v.to(self.dtype)
-        o_s = _attention.apply(q, k, v, sparse_map, lut, real_topk, self.BLKQ, self.BLKK)
-        o = _linear_proj_add.apply(q, k, v, self.proj_l.weight, self.proj_l.bias, o_s, self.feature_map)
+        o = _sla_core.apply(q, k, v, self.proj_l.weight, self.proj_l.bias, sparse_map, lut, real_topk, self.BLKQ,
+                            self.BLKK, self.feature_map)
         o = o.to(dtype)
 
         if return_sparsity:
