@@ -99,7 +99,8 @@ int sla_linear_fwd(const void* q, const void* k, const void* v, const float* wei
 /* Linear branch backward.  d_out is the gradient of `out` above.  Writes dq, dk, dv in `dtype`
  * (gradients of the linear branch only; the residual's gradient is d_out itself) and the
  * fp32 gradients of weight (D,D) and bias (D).  With accumulate != 0, dq/dk/dv already hold
- * the gradients of the sparse branch and the linear ones are added to them (in fp32, one rounding).
+ * the gradients of the sparse branch and the linear ones, rounded to `dtype`, are added to them
+ * as a tensor addition in `dtype` would (the sum is formed in fp32 and rounded once more).
  * Replaces torch autograd through sparse_linear_attention/core.py:90-99. */
 int sla_linear_bwd(const void* q, const void* k, const void* v, const float* weight, const float* bias,
                    const void* d_out, void* dq, void* dk, void* dv, float* d_weight, float* d_bias,

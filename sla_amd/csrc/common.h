@@ -111,6 +111,113 @@ static __device__ __forceinline__ i16x8_t buf_load_b128(__amdgpu_buffer_rsrc_t r
   return __builtin_bit_cast(i16x8_t, __builtin_amdgcn_raw_buffer_load_b128(r, (int)byte_off, 0, 0));
 }
 
+// Orders this wave's LDS writes before its later LDS reads when lanes exchange data through a
+// wave-private region: the hardware keeps one wave's LDS operations in order, this keeps the compiler
+// from moving them across the hand-over.  Emits no instruction.
+static __device__ __forceinline__ void wave_lds_fence() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// ---- row-contiguous output of a tile held in MFMA accumulator layout ---------------------------
+// In the transposed formulations a lane owns one row (query / key) of a 32-row tile and, per 32-column
+// tile dt and register group i4, the 4 adjacent columns 32dt + 8i4 + 4g.. of that row.  Storing those
+// 8-byte pieces directly makes every lane of a wave touch a different 256-byte row.  Instead the wave
+// parks the tile in a private LDS staging area and moves it with 16-byte accesses in which D/8 adjacent
+// lanes cover one whole row; inputs take the same route in reverse.
+// `stage` holds 32 rows of (D + 8) elements and is private to the calling wave (the LDS queue of a wave
+// is in order, so no workgroup barrier is needed).
+// Row-contiguous tile traffic: 32 rows of D 16-bit elements move as 16-byte pieces, D/8 adjacent lanes
+// per row, D/16 pieces per lane.  Piece i of a lane is (row, col) = ((lane + 64 i) / (D/8), 8 ((lane + 64 i) % (D/8))).
+template <int D>
+struct TileRows {
+  static constexpr int CPR = D / 8, N = 32 * CPR / 64, SSTR = D + 8;
+  i16x8_t x[N];
+
+  // global -> registers; rows at or past rows_valid read as zero
+  __device__ __forceinline__ void fetch(const uint16_t* gtile, int rows_valid, int lane) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const int idx = lane + 64 * i, row = idx / CPR, col = (idx % CPR) * 8;
+      x[i] = i16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+      if (row < rows_valid) x[i] = *reinterpret_cast<const i16x8_t*>(gtile + (size_t)row * D + col);
+    }
+  }
+  // registers -> the wave's staging tile
+  __device__ __forceinline__ void park(uint16_t* stage, int lane) const {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const int idx = lane + 64 * i, row = idx / CPR, col = (idx % CPR) * 8;
+      *reinterpret_cast<i16x8_t*>(&stage[row * SSTR + col]) = x[i];
+    }
+    wave_lds_fence();
+  }
+  // staging tile -> registers
+  __device__ __forceinline__ void unpark(const uint16_t* stage, int lane) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const int idx = lane + 64 * i, row = idx / CPR, col = (idx % CPR) * 8;
+      x[i] = *reinterpret_cast<const i16x8_t*>(&stage[row * SSTR + col]);
+    }
+  }
+  // registers -> global
+  __device__ __forceinline__ void store(uint16_t* gtile, int rows_valid, int lane) const {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const int idx = lane + 64 * i, row = idx / CPR, col = (idx % CPR) * 8;
+      if (row < rows_valid) *reinterpret_cast<i16x8_t*>(gtile + (size_t)row * D + col) = x[i];
+    }
+  }
+  // this += other, element-wise in fp32 with one rounding
+  template <typename E>
+  __device__ __forceinline__ void add(const TileRows& o) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      i32x4_t w;
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        w[j] = (int)E::pack2(E::to_float((uint16_t)x[i][2 * j]) + E::to_float((uint16_t)o.x[i][2 * j]),
+                             E::to_float((uint16_t)x[i][2 * j + 1]) + E::to_float((uint16_t)o.x[i][2 * j + 1]));
+      x[i] = __builtin_bit_cast(i16x8_t, w);
+    }
+  }
+};
+
+// Writes a tile held in accumulator register order (val[dt][16], lane = row) into the staging tile.
+template <typename E, int D>
+static __device__ __forceinline__ void park_acc_tile(uint16_t* stage, const float (&val)[D / 32][16], int lane) {
+  constexpr int SSTR = D + 8;
+  const int g = lane >> 5, r = lane & 31;
+#pragma unroll
+  for (int dt = 0; dt < D / 32; ++dt)
+#pragma unroll
+    for (int i4 = 0; i4 < 4; ++i4) {
+      i32x2_t w;
+      w[0] = (int)E::pack2(val[dt][4 * i4 + 0], val[dt][4 * i4 + 1]);
+      w[1] = (int)E::pack2(val[dt][4 * i4 + 2], val[dt][4 * i4 + 3]);
+      *reinterpret_cast<i32x2_t*>(&stage[r * SSTR + 32 * dt + 8 * i4 + 4 * g]) = w;
+    }
+  wave_lds_fence();
+}
+
+// Accumulator-order tile -> global rows.  An addend is added after the value has been rounded to
+// 16 bit, as a separate 16-bit tensor addition would: `addend` is a tile fetched earlier; with
+// ADD_DEST the addend is what the destination rows hold (read here, while the tile sits in LDS).
+template <typename E, int D, bool ADD_DEST = false>
+static __device__ __forceinline__ void store_acc_tile(uint16_t* stage, const float (&val)[D / 32][16], uint16_t* gtile,
+                                                       const TileRows<D>* addend, int rows_valid, int lane) {
+  TileRows<D> old;
+  if (ADD_DEST) old.fetch(gtile, rows_valid, lane);
+  park_acc_tile<E, D>(stage, val, lane);
+  TileRows<D> t;
+  t.unpark(stage, lane);
+  if (ADD_DEST) t.template add<E>(old);
+  else if (addend) t.template add<E>(*addend);
+  t.store(gtile, rows_valid, lane);
+  wave_lds_fence();   // the staging area may be rewritten right after
+}
+
 static __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 static __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 

@@ -6,33 +6,53 @@
 //   o_l = (fq kvsum) / (1e-5 + sum_d fq*ksum)        (16-bit results)
 //   out = o_s + (o_l W^T + b)                        (W, b cast to 16 bit as autocast does)
 //
-// Three kernels:
+// Kernels:
 //   state_partial : streams K and V once; each workgroup owns a slice of L and forms its
 //                   share of phi(K)^T V on the MFMA (both operands read transposed from LDS)
 //                   and of sum phi(K) on the vector ALU; fp32 partials to the workspace.
 //   state_reduce  : adds the partials in ascending slice order, rounds to 16 bit, stores the
 //                   state TRANSPOSED (KVT[d2][d1]) so the next kernel reads MFMA rows directly.
-//   out           : one wavefront per 32 queries.  Both products are formed transposed
-//                   (N^T = KVT phi(Q)^T, then OUT^T = W Y^T) so the per-query divisor is a
-//                   per-lane scalar and Y^T leaves the first accumulator already in the
-//                   B-operand layout of the second product.
+//   fold          : KVW = KV W^T per head (16 bit), so numerator and projection are one product.
+//   out           : one wavefront per 32 queries.  OUT^T = KVW^T phi(Q)^T is formed transposed so the
+//                   per-query divisor is a per-lane scalar; the tile is scaled, biased, parked in LDS
+//                   and written (plus the residual) with whole-row 16-byte accesses.
 #include "linear_state.h"
 
 namespace sla {
 
-// ---- kernel 3: output --------------------------------------------------------------------
+// ---- kernel 3: fold the projection into the state -------------------------------------------------
+// kvwt[bh][e][d1] = round16( sum_d2 round16(W[e][d2]) * KVT[d2][d1] ), fp32 accumulation in ascending d2.
+// (phi(Q) KV / den) W^T = (phi(Q) (KV W^T)) / den, so the output kernel needs one product per query tile.
+// grid (D*D/256, BH): thread (e, d1); the 256 threads of a workgroup share at most two rows e.
+template <typename Tag>
+__global__ __launch_bounds__(256) void linear_fold_kernel(const uint16_t* __restrict__ kvt, const float* __restrict__ weight,
+                                                          uint16_t* __restrict__ kvwt, int D) {
+  using E = Elem<Tag>;
+  const int bh = blockIdx.y;
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= D * D) return;
+  const int e = i / D, d1 = i % D;
+  const uint16_t* s = kvt + (size_t)bh * D * D + d1;
+  const float* w = weight + (size_t)e * D;
+  float acc = 0.f;
+#pragma unroll 8
+  for (int d2 = 0; d2 < D; ++d2) acc += round16<Tag>(w[d2]) * E::to_float(s[(size_t)d2 * D]);
+  kvwt[(size_t)bh * D * D + i] = E::from_float(acc);
+}
+
+// ---- kernel 4: output --------------------------------------------------------------------
 // grid (ceil(L / (128*TILES)), BH), 256 threads = 4 waves x 32 queries, TILES steps per workgroup.
 template <typename Tag, int D>
-__global__ __launch_bounds__(256) void linear_out_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ kvt,
-                                                         const uint16_t* __restrict__ z, const float* __restrict__ weight,
-                                                         const float* __restrict__ bias, const uint16_t* __restrict__ residual,
-                                                         uint16_t* __restrict__ out, int L, int fmap, int tiles_per_wg) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void linear_out_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ kvwt,
+                                                         const uint16_t* __restrict__ z, const float* __restrict__ bias,
+                                                         const uint16_t* __restrict__ residual, uint16_t* __restrict__ out,
+                                                         int L, int fmap, int tiles_per_wg) {
   using E = Elem<Tag>;
   constexpr int DC = D / 16;
   constexpr int DT = D / 32;
   constexpr int STR = D + 8;
-  __shared__ __attribute__((aligned(16))) uint16_t sKVT[D * STR];   // [d2][d1]
-  __shared__ __attribute__((aligned(16))) uint16_t sW[D * STR];     // [e][slot-permuted d2]
+  __shared__ __attribute__((aligned(16))) uint16_t sKVW[D * STR];       // [e][d1]
+  __shared__ __attribute__((aligned(16))) uint16_t sStage[4][32 * STR];  // per-wave output staging
   __shared__ float sBias[D];
   __shared__ float sZ[D];
 
@@ -40,26 +60,12 @@ __global__ __launch_bounds__(256) void linear_out_kernel(const uint16_t* __restr
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int g = lane >> 5, r = lane & 31;
 
-  // stage the state and the projection once per workgroup
+  // stage the folded state once per workgroup
   {
-    const uint16_t* src = kvt + (size_t)bh * D * D;
+    const uint16_t* src = kvwt + (size_t)bh * D * D;
     for (int idx = tid; idx < D * D / 8; idx += 256) {
       const int row = idx / (D / 8), col = (idx % (D / 8)) * 8;
-      *reinterpret_cast<i16x8_t*>(&sKVT[row * STR + col]) = *reinterpret_cast<const i16x8_t*>(src + (size_t)row * D + col);
-    }
-    // W[e][.] re-ordered so that the 8 contraction slots of lane group gg in chunk c are adjacent:
-    // slot j <-> d2 = 16c + 8*(j/4) + 4gg + j%4  (the accumulator layout of the first product)
-    for (int idx = tid; idx < D * DC * 2; idx += 256) {
-      const int e = idx / (DC * 2), c = (idx / 2) % DC, gg = idx & 1;
-      const float* w0 = weight + (size_t)e * D + 16 * c + 4 * gg;
-      const f32x4_t lo = *reinterpret_cast<const f32x4_t*>(w0);
-      const f32x4_t hi = *reinterpret_cast<const f32x4_t*>(w0 + 8);
-      i32x4_t pw;
-      pw[0] = (int)E::pack2(lo[0], lo[1]);
-      pw[1] = (int)E::pack2(lo[2], lo[3]);
-      pw[2] = (int)E::pack2(hi[0], hi[1]);
-      pw[3] = (int)E::pack2(hi[2], hi[3]);
-      *reinterpret_cast<i32x4_t*>(&sW[e * STR + 16 * c + 8 * gg]) = pw;
+      *reinterpret_cast<i16x8_t*>(&sKVW[row * STR + col]) = *reinterpret_cast<const i16x8_t*>(src + (size_t)row * D + col);
     }
     if (tid < D) {
       sBias[tid] = round16<Tag>(bias[tid]);
@@ -69,21 +75,29 @@ __global__ __launch_bounds__(256) void linear_out_kernel(const uint16_t* __restr
   __syncthreads();
 
   const uint16_t* qh = q + (size_t)bh * L * D;
+  uint16_t* stage = sStage[wave];
+  const int first_row = blockIdx.x * tiles_per_wg * 128 + wave * 32;
+  TileRows<D> qt;                      // q rows of the tile about to be processed, fetched one tile ahead
+  if (first_row < L) qt.fetch(qh + (size_t)first_row * D, min(32, L - first_row), lane);
   for (int tt = 0; tt < tiles_per_wg; ++tt) {
-    const int row0 = (blockIdx.x * tiles_per_wg + tt) * 128 + wave * 32;
+    const int row0 = first_row + tt * 128;
     if (row0 >= L) break;
-    const int qrow = row0 + r;
-    const bool ok = qrow < L;
+    const int rows_valid = min(32, L - row0);
+    const size_t off = ((size_t)bh * L + row0) * D;
 
     // phi(q): this lane holds d = 16c + 8g + j of its row; lane^32 holds the other half
+    qt.park(stage, lane);
     float f[DC][8];
 #pragma unroll
     for (int c = 0; c < DC; ++c) {
-      i16x8_t x = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (ok) x = *reinterpret_cast<const i16x8_t*>(qh + (size_t)qrow * D + 16 * c + 8 * g);
+      const i16x8_t x = *reinterpret_cast<const i16x8_t*>(&stage[r * STR + 16 * c + 8 * g]);
 #pragma unroll
       for (int j = 0; j < 8; ++j) f[c][j] = E::to_float((uint16_t)x[j]);
     }
+    wave_lds_fence();
+    TileRows<D> res;
+    if (residual) res.fetch(residual + off, rows_valid, lane);
+    if (tt + 1 < tiles_per_wg && row0 + 128 < L) qt.fetch(qh + (size_t)(row0 + 128) * D, min(32, L - row0 - 128), lane);
     float row_mx, row_inv;
     phi_row_pair<Tag, DC>(fmap, f, row_mx, row_inv);
     // divisor: 1e-5 + sum_d round16(fq*z), each step rounded to 16 bit as the reference's tensors are
@@ -102,69 +116,22 @@ __global__ __launch_bounds__(256) void linear_out_kernel(const uint16_t* __restr
     den = round16<Tag>(1e-5f + round16<Tag>(den));
     const float inv_den = 1.0f / den;
 
-    // N^T = KVT phi(Q)^T : DT tiles of 32 d2-rows x 32 queries
-    f32x16_t nacc[DT];
+    // OUT^T = KVW^T-rows x phi(Q)^T : DT tiles of 32 output channels x 32 queries
+    float val[DT][16];
 #pragma unroll
     for (int t = 0; t < DT; ++t) {
+      f32x16_t acc;
 #pragma unroll
-      for (int i = 0; i < 16; ++i) nacc[t][i] = 0.f;
+      for (int i = 0; i < 16; ++i) acc[i] = 0.f;
 #pragma unroll
       for (int c = 0; c < DC; ++c) {
-        const i16x8_t a = *reinterpret_cast<const i16x8_t*>(&sKVT[(32 * t + r) * STR + 16 * c + 8 * g]);
-        nacc[t] = E::mfma32(a, qf[c], nacc[t]);
+        const i16x8_t a = *reinterpret_cast<const i16x8_t*>(&sKVW[(32 * t + r) * STR + 16 * c + 8 * g]);
+        acc = E::mfma32(a, qf[c], acc);
       }
+#pragma unroll
+      for (int i = 0; i < 16; ++i) val[t][i] = acc[i] * inv_den + sBias[32 * t + 8 * (i >> 2) + 4 * g + (i & 3)];
     }
-    // Y^T = round16(round16(N^T) / den), packed straight into B-operand fragments
-    i16x8_t yf[DT][2];
-#pragma unroll
-    for (int t = 0; t < DT; ++t)
-#pragma unroll
-      for (int c2 = 0; c2 < 2; ++c2) {
-        i32x4_t pw;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const float a = round16<Tag>(nacc[t][8 * c2 + 2 * j]) * inv_den;
-          const float b = round16<Tag>(nacc[t][8 * c2 + 2 * j + 1]) * inv_den;
-          pw[j] = (int)E::pack2(a, b);
-        }
-        yf[t][c2] = __builtin_bit_cast(i16x8_t, pw);
-      }
-    // OUT^T = W Y^T : contraction chunk (t, c2) covers d2 = 32t + 16c2 .. +15
-    f32x16_t oacc[DT];
-#pragma unroll
-    for (int et = 0; et < DT; ++et) {
-#pragma unroll
-      for (int i = 0; i < 16; ++i) oacc[et][i] = 0.f;
-#pragma unroll
-      for (int t = 0; t < DT; ++t)
-#pragma unroll
-        for (int c2 = 0; c2 < 2; ++c2) {
-          const i16x8_t a = *reinterpret_cast<const i16x8_t*>(&sW[(32 * et + r) * STR + 16 * (2 * t + c2) + 8 * g]);
-          oacc[et] = E::mfma32(a, yf[t][c2], oacc[et]);
-        }
-    }
-    if (ok) {
-      const size_t off = ((size_t)bh * L + qrow) * D;
-#pragma unroll
-      for (int et = 0; et < DT; ++et)
-#pragma unroll
-        for (int i4 = 0; i4 < 4; ++i4) {
-          const int e0 = 32 * et + 8 * i4 + 4 * g;
-          float y[4];
-#pragma unroll
-          for (int j = 0; j < 4; ++j) y[j] = round16<Tag>(oacc[et][4 * i4 + j] + sBias[e0 + j]);
-          if (residual) {
-            const i32x2_t rv = *reinterpret_cast<const i32x2_t*>(residual + off + e0);
-            const uint16_t* rp = reinterpret_cast<const uint16_t*>(&rv);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) y[j] += E::to_float(rp[j]);
-          }
-          i32x2_t w;
-          w[0] = (int)E::pack2(y[0], y[1]);
-          w[1] = (int)E::pack2(y[2], y[3]);
-          *reinterpret_cast<i32x2_t*>(out + off + e0) = w;
-        }
-    }
+    store_acc_tile<E, D>(stage, val, out + off, residual ? &res : nullptr, rows_valid, lane);
   }
 }
 
@@ -176,11 +143,13 @@ static int linear_fwd_impl(const void* q, const void* k, const void* v, const fl
                            const void* residual, void* out, int fmap, int BH, int L, char* ws, hipStream_t st) {
   const LinWs w = lin_ws(BH, L, D);
   uint16_t* kvt = (uint16_t*)(ws + w.kvt);
+  uint16_t* kvwt = (uint16_t*)(ws + w.kvwt);
   uint16_t* z = (uint16_t*)(ws + w.z);
-  launch_state_build<Tag, D>(k, v, fmap, BH, L, ws, w, st);
-  const int tiles = 4;
-  hipLaunchKernelGGL((linear_out_kernel<Tag, D>), dim3(cdiv(L, 128 * tiles), BH), dim3(256), 0, st, (const uint16_t*)q, kvt,
-                     z, weight, bias, (const uint16_t*)residual, (uint16_t*)out, L, fmap, tiles);
+  launch_state_build<Tag, D>(k, v, weight, fmap, BH, L, ws, w, st);
+  hipLaunchKernelGGL((linear_fold_kernel<Tag>), dim3(cdiv(D * D, 256), BH), dim3(256), 0, st, kvt, weight, kvwt, D);
+  const int tiles = balanced_tiles(cdiv(L, 128), BH, 2);
+  hipLaunchKernelGGL((linear_out_kernel<Tag, D>), dim3(cdiv(L, 128 * tiles), BH), dim3(256), 0, st, (const uint16_t*)q, kvwt,
+                     z, bias, (const uint16_t*)residual, (uint16_t*)out, L, fmap, tiles);
   return check_launch("linear_fwd");
 }
 

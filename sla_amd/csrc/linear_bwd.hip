@@ -21,10 +21,14 @@
 namespace sla {
 
 // ---- rows ---------------------------------------------------------------------------------
-template <typename Tag, int D>
-__global__ __launch_bounds__(256) void linear_bwd_rows_kernel(
+// grid (ceil(L / (32*NW*tiles)), BH), NW waves of 32 queries each.  Inputs and outputs move through a
+// wave-private LDS staging tile so that global traffic is whole 256-byte rows; the next tile's q and G
+// rows are fetched into registers while the current tile is computed.
+template <typename Tag, int D, int NW>
+__global__ __launch_bounds__(64 * NW) void linear_bwd_rows_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ gout, const uint16_t* __restrict__ kvt,
-    const uint16_t* __restrict__ z, const float* __restrict__ weight, uint16_t* __restrict__ dq, uint16_t* __restrict__ dn_out,
+    const uint16_t* __restrict__ kvp, const uint16_t* __restrict__ z, const uint16_t* __restrict__ wt,
+    uint16_t* __restrict__ dq, uint16_t* __restrict__ dn_out,
     uint16_t* __restrict__ y_out, float* __restrict__ dden_out, int L, int fmap, int tiles_per_wg, int accumulate) {
   using E = Elem<Tag>;
   constexpr int DC = D / 16;
@@ -33,6 +37,7 @@ __global__ __launch_bounds__(256) void linear_bwd_rows_kernel(
   __shared__ __attribute__((aligned(16))) uint16_t sKVT[D * STR];  // [d2][d1]          A of n^T = KVT a^T
   __shared__ __attribute__((aligned(16))) uint16_t sKVP[D * STR];  // [d1][perm d2]     A of da^T = S dn^T
   __shared__ __attribute__((aligned(16))) uint16_t sWT[D * STR];   // [d][e]            A of dy^T = W^T G^T
+  __shared__ __attribute__((aligned(16))) uint16_t sStage[NW][32 * STR];
   __shared__ __attribute__((aligned(16))) float sZ[D];
 
   const int bh = blockIdx.y;
@@ -40,48 +45,64 @@ __global__ __launch_bounds__(256) void linear_bwd_rows_kernel(
   const int g = lane >> 5, r = lane & 31;
 
   {
+    // all three operand matrices arrive in 16 bit and in the layout their MFMA reads want
     const uint16_t* src = kvt + (size_t)bh * D * D;
-    for (int idx = tid; idx < D * D / 8; idx += 256) {
+    const uint16_t* srcp = kvp + (size_t)bh * D * D;
+    for (int idx = tid; idx < D * D / 8; idx += 64 * NW) {
       const int row = idx / (D / 8), col = (idx % (D / 8)) * 8;
       *reinterpret_cast<i16x8_t*>(&sKVT[row * STR + col]) = *reinterpret_cast<const i16x8_t*>(src + (size_t)row * D + col);
-    }
-    // S[d1][d2] = KVT[d2][d1], columns re-ordered to the accumulator slot order:
-    // slot j of chunk c, lane group gg  <->  d2 = 16c + 8*(j/4) + 4gg + j%4
-    for (int idx = tid; idx < D * D; idx += 256) {
-      const int d2 = idx / D, d1 = idx % D;
-      const int c = d2 >> 4, w16 = d2 & 15;
-      const int gg = (w16 >> 2) & 1, j = ((w16 >> 3) << 2) | (w16 & 3);
-      sKVP[d1 * STR + 16 * c + 8 * gg + j] = src[idx];
-    }
-    for (int idx = tid; idx < D * D; idx += 256) {
-      const int e = idx / D, d = idx % D;
-      sWT[d * STR + e] = E::from_float(weight[idx]);
+      *reinterpret_cast<i16x8_t*>(&sKVP[row * STR + col]) = *reinterpret_cast<const i16x8_t*>(srcp + (size_t)row * D + col);
+      *reinterpret_cast<i16x8_t*>(&sWT[row * STR + col]) = *reinterpret_cast<const i16x8_t*>(wt + (size_t)row * D + col);
     }
     if (tid < D) sZ[tid] = E::to_float(z[(size_t)bh * D + tid]);
   }
   __syncthreads();
 
   const size_t head_off = (size_t)bh * L * D;
+  uint16_t* stage = sStage[wave];
+  constexpr int STEP = 32 * NW;
+  const int first_row = blockIdx.x * tiles_per_wg * STEP + wave * 32;
+  TileRows<D> qt, gt;                  // q and G rows of the tile about to be processed
+  if (first_row < L) {
+    qt.fetch(q + head_off + (size_t)first_row * D, min(32, L - first_row), lane);
+    gt.fetch(gout + head_off + (size_t)first_row * D, min(32, L - first_row), lane);
+  }
   for (int tt = 0; tt < tiles_per_wg; ++tt) {
-    const int row0 = (blockIdx.x * tiles_per_wg + tt) * 128 + wave * 32;
+    const int row0 = first_row + tt * STEP;
     if (row0 >= L) break;
+    const int rows_valid = min(32, L - row0);
     const int qrow = row0 + r;
     const bool ok = qrow < L;
-    const size_t roff = head_off + (size_t)qrow * D;
+    const size_t toff = head_off + (size_t)row0 * D;
 
+    // q in B-operand order (d = 16c + 8g + j) and in accumulator order (d = 32t + 8i4 + 4g + j)
+    qt.park(stage, lane);
     float f[DC][8];
-    i16x8_t gf[DC];
 #pragma unroll
     for (int c = 0; c < DC; ++c) {
-      i16x8_t x = {0, 0, 0, 0, 0, 0, 0, 0};
-      gf[c] = i16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
-      if (ok) {
-        x = *reinterpret_cast<const i16x8_t*>(q + roff + 16 * c + 8 * g);
-        gf[c] = *reinterpret_cast<const i16x8_t*>(gout + roff + 16 * c + 8 * g);
-      }
+      const i16x8_t x = *reinterpret_cast<const i16x8_t*>(&stage[r * STR + 16 * c + 8 * g]);
 #pragma unroll
       for (int j = 0; j < 8; ++j) f[c][j] = E::to_float((uint16_t)x[j]);
     }
+    i32x2_t xraw[DT][4];
+#pragma unroll
+    for (int t1 = 0; t1 < DT; ++t1)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; ++i4)
+        xraw[t1][i4] = *reinterpret_cast<const i32x2_t*>(&stage[r * STR + 32 * t1 + 8 * i4 + 4 * g]);
+    wave_lds_fence();
+    gt.park(stage, lane);
+    i16x8_t gf[DC];
+#pragma unroll
+    for (int c = 0; c < DC; ++c) gf[c] = *reinterpret_cast<const i16x8_t*>(&stage[r * STR + 16 * c + 8 * g]);
+    wave_lds_fence();
+    TileRows<D> dq_old;
+    if (accumulate) dq_old.fetch(dq + toff, rows_valid, lane);
+    if (tt + 1 < tiles_per_wg && row0 + STEP < L) {
+      qt.fetch(q + toff + (size_t)STEP * D, min(32, L - row0 - STEP), lane);
+      gt.fetch(gout + toff + (size_t)STEP * D, min(32, L - row0 - STEP), lane);
+    }
+
     float row_mx, row_inv;
     phi_row_pair<Tag, DC>(fmap, f, row_mx, row_inv);
     float den = 0.f;
@@ -100,20 +121,26 @@ __global__ __launch_bounds__(256) void linear_bwd_rows_kernel(
     const float inv_den = 1.0f / den;
 
     // y^T = (KVT a^T) / den ; dy^T = W^T G^T
-    f32x16_t yacc[DT], dyacc[DT];
+    float yv[DT][16], dnv[DT][16];
 #pragma unroll
     for (int t = 0; t < DT; ++t) {
+      f32x16_t yacc, dyacc;
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        yacc[t][i] = 0.f;
-        dyacc[t][i] = 0.f;
+        yacc[i] = 0.f;
+        dyacc[i] = 0.f;
       }
 #pragma unroll
       for (int c = 0; c < DC; ++c) {
         const i16x8_t a1 = *reinterpret_cast<const i16x8_t*>(&sKVT[(32 * t + r) * STR + 16 * c + 8 * g]);
-        yacc[t] = E::mfma32(a1, af[c], yacc[t]);
+        yacc = E::mfma32(a1, af[c], yacc);
         const i16x8_t a2 = *reinterpret_cast<const i16x8_t*>(&sWT[(32 * t + r) * STR + 16 * c + 8 * g]);
-        dyacc[t] = E::mfma32(a2, gf[c], dyacc[t]);
+        dyacc = E::mfma32(a2, gf[c], dyacc);
+      }
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        yv[t][i] = yacc[i];
+        dnv[t][i] = dyacc[i];
       }
     }
     float dden = 0.f;
@@ -121,36 +148,28 @@ __global__ __launch_bounds__(256) void linear_bwd_rows_kernel(
     for (int t = 0; t < DT; ++t)
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        yacc[t][i] *= inv_den;
-        dden += dyacc[t][i] * yacc[t][i];
-        dyacc[t][i] *= inv_den;          // dn^T
+        yv[t][i] *= inv_den;
+        dden += dnv[t][i] * yv[t][i];
+        dnv[t][i] *= inv_den;          // dn^T
       }
     dden += __shfl_xor(dden, 32);
     dden = -dden * inv_den;
+    if (ok && g == 0) dden_out[(size_t)bh * L + qrow] = dden;
 
-    // dn^T as B operand; dn and y to memory for the state kernel
+    // dn^T as B operand (register 8c2+j of tile t is d2 = 32t + 8*((8c2+j)/4) + 4g + j%4, the order sKVP's
+    // columns are stored in); dn and y go to memory for the state kernel
     i16x8_t dnf[DT][2];
 #pragma unroll
     for (int t = 0; t < DT; ++t)
 #pragma unroll
       for (int c2 = 0; c2 < 2; ++c2) {
-        i32x4_t pw, yw;
+        i32x4_t pw;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          pw[j] = (int)E::pack2(dyacc[t][8 * c2 + 2 * j], dyacc[t][8 * c2 + 2 * j + 1]);
-          yw[j] = (int)E::pack2(yacc[t][8 * c2 + 2 * j], yacc[t][8 * c2 + 2 * j + 1]);
-        }
+        for (int j = 0; j < 4; ++j) pw[j] = (int)E::pack2(dnv[t][8 * c2 + 2 * j], dnv[t][8 * c2 + 2 * j + 1]);
         dnf[t][c2] = __builtin_bit_cast(i16x8_t, pw);
-        if (ok) {
-          // registers 8c2..8c2+3 are d = 32t+16c2+4g.., registers 8c2+4..+7 are d = 32t+16c2+8+4g..
-          const int d0 = 32 * t + 16 * c2 + 4 * g;
-          *reinterpret_cast<i32x2_t*>(dn_out + roff + d0) = i32x2_t{pw[0], pw[1]};
-          *reinterpret_cast<i32x2_t*>(dn_out + roff + d0 + 8) = i32x2_t{pw[2], pw[3]};
-          *reinterpret_cast<i32x2_t*>(y_out + roff + d0) = i32x2_t{yw[0], yw[1]};
-          *reinterpret_cast<i32x2_t*>(y_out + roff + d0 + 8) = i32x2_t{yw[2], yw[3]};
-        }
       }
-    if (ok && g == 0) dden_out[(size_t)bh * L + qrow] = dden;
+    store_acc_tile<E, D>(stage, dnv, dn_out + toff, nullptr, rows_valid, lane);
+    store_acc_tile<E, D>(stage, yv, y_out + toff, nullptr, rows_valid, lane);
 
     // da^T = S dn^T + z dden
     float da[DT][16], xq[DT][16];
@@ -169,9 +188,7 @@ __global__ __launch_bounds__(256) void linear_bwd_rows_kernel(
 #pragma unroll
       for (int i4 = 0; i4 < 4; ++i4) {
         const int d0 = 32 * t1 + 8 * i4 + 4 * g;
-        i32x2_t xv = {0, 0};
-        if (ok) xv = *reinterpret_cast<const i32x2_t*>(q + roff + d0);
-        const uint16_t* xp = reinterpret_cast<const uint16_t*>(&xv);
+        const uint16_t* xp = reinterpret_cast<const uint16_t*>(&xraw[t1][i4]);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           da[t1][4 * i4 + j] = acc[4 * i4 + j] + sZ[d0 + j] * dden;
@@ -180,24 +197,7 @@ __global__ __launch_bounds__(256) void linear_bwd_rows_kernel(
       }
     }
     phi_backward<DT>(fmap, xq, da, row_mx, row_inv);
-    if (ok) {
-#pragma unroll
-      for (int t1 = 0; t1 < DT; ++t1)
-#pragma unroll
-        for (int i4 = 0; i4 < 4; ++i4) {
-          uint16_t* dst = dq + roff + 32 * t1 + 8 * i4 + 4 * g;
-          if (accumulate) {
-            const i32x2_t old = *reinterpret_cast<const i32x2_t*>(dst);
-            const uint16_t* op = reinterpret_cast<const uint16_t*>(&old);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) da[t1][4 * i4 + j] += E::to_float(op[j]);
-          }
-          i32x2_t w;
-          w[0] = (int)E::pack2(da[t1][4 * i4 + 0], da[t1][4 * i4 + 1]);
-          w[1] = (int)E::pack2(da[t1][4 * i4 + 2], da[t1][4 * i4 + 3]);
-          *reinterpret_cast<i32x2_t*>(dst) = w;
-        }
-    }
+    store_acc_tile<E, D>(stage, da, dq + toff, accumulate ? &dq_old : nullptr, rows_valid, lane);
   }
 }
 
@@ -378,7 +378,7 @@ __global__ __launch_bounds__(256) void linear_bwd_reduce_kernel(const float* __r
     const float* p = ds_part + (size_t)bh * nsplit * DD + i;
     const float* pw = dw_part + (size_t)bh * nsplit * DD + i;
     float s = 0.f, sw = 0.f;
-#pragma unroll 4
+#pragma unroll 8
     for (int sp = 0; sp < nsplit; ++sp) {
       s += p[(size_t)sp * DD];
       sw += pw[(size_t)sp * DD];
@@ -423,24 +423,27 @@ __global__ __launch_bounds__(256) void linear_bwd_reduce_heads_kernel(const floa
 }
 
 // ---- kv -----------------------------------------------------------------------------------
-template <typename Tag, int D>
-__global__ __launch_bounds__(256) void linear_bwd_kv_kernel(const uint16_t* __restrict__ k, const uint16_t* __restrict__ v,
-                                                            const uint16_t* __restrict__ ds, const uint16_t* __restrict__ dst,
-                                                            const float* __restrict__ dz, uint16_t* __restrict__ dk,
-                                                            uint16_t* __restrict__ dv, int L, int fmap, int tiles_per_wg,
-                                                            int accumulate) {
+// Same tile traffic as the rows kernel: NW waves of 32 keys, whole-row global accesses through a
+// wave-private staging tile.
+template <typename Tag, int D, int NW>
+__global__ __launch_bounds__(64 * NW) void linear_bwd_kv_kernel(const uint16_t* __restrict__ k, const uint16_t* __restrict__ v,
+                                                                const uint16_t* __restrict__ ds,
+                                                                const uint16_t* __restrict__ dst, const float* __restrict__ dz,
+                                                                uint16_t* __restrict__ dk, uint16_t* __restrict__ dv, int L,
+                                                                int fmap, int tiles_per_wg, int accumulate) {
   using E = Elem<Tag>;
   constexpr int DC = D / 16;
   constexpr int DT = D / 32;
   constexpr int STR = D + 8;
   __shared__ __attribute__((aligned(16))) uint16_t sDS[D * STR];   // [d1][d2]  A of dc^T = dS v^T
   __shared__ __attribute__((aligned(16))) uint16_t sDST[D * STR];  // [d2][d1]  A of dv^T = dS^T c^T
+  __shared__ __attribute__((aligned(16))) uint16_t sStage[NW][32 * STR];
   __shared__ __attribute__((aligned(16))) float sDZ[D];
 
   const int bh = blockIdx.y;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int g = lane >> 5, r = lane & 31;
-  for (int idx = tid; idx < D * D / 8; idx += 256) {
+  for (int idx = tid; idx < D * D / 8; idx += 64 * NW) {
     const int row = idx / (D / 8), col = (idx % (D / 8)) * 8;
     *reinterpret_cast<i16x8_t*>(&sDS[row * STR + col]) =
         *reinterpret_cast<const i16x8_t*>(ds + (size_t)bh * D * D + (size_t)row * D + col);
@@ -451,97 +454,98 @@ __global__ __launch_bounds__(256) void linear_bwd_kv_kernel(const uint16_t* __re
   __syncthreads();
 
   const size_t head_off = (size_t)bh * L * D;
+  uint16_t* stage = sStage[wave];
+  constexpr int STEP = 32 * NW;
+  const int first_row = blockIdx.x * tiles_per_wg * STEP + wave * 32;
   for (int tt = 0; tt < tiles_per_wg; ++tt) {
-    const int row0 = (blockIdx.x * tiles_per_wg + tt) * 128 + wave * 32;
+    const int row0 = first_row + tt * STEP;
     if (row0 >= L) break;
-    const int krow = row0 + r;
-    const bool ok = krow < L;
-    const size_t roff = head_off + (size_t)krow * D;
+    const int rows_valid = min(32, L - row0);
+    const size_t toff = head_off + (size_t)row0 * D;
 
+    // two waves share a SIMD and cover each other's load latency; registers are too scarce to fetch ahead
+    TileRows<D> kt, vt;
+    kt.fetch(k + toff, rows_valid, lane);
+    vt.fetch(v + toff, rows_valid, lane);
+    kt.park(stage, lane);
     float f[DC][8];
-    i16x8_t vf[DC];
 #pragma unroll
     for (int c = 0; c < DC; ++c) {
-      i16x8_t x = {0, 0, 0, 0, 0, 0, 0, 0};
-      vf[c] = i16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
-      if (ok) {
-        x = *reinterpret_cast<const i16x8_t*>(k + roff + 16 * c + 8 * g);
-        vf[c] = *reinterpret_cast<const i16x8_t*>(v + roff + 16 * c + 8 * g);
-      }
+      const i16x8_t x = *reinterpret_cast<const i16x8_t*>(&stage[r * STR + 16 * c + 8 * g]);
 #pragma unroll
       for (int j = 0; j < 8; ++j) f[c][j] = E::to_float((uint16_t)x[j]);
     }
+    i32x2_t xraw[DT][4];
+#pragma unroll
+    for (int t = 0; t < DT; ++t)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; ++i4)
+        xraw[t][i4] = *reinterpret_cast<const i32x2_t*>(&stage[r * STR + 32 * t + 8 * i4 + 4 * g]);
+    wave_lds_fence();
+    vt.park(stage, lane);
+    i16x8_t vf[DC];
+#pragma unroll
+    for (int c = 0; c < DC; ++c) vf[c] = *reinterpret_cast<const i16x8_t*>(&stage[r * STR + 16 * c + 8 * g]);
+    wave_lds_fence();
     float row_mx, row_inv;
     phi_row_pair<Tag, DC>(fmap, f, row_mx, row_inv);
-    i16x8_t cf[DC];
+    {
+      // dv^T = dS^T c^T
+      i16x8_t cf[DC];
 #pragma unroll
-    for (int c = 0; c < DC; ++c) {
-      i32x4_t pw;
+      for (int c = 0; c < DC; ++c) {
+        i32x4_t pw;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) pw[j] = (int)E::pack2(f[c][2 * j], f[c][2 * j + 1]);
-      cf[c] = __builtin_bit_cast(i16x8_t, pw);
+        for (int j = 0; j < 4; ++j) pw[j] = (int)E::pack2(f[c][2 * j], f[c][2 * j + 1]);
+        cf[c] = __builtin_bit_cast(i16x8_t, pw);
+      }
+      float dvv[DT][16];
+#pragma unroll
+      for (int t = 0; t < DT; ++t) {
+        f32x16_t vacc;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) vacc[i] = 0.f;
+#pragma unroll
+        for (int c = 0; c < DC; ++c) {
+          const i16x8_t a2 = *reinterpret_cast<const i16x8_t*>(&sDST[(32 * t + r) * STR + 16 * c + 8 * g]);
+          vacc = E::mfma32(a2, cf[c], vacc);
+        }
+#pragma unroll
+        for (int i = 0; i < 16; ++i) dvv[t][i] = vacc[i];
+      }
+      if (accumulate)
+        store_acc_tile<E, D, true>(stage, dvv, dv + toff, nullptr, rows_valid, lane);
+      else
+        store_acc_tile<E, D, false>(stage, dvv, dv + toff, nullptr, rows_valid, lane);
     }
+    // dc^T = dS v^T + dz ; dk = phi'(k) dc
     float dc[DT][16], xk[DT][16];
 #pragma unroll
     for (int t = 0; t < DT; ++t) {
-      f32x16_t acc, vacc;
+      f32x16_t acc;
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        acc[i] = 0.f;
-        vacc[i] = 0.f;
-      }
+      for (int i = 0; i < 16; ++i) acc[i] = 0.f;
 #pragma unroll
       for (int c = 0; c < DC; ++c) {
         const i16x8_t a1 = *reinterpret_cast<const i16x8_t*>(&sDS[(32 * t + r) * STR + 16 * c + 8 * g]);
         acc = E::mfma32(a1, vf[c], acc);
-        const i16x8_t a2 = *reinterpret_cast<const i16x8_t*>(&sDST[(32 * t + r) * STR + 16 * c + 8 * g]);
-        vacc = E::mfma32(a2, cf[c], vacc);
       }
 #pragma unroll
       for (int i4 = 0; i4 < 4; ++i4) {
         const int d0 = 32 * t + 8 * i4 + 4 * g;
-        i32x2_t xv = {0, 0};
-        if (ok) xv = *reinterpret_cast<const i32x2_t*>(k + roff + d0);
-        const uint16_t* xp = reinterpret_cast<const uint16_t*>(&xv);
+        const uint16_t* xp = reinterpret_cast<const uint16_t*>(&xraw[t][i4]);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           dc[t][4 * i4 + j] = acc[4 * i4 + j] + sDZ[d0 + j];
           xk[t][4 * i4 + j] = E::to_float(xp[j]);
         }
-        if (ok) {
-          float dvv[4] = {vacc[4 * i4 + 0], vacc[4 * i4 + 1], vacc[4 * i4 + 2], vacc[4 * i4 + 3]};
-          if (accumulate) {
-            const i32x2_t old = *reinterpret_cast<const i32x2_t*>(dv + roff + d0);
-            const uint16_t* op = reinterpret_cast<const uint16_t*>(&old);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) dvv[j] += E::to_float(op[j]);
-          }
-          i32x2_t w;
-          w[0] = (int)E::pack2(dvv[0], dvv[1]);
-          w[1] = (int)E::pack2(dvv[2], dvv[3]);
-          *reinterpret_cast<i32x2_t*>(dv + roff + d0) = w;
-        }
       }
     }
     phi_backward<DT>(fmap, xk, dc, row_mx, row_inv);
-    if (ok) {
-#pragma unroll
-      for (int t = 0; t < DT; ++t)
-#pragma unroll
-        for (int i4 = 0; i4 < 4; ++i4) {
-          uint16_t* dst = dk + roff + 32 * t + 8 * i4 + 4 * g;
-          if (accumulate) {
-            const i32x2_t old = *reinterpret_cast<const i32x2_t*>(dst);
-            const uint16_t* op = reinterpret_cast<const uint16_t*>(&old);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) dc[t][4 * i4 + j] += E::to_float(op[j]);
-          }
-          i32x2_t w;
-          w[0] = (int)E::pack2(dc[t][4 * i4 + 0], dc[t][4 * i4 + 1]);
-          w[1] = (int)E::pack2(dc[t][4 * i4 + 2], dc[t][4 * i4 + 3]);
-          *reinterpret_cast<i32x2_t*>(dst) = w;
-        }
-    }
+    if (accumulate)
+      store_acc_tile<E, D, true>(stage, dc, dk + toff, nullptr, rows_valid, lane);
+    else
+      store_acc_tile<E, D, false>(stage, dc, dk + toff, nullptr, rows_valid, lane);
   }
 }
 
@@ -577,16 +581,18 @@ static int linear_bwd_impl(const void* q, const void* k, const void* v, const fl
                            void* dk, void* dv, float* d_weight, float* d_bias, int fmap, int BH, int L, int accumulate,
                            char* ws, hipStream_t st) {
   const LinBwdWs w = lin_bwd_ws(BH, L, D);
-  launch_state_build<Tag, D>(k, v, fmap, BH, L, ws, w.fwd, st);
+  launch_state_build<Tag, D>(k, v, weight, fmap, BH, L, ws, w.fwd, st);
   uint16_t* kvt = (uint16_t*)(ws + w.fwd.kvt);
   uint16_t* z = (uint16_t*)(ws + w.fwd.z);
   uint16_t* dn = (uint16_t*)(ws + w.dn);
   uint16_t* y = (uint16_t*)(ws + w.y);
   float* dden = (float*)(ws + w.dden);
-  const int tiles = 4;
-  const dim3 row_grid(cdiv(L, 128 * tiles), BH);
-  hipLaunchKernelGGL((linear_bwd_rows_kernel<Tag, D>), row_grid, dim3(256), 0, st, (const uint16_t*)q,
-                     (const uint16_t*)d_out, kvt, z, weight, (uint16_t*)dq, dn, y, dden, L, fmap, tiles, accumulate);
+  constexpr int NW_ROWS = 4, NW_KV = 8;   // one workgroup per compute unit either way (LDS)
+  const int tiles_rows = balanced_tiles(cdiv(L, 32 * NW_ROWS), BH, 1);
+  const int tiles_kv = balanced_tiles(cdiv(L, 32 * NW_KV), BH, 1);
+  hipLaunchKernelGGL((linear_bwd_rows_kernel<Tag, D, NW_ROWS>), dim3(cdiv(L, 32 * NW_ROWS * tiles_rows), BH), dim3(64 * NW_ROWS), 0, st, (const uint16_t*)q,
+                     (const uint16_t*)d_out, kvt, (const uint16_t*)(ws + w.fwd.kvp), z, (const uint16_t*)(ws + w.fwd.wt), (uint16_t*)dq, dn, y,
+                     dden, L, fmap, tiles_rows, accumulate);
   hipLaunchKernelGGL((linear_bwd_states_kernel<Tag, D>), dim3(w.fwd.nsplit, BH), dim3(256), 0, st, (const uint16_t*)q, dn,
                      (const uint16_t*)d_out, y, dden, (float*)(ws + w.ds_part), (float*)(ws + w.dw_part),
                      (float*)(ws + w.dz_part), (float*)(ws + w.db_part), L, w.fwd.rows_per_split, fmap);
@@ -596,9 +602,9 @@ static int linear_bwd_impl(const void* q, const void* k, const void* v, const fl
                      (float*)(ws + w.dw_head), (float*)(ws + w.db_head), w.fwd.nsplit, D);
   hipLaunchKernelGGL(linear_bwd_reduce_heads_kernel, dim3(cdiv(D * D, 256)), dim3(256), 0, st,
                      (const float*)(ws + w.dw_head), (const float*)(ws + w.db_head), d_weight, d_bias, BH, D);
-  hipLaunchKernelGGL((linear_bwd_kv_kernel<Tag, D>), row_grid, dim3(256), 0, st, (const uint16_t*)k, (const uint16_t*)v,
+  hipLaunchKernelGGL((linear_bwd_kv_kernel<Tag, D, NW_KV>), dim3(cdiv(L, 32 * NW_KV * tiles_kv), BH), dim3(64 * NW_KV), 0, st, (const uint16_t*)k, (const uint16_t*)v,
                      (const uint16_t*)(ws + w.ds), (const uint16_t*)(ws + w.dst), (const float*)(ws + w.dz), (uint16_t*)dk,
-                     (uint16_t*)dv, L, fmap, tiles, accumulate);
+                     (uint16_t*)dv, L, fmap, tiles_kv, accumulate);
   return check_launch("linear_bwd");
 }
 

@@ -101,6 +101,16 @@ static inline LinSplit lin_split(int BH, int L) {
   return s;
 }
 
+// Row-tile kernels: a workgroup stages per-head matrices once and then walks `tiles` steps of its head.
+// With T steps per head, BH heads and room for wg_per_cu workgroups on each of the 256 compute units,
+// pick `tiles` so that all workgroups are resident at once and carry near-equal work.
+static inline int balanced_tiles(int T, int BH, int wg_per_cu) {
+  const int slots = 256 * wg_per_cu;
+  if (BH >= slots) return T < 8 ? T : 8;
+  const int per_head = slots / BH;
+  return cdiv(T, per_head);
+}
+
 int validate_linear(int dtype, int fmap, int B, int H, int L, int D);
 
 }  // namespace sla

@@ -139,30 +139,57 @@ __global__ __launch_bounds__(256) void linear_state_partial_kernel(const uint16_
 }
 
 // ---- kernel 2: reduce partials, round to 16 bit -------------------------------------------
+// Position of column d2 inside a row whose columns are re-ordered to the accumulator slot order of the
+// 32x32 MFMA: slot j of 16-column chunk c, lane group gg  <->  d2 = 16c + 8*(j/4) + 4gg + j%4.
+static __device__ __host__ __forceinline__ int slot_order_pos(int d2) {
+  const int c = d2 >> 4, w16 = d2 & 15;
+  const int gg = (w16 >> 2) & 1, j = ((w16 >> 3) << 2) | (w16 & 3);
+  return 16 * c + 8 * gg + j;
+}
+
+// kvt[bh][d2][d1] (transposed state) and kvp[bh][d1][slot order of d2] (for the backward's S dn^T product)
 template <typename Tag>
 __global__ void linear_state_reduce_kernel(const float* __restrict__ kv_part, const float* __restrict__ z_part,
-                                           uint16_t* __restrict__ kvt, uint16_t* __restrict__ z, int nsplit, int DD, int D) {
+                                           uint16_t* __restrict__ kvt, uint16_t* __restrict__ kvp, uint16_t* __restrict__ z,
+                                           int nsplit, int DD, int D) {
   using E = Elem<Tag>;
   const int bh = blockIdx.y;
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < DD) {
     const float* p = kv_part + (size_t)bh * nsplit * DD + i;
     float s = 0.f;
+#pragma unroll 8
     for (int sp = 0; sp < nsplit; ++sp) s += p[(size_t)sp * DD];
-    kvt[(size_t)bh * DD + i] = E::from_float(s);
+    const uint16_t h = E::from_float(s);
+    kvt[(size_t)bh * DD + i] = h;
+    const int d2 = i / D, d1 = i % D;
+    kvp[(size_t)bh * DD + d1 * D + slot_order_pos(d2)] = h;
   }
   if (i < D) {
     const float* p = z_part + (size_t)bh * nsplit * D + i;
     float s = 0.f;
+#pragma unroll 8
     for (int sp = 0; sp < nsplit; ++sp) s += p[(size_t)sp * D];
     z[(size_t)bh * D + i] = E::from_float(s);
   }
 }
 
+// 16-bit transposed copy of the projection weight: wt[d][e] (A operand of dY^T = W^T G^T).
+// One thread per element.
+template <typename Tag>
+__global__ void linear_prep_weight_kernel(const float* __restrict__ weight, uint16_t* __restrict__ wt, int D) {
+  using E = Elem<Tag>;
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= D * D) return;
+  const int e = i / D, d = i % D;
+  const uint16_t h = E::from_float(weight[i]);
+  wt[d * D + e] = h;
+}
+
 // ---- workspace layout of the state build -----------------------------------------------------
 struct LinWs {
   int nsplit, rows_per_split;
-  size_t kv_part, z_part, kvt, z, total;
+  size_t kv_part, z_part, kvt, kvp, kvwt, z, wt, total;
 };
 
 static inline LinWs lin_ws(int BH, int L, int D) {
@@ -174,24 +201,29 @@ static inline LinWs lin_ws(int BH, int L, int D) {
   w.kv_part = off; off += align_up((int64_t)BH * w.nsplit * D * D * 4, 256);
   w.z_part = off;  off += align_up((int64_t)BH * w.nsplit * D * 4, 256);
   w.kvt = off;     off += align_up((int64_t)BH * D * D * 2, 256);
+  w.kvp = off;     off += align_up((int64_t)BH * D * D * 2, 256);
+  w.kvwt = off;    off += align_up((int64_t)BH * D * D * 2, 256);
   w.z = off;       off += align_up((int64_t)BH * D * 2, 256);
+  w.wt = off;      off += align_up((int64_t)D * D * 2, 256);
   w.total = off;
   return w;
 }
 
 
-// Streams K and V once and leaves KVT (16 bit, [d2][d1]) and z (16 bit) in the workspace.
+// Streams K and V once and leaves KVT, KVP, z (16 bit) and the 16-bit transposed weight in the workspace.
 template <typename Tag, int D>
-static inline void launch_state_build(const void* k, const void* v, int fmap, int BH, int L, char* ws, const LinWs& w,
-                                      hipStream_t st) {
+static inline void launch_state_build(const void* k, const void* v, const float* weight, int fmap, int BH, int L, char* ws,
+                                      const LinWs& w, hipStream_t st) {
   float* kv_part = (float*)(ws + w.kv_part);
   float* z_part = (float*)(ws + w.z_part);
   uint16_t* kvt = (uint16_t*)(ws + w.kvt);
   uint16_t* z = (uint16_t*)(ws + w.z);
   hipLaunchKernelGGL((linear_state_partial_kernel<Tag, D>), dim3(w.nsplit, BH), dim3(256), 0, st, (const uint16_t*)k,
                      (const uint16_t*)v, kv_part, z_part, L, w.rows_per_split, fmap);
-  hipLaunchKernelGGL((linear_state_reduce_kernel<Tag>), dim3(cdiv(D * D, 256), BH), dim3(256), 0, st, kv_part, z_part, kvt, z,
-                     w.nsplit, D * D, D);
+  hipLaunchKernelGGL((linear_state_reduce_kernel<Tag>), dim3(cdiv(D * D, 256), BH), dim3(256), 0, st, kv_part, z_part, kvt,
+                     (uint16_t*)(ws + w.kvp), z, w.nsplit, D * D, D);
+  hipLaunchKernelGGL((linear_prep_weight_kernel<Tag>), dim3(cdiv(D * D, 256)), dim3(256), 0, st, weight,
+                     (uint16_t*)(ws + w.wt), D);
 }
 
 }  // namespace sla
