@@ -97,12 +97,14 @@ __global__ __launch_bounds__(64) void bwd_col_lists_kernel(const int8_t* __restr
 }
 
 // ---- dQ ---------------------------------------------------------------------------------
+// One workgroup per query block, one wave per 32 queries.  Register use is held to 256 so that two waves
+// share a SIMD.  K and V tiles go global -> registers -> LDS; both tiles of the next step are in flight
+// during the whole current step.
 template <typename Tag, int D, int BLKQ>
-__global__ __launch_bounds__(BLKQ * 2) void bwd_dq_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ k,
-                                                          const uint16_t* __restrict__ v, const uint16_t* __restrict__ d_o,
-                                                          const float* __restrict__ lse, const float* __restrict__ delta,
-                                                          const void* __restrict__ lut, int lut64, uint16_t* __restrict__ dq,
-                                                          int L, int Mblk, int topk, float qk_scale, int total) {
+__global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))) void bwd_dq_kernel(
+    const uint16_t* __restrict__ q, const uint16_t* __restrict__ k, const uint16_t* __restrict__ v,
+    const uint16_t* __restrict__ d_o, const float* __restrict__ lse, const float* __restrict__ delta,
+    const void* __restrict__ lut, int lut64, uint16_t* __restrict__ dq, int L, int Mblk, int topk, float qk_scale, int total) {
   using E = Elem<Tag>;
   constexpr int BLKK = 64;
   constexpr int NT = BLKQ * 2;
@@ -125,20 +127,19 @@ __global__ __launch_bounds__(BLKQ * 2) void bwd_dq_kernel(const uint16_t* __rest
   const float c_log2e = qk_scale * 1.4426950408889634f;
 
   const size_t head_off = (size_t)bh * L * D;
-  const uint16_t* kh = k + head_off;
-  const uint16_t* vh = v + head_off;
+  const uint32_t head_bytes = (uint32_t)L * D * 2;
+  const __amdgpu_buffer_rsrc_t qh = make_rsrc(q + head_off, head_bytes);
+  const __amdgpu_buffer_rsrc_t doh = make_rsrc(d_o + head_off, head_bytes);
+  const __amdgpu_buffer_rsrc_t kh = make_rsrc(k + head_off, head_bytes);
+  const __amdgpu_buffer_rsrc_t vh = make_rsrc(v + head_off, head_bytes);
   const int qrow = mb * BLKQ + wave * 32 + r;
   const bool qok = qrow < L;
 
   i16x8_t qf[DC], dof[DC];
 #pragma unroll
   for (int c = 0; c < DC; ++c) {
-    qf[c] = i16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
-    dof[c] = i16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
-    if (qok) {
-      qf[c] = *reinterpret_cast<const i16x8_t*>(q + head_off + (size_t)qrow * D + 16 * c + 8 * g);
-      dof[c] = *reinterpret_cast<const i16x8_t*>(d_o + head_off + (size_t)qrow * D + 16 * c + 8 * g);
-    }
+    qf[c] = buf_load_b128(qh, ((uint32_t)qrow * D + 16 * c + 8 * g) * 2);      // rows past L read as zero
+    dof[c] = buf_load_b128(doh, ((uint32_t)qrow * D + 16 * c + 8 * g) * 2);
   }
   // rows past L: lse = +inf makes every probability exactly 0 (the reference loads `other=inf`)
   const float lse_q = qok ? lse[(size_t)bh * L + qrow] : INFINITY;
@@ -155,13 +156,9 @@ __global__ __launch_bounds__(BLKQ * 2) void bwd_dq_kernel(const uint16_t* __rest
     for (int i = 0; i < NLD; ++i) {
       const int idx = tid + i * NT;
       const int row = idx / CPR, col = (idx % CPR) * 8;
-      const int grow = nb * BLKK + row;
-      kreg[i] = i16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
-      vreg[i] = i16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
-      if (grow < L) {
-        kreg[i] = *reinterpret_cast<const i16x8_t*>(kh + (size_t)grow * D + col);
-        vreg[i] = *reinterpret_cast<const i16x8_t*>(vh + (size_t)grow * D + col);
-      }
+      const uint32_t off = ((uint32_t)(nb * BLKK + row) * D + col) * 2;      // rows past L read as zero
+      kreg[i] = buf_load_b128(kh, off);
+      vreg[i] = buf_load_b128(vh, off);
     }
   };
   auto store_tile = [&]() {
@@ -184,14 +181,18 @@ __global__ __launch_bounds__(BLKQ * 2) void bwd_dq_kernel(const uint16_t* __rest
   const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
 
   int nb = topk > 0 ? lut_at(0) : 0;
-  if (topk > 0) load_tile(nb);
-  for (int it = 0; it < topk; ++it) {
-    __syncthreads();
+  int nb_next = topk > 1 ? lut_at(1) : 0;
+  if (topk > 0) {
+    load_tile(nb);
     store_tile();
-    __syncthreads();
+  }
+  __syncthreads();
+  for (int it = 0; it < topk; ++it) {
     const int kv_valid = L - nb * BLKK;
-    if (it + 1 < topk) {
-      nb = lut_at(it + 1);
+    const bool more = it + 1 < topk;
+    if (more) {
+      nb = nb_next;
+      nb_next = it + 2 < topk ? lut_at(it + 2) : 0;
       load_tile(nb);
     }
 #pragma unroll
@@ -206,18 +207,15 @@ __global__ __launch_bounds__(BLKQ * 2) void bwd_dq_kernel(const uint16_t* __rest
       for (int c = 0; c < DC; ++c) {
         const i16x8_t a = *reinterpret_cast<const i16x8_t*>(&sK[(32 * t + r) * KSTR + 16 * c + 8 * g]);
         s = E::mfma32(a, qf[c], s);
-      }
-#pragma unroll
-      for (int c = 0; c < DC; ++c) {
-        const i16x8_t a = *reinterpret_cast<const i16x8_t*>(&sV[(32 * t + r) * VSTR + 16 * c + 8 * g]);
-        dp = E::mfma32(a, dof[c], dp);
+        const i16x8_t b = *reinterpret_cast<const i16x8_t*>(&sV[(32 * t + r) * VSTR + 16 * c + 8 * g]);
+        dp = E::mfma32(b, dof[c], dp);
       }
       // dS^T = P^T * (dP^T - delta), zero on key rows past L
+      const int lim = kv_valid - 4 * g;      // key index of register i is 32t + 8(i/4) + i%4 + 4g
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        const int key = 32 * t + 8 * (i >> 2) + 4 * g + (i & 3);
         float p = fast_exp2(__builtin_fmaf(s[i], c_log2e, -lse_q));
-        if (key >= kv_valid) p = 0.f;
+        if (32 * t + 8 * (i >> 2) + (i & 3) >= lim) p = 0.f;
         s[i] = p * (dp[i] - delta_q);
       }
 #pragma unroll
@@ -234,6 +232,9 @@ __global__ __launch_bounds__(BLKQ * 2) void bwd_dq_kernel(const uint16_t* __rest
         }
       }
     }
+    __syncthreads();                       // both tiles fully consumed
+    if (more) store_tile();
+    __syncthreads();                       // next tiles visible
   }
   if (qok) {
     uint16_t* orow = dq + head_off + (size_t)qrow * D;
