@@ -18,6 +18,7 @@
 //   dkdv       : per key block over its list; S = Q K^T and dP = dO V^T with K^T/V^T resident
 //                in registers as B operands; P and dS leave the accumulators in B-operand layout
 //                for dV^T += dO^T P and dK^T += Q^T dS (Q^T, dO^T via transposing LDS reads).
+//                Four waves: two key halves x two halves of the head dimension.
 #include "common.h"
 
 namespace sla {
@@ -251,20 +252,25 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
 }
 
 // ---- dK, dV -----------------------------------------------------------------------------
-// One workgroup (2 waves) per key block; wave w owns keys 32w..32w+31 of it.
+// One workgroup of four waves per key block.  Wave (kh, dh): kh = wave % 2 selects keys 32kh..32kh+31 of
+// the block, dh = wave / 2 selects the half of the head dimension whose dK^T / dV^T rows this wave
+// accumulates.  Per tile of 64 query rows the two waves that share kh split the rows: each forms S and dP
+// for its 32 rows, turns them into P and dS (accumulator layout = B-operand layout of the second
+// products) and hands a copy to its partner through LDS; then each adds all 64 rows into its own half of
+// dV^T += dO^T P and dK^T += Q^T dS.  Splitting the accumulators this way keeps a wave at 256 registers,
+// so two waves share a SIMD.
 template <typename Tag, int D, int BLKQ>
-__global__ __launch_bounds__(128) void bwd_dkdv_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ k,
-                                                       const uint16_t* __restrict__ v, const uint16_t* __restrict__ d_o,
-                                                       const float* __restrict__ lse, const float* __restrict__ delta,
-                                                       const int* __restrict__ list, const int* __restrict__ count,
-                                                       uint16_t* __restrict__ dk, uint16_t* __restrict__ dv, int L, int Mblk,
-                                                       int Nblk, float qk_scale, int total) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void bwd_dkdv_kernel(
+    const uint16_t* __restrict__ q, const uint16_t* __restrict__ k, const uint16_t* __restrict__ v,
+    const uint16_t* __restrict__ d_o, const float* __restrict__ lse, const float* __restrict__ delta,
+    const int* __restrict__ list, const int* __restrict__ count, uint16_t* __restrict__ dk, uint16_t* __restrict__ dv, int L,
+    int Mblk, int Nblk, float qk_scale, int total) {
   using E = Elem<Tag>;
   constexpr int TQ = 64;                  // query rows per LDS tile
   constexpr int SUB = BLKQ / TQ;          // tiles per listed query block
-  constexpr int NT = 128;
+  constexpr int NT = 256;
   constexpr int DC = D / 16;
-  constexpr int DT = D / 32;
+  constexpr int DH = D / 64;              // 32-row tiles of dK^T / dV^T owned by one wave
   constexpr int STR = D + 16;             // Q and dO are read row-wise and transposed
   constexpr int CPR = D / 8;
   constexpr int NLD = TQ * CPR / NT;
@@ -273,38 +279,40 @@ __global__ __launch_bounds__(128) void bwd_dkdv_kernel(const uint16_t* __restric
   __shared__ __attribute__((aligned(16))) uint16_t sDO[TQ * STR];
   __shared__ __attribute__((aligned(16))) float sLse[TQ];
   __shared__ __attribute__((aligned(16))) float sDelta[TQ];
+  __shared__ __attribute__((aligned(16))) i16x8_t sXP[4][2][64];    // [wave][16-row group][lane] packed P
+  __shared__ __attribute__((aligned(16))) i16x8_t sXS[4][2][64];    // same for dS
 
   const int logical = xcd_remap(blockIdx.x, gridDim.x, total);
   if (logical < 0) return;
   const int bh = logical / Nblk;
   const int nb = logical - bh * Nblk;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int kh = wave & 1, dh = wave >> 1;
   const int g = lane >> 5, r = lane & 31;
   const float c_log2e = qk_scale * 1.4426950408889634f;
 
   const size_t head_off = (size_t)bh * L * D;
-  const uint16_t* qh = q + head_off;
-  const uint16_t* doh = d_o + head_off;
+  const uint32_t head_bytes = (uint32_t)L * D * 2;
+  const __amdgpu_buffer_rsrc_t qh = make_rsrc(q + head_off, head_bytes);
+  const __amdgpu_buffer_rsrc_t doh = make_rsrc(d_o + head_off, head_bytes);
+  const __amdgpu_buffer_rsrc_t kb = make_rsrc(k + head_off, head_bytes);
+  const __amdgpu_buffer_rsrc_t vb = make_rsrc(v + head_off, head_bytes);
   const float* lseh = lse + (size_t)bh * L;
   const float* deltah = delta + (size_t)bh * L;
 
   // K^T and V^T fragments (B operands): this lane's key column, 8 adjacent d per chunk
-  const int krow = nb * 64 + wave * 32 + r;
+  const int krow = nb * 64 + kh * 32 + r;
   const bool kok = krow < L;
   i16x8_t kf[DC], vf[DC];
 #pragma unroll
   for (int c = 0; c < DC; ++c) {
-    kf[c] = i16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
-    vf[c] = i16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
-    if (kok) {
-      kf[c] = *reinterpret_cast<const i16x8_t*>(k + head_off + (size_t)krow * D + 16 * c + 8 * g);
-      vf[c] = *reinterpret_cast<const i16x8_t*>(v + head_off + (size_t)krow * D + 16 * c + 8 * g);
-    }
+    kf[c] = buf_load_b128(kb, ((uint32_t)krow * D + 16 * c + 8 * g) * 2);     // rows past L read as zero
+    vf[c] = buf_load_b128(vb, ((uint32_t)krow * D + 16 * c + 8 * g) * 2);
   }
 
-  f32x16_t dkacc[DT], dvacc[DT];
+  f32x16_t dkacc[DH], dvacc[DH];
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt)
+  for (int dt = 0; dt < DH; ++dt)
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       dkacc[dt][i] = 0.f;
@@ -322,13 +330,9 @@ __global__ __launch_bounds__(128) void bwd_dkdv_kernel(const uint16_t* __restric
     for (int i = 0; i < NLD; ++i) {
       const int idx = tid + i * NT;
       const int row = idx / CPR, col = (idx % CPR) * 8;
-      const int grow = row0 + row;
-      qreg[i] = i16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
-      doreg[i] = i16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
-      if (grow < L) {
-        qreg[i] = *reinterpret_cast<const i16x8_t*>(qh + (size_t)grow * D + col);
-        doreg[i] = *reinterpret_cast<const i16x8_t*>(doh + (size_t)grow * D + col);
-      }
+      const uint32_t off = ((uint32_t)(row0 + row) * D + col) * 2;            // rows past L read as zero
+      qreg[i] = buf_load_b128(qh, off);
+      doreg[i] = buf_load_b128(doh, off);
     }
     if (tid < TQ) {
       const int grow = row0 + tid;
@@ -353,79 +357,100 @@ __global__ __launch_bounds__(128) void bwd_dkdv_kernel(const uint16_t* __restric
   const int tr_row = (lane & 15) >> 2;
   const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
 
-  if (ntile > 0) load_tile(tile_row0(0));
-  for (int ti = 0; ti < ntile; ++ti) {
-    __syncthreads();
+  int row_next = ntile > 1 ? tile_row0(1) : 0;
+  if (ntile > 0) {
+    load_tile(tile_row0(0));
     store_tile();
-    __syncthreads();
-    if (ti + 1 < ntile) load_tile(tile_row0(ti + 1));
+  }
+  __syncthreads();
+  for (int ti = 0; ti < ntile; ++ti) {
+    if (ti + 1 < ntile) {
+      load_tile(row_next);
+      row_next = ti + 2 < ntile ? tile_row0(ti + 2) : 0;
+    }
+    // ---- phase 1: P and dS of query rows 32dh..32dh+31 of the tile against this wave's 32 keys ----
+    f32x16_t s, dp;
 #pragma unroll
-    for (int t = 0; t < TQ / 32; ++t) {
-      f32x16_t s, dp;
+    for (int i = 0; i < 16; ++i) {
+      s[i] = 0.f;
+      dp[i] = 0.f;
+    }
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        s[i] = 0.f;
-        dp[i] = 0.f;
+    for (int c = 0; c < DC; ++c) {
+      const i16x8_t a = *reinterpret_cast<const i16x8_t*>(&sQ[(32 * dh + r) * STR + 16 * c + 8 * g]);
+      s = E::mfma32(a, kf[c], s);
+      const i16x8_t b = *reinterpret_cast<const i16x8_t*>(&sDO[(32 * dh + r) * STR + 16 * c + 8 * g]);
+      dp = E::mfma32(b, vf[c], dp);
+    }
+    // accumulator rows are queries 32dh + 8*(i/4) + 4g + i%4; this lane's column is its key
+#pragma unroll
+    for (int i4 = 0; i4 < 4; ++i4) {
+      const f32x4_t l4 = *reinterpret_cast<const f32x4_t*>(&sLse[32 * dh + 8 * i4 + 4 * g]);
+      const f32x4_t d4 = *reinterpret_cast<const f32x4_t*>(&sDelta[32 * dh + 8 * i4 + 4 * g]);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int i = 4 * i4 + j;
+        float p = fast_exp2(__builtin_fmaf(s[i], c_log2e, -l4[j]));
+        if (!kok) p = 0.f;
+        s[i] = p;
+        dp[i] = p * (dp[i] - d4[j]);
       }
+    }
+    i16x8_t pmine[2], smine[2];
 #pragma unroll
-      for (int c = 0; c < DC; ++c) {
-        const i16x8_t a = *reinterpret_cast<const i16x8_t*>(&sQ[(32 * t + r) * STR + 16 * c + 8 * g]);
-        s = E::mfma32(a, kf[c], s);
+    for (int c2 = 0; c2 < 2; ++c2) {
+      i32x4_t pw, dw;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        pw[j] = (int)E::pack2(s[8 * c2 + 2 * j], s[8 * c2 + 2 * j + 1]);
+        dw[j] = (int)E::pack2(dp[8 * c2 + 2 * j], dp[8 * c2 + 2 * j + 1]);
       }
+      pmine[c2] = __builtin_bit_cast(i16x8_t, pw);
+      smine[c2] = __builtin_bit_cast(i16x8_t, dw);
+      sXP[wave][c2][lane] = pmine[c2];
+      sXS[wave][c2][lane] = smine[c2];
+    }
+    __syncthreads();                       // partner's P and dS visible
+    // ---- phase 2: all 64 query rows into this wave's half of dV^T and dK^T ----
 #pragma unroll
-      for (int c = 0; c < DC; ++c) {
-        const i16x8_t a = *reinterpret_cast<const i16x8_t*>(&sDO[(32 * t + r) * STR + 16 * c + 8 * g]);
-        dp = E::mfma32(a, vf[c], dp);
-      }
-      // accumulator rows are queries 32t + 8*(i/4) + 4g + i%4; this lane's column is its key
-#pragma unroll
-      for (int i4 = 0; i4 < 4; ++i4) {
-        const f32x4_t l4 = *reinterpret_cast<const f32x4_t*>(&sLse[32 * t + 8 * i4 + 4 * g]);
-        const f32x4_t d4 = *reinterpret_cast<const f32x4_t*>(&sDelta[32 * t + 8 * i4 + 4 * g]);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const int i = 4 * i4 + j;
-          float p = fast_exp2(__builtin_fmaf(s[i], c_log2e, -l4[j]));
-          if (!kok) p = 0.f;
-          s[i] = p;
-          dp[i] = p * (dp[i] - d4[j]);
-        }
-      }
+    for (int h = 0; h < 2; ++h)
 #pragma unroll
       for (int c2 = 0; c2 < 2; ++c2) {
-        i32x4_t pw, dw;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          pw[j] = (int)E::pack2(s[8 * c2 + 2 * j], s[8 * c2 + 2 * j + 1]);
-          dw[j] = (int)E::pack2(dp[8 * c2 + 2 * j], dp[8 * c2 + 2 * j + 1]);
+        // rows 32h + 16c2..: own registers when h == dh, else the partner's copy (wave ^ 2: same keys, other rows)
+        i16x8_t pb = pmine[c2], dsb = smine[c2];
+        if (h != dh) {
+          pb = sXP[wave ^ 2][c2][lane];
+          dsb = sXS[wave ^ 2][c2][lane];
         }
-        const i16x8_t pb = __builtin_bit_cast(i16x8_t, pw);
-        const i16x8_t dsb = __builtin_bit_cast(i16x8_t, dw);
-        const int q0 = 32 * t + 16 * c2 + 4 * g + tr_row;
+        const int q0 = 32 * h + 16 * c2 + 4 * g + tr_row;
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-          const uint16_t* pdo = &sDO[q0 * STR + 32 * dt + tr_col];
+        for (int dt = 0; dt < DH; ++dt) {
+          const int dcol = 32 * (DH * dh + dt) + tr_col;
+          const uint16_t* pdo = &sDO[q0 * STR + dcol];
           dvacc[dt] = E::mfma32(concat4(lds_read_tr16(pdo), lds_read_tr16(pdo + 8 * STR)), pb, dvacc[dt]);
-          const uint16_t* pq = &sQ[q0 * STR + 32 * dt + tr_col];
+          const uint16_t* pq = &sQ[q0 * STR + dcol];
           dkacc[dt] = E::mfma32(concat4(lds_read_tr16(pq), lds_read_tr16(pq + 8 * STR)), dsb, dkacc[dt]);
         }
       }
-    }
+    __syncthreads();                       // tile and exchange buffers fully consumed
+    if (ti + 1 < ntile) store_tile();
+    __syncthreads();                       // next tile visible
   }
   if (kok) {
     uint16_t* dkrow = dk + head_off + (size_t)krow * D;
     uint16_t* dvrow = dv + head_off + (size_t)krow * D;
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
+    for (int dt = 0; dt < DH; ++dt)
 #pragma unroll
       for (int i4 = 0; i4 < 4; ++i4) {
+        const int d0 = 32 * (DH * dh + dt) + 8 * i4 + 4 * g;
         i32x2_t w;
         w[0] = (int)E::pack2(dkacc[dt][4 * i4 + 0] * qk_scale, dkacc[dt][4 * i4 + 1] * qk_scale);
         w[1] = (int)E::pack2(dkacc[dt][4 * i4 + 2] * qk_scale, dkacc[dt][4 * i4 + 3] * qk_scale);
-        *reinterpret_cast<i32x2_t*>(dkrow + 32 * dt + 8 * i4 + 4 * g) = w;
+        *reinterpret_cast<i32x2_t*>(dkrow + d0) = w;
         w[0] = (int)E::pack2(dvacc[dt][4 * i4 + 0], dvacc[dt][4 * i4 + 1]);
         w[1] = (int)E::pack2(dvacc[dt][4 * i4 + 2], dvacc[dt][4 * i4 + 3]);
-        *reinterpret_cast<i32x2_t*>(dvrow + 32 * dt + 8 * i4 + 4 * g) = w;
+        *reinterpret_cast<i32x2_t*>(dvrow + d0) = w;
       }
   }
 }
@@ -472,7 +497,7 @@ static int bwd_impl(const void* q, const void* k, const void* v, const void* o, 
                      (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse, delta, lut, lut64, (uint16_t*)dq, L,
                      Mblk, topk, qk_scale, total_q);
   const int total_k = BH * Nblk;
-  hipLaunchKernelGGL((bwd_dkdv_kernel<Tag, D, BLKQ>), dim3(xcd_grid(total_k)), dim3(128), 0, st, (const uint16_t*)q,
+  hipLaunchKernelGGL((bwd_dkdv_kernel<Tag, D, BLKQ>), dim3(xcd_grid(total_k)), dim3(256), 0, st, (const uint16_t*)q,
                      (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse, delta, list, count, (uint16_t*)dk,
                      (uint16_t*)dv, L, Mblk, Nblk, qk_scale, total_k);
   return check_launch("sparse_attn_bwd");
