@@ -96,6 +96,17 @@ int sla_linear_fwd(const void* q, const void* k, const void* v, const float* wei
                    const void* residual, void* out, int dtype, int fmap, int B, int H, int L, int D,
                    void* workspace, int64_t workspace_bytes, void* stream);
 
+/* The two halves of sla_linear_fwd, for callers that overlap them with other work: the state half
+ * depends on k and v only (it can run beside the mask builder on another stream), the output half
+ * consumes the workspace the state half filled (same workspace size, SLA_WS_LINEAR_FWD).
+ * sla_linear_fwd == sla_linear_state_fwd followed by sla_linear_out_fwd on one stream.
+ * Replace sparse_linear_attention/core.py:90-95 (feature map of k, calc_linear's k^T v and k sum) and
+ * core.py:90-100 (feature map of q, the rest of calc_linear, proj_l, sum) respectively. */
+int sla_linear_state_fwd(const void* k, const void* v, const float* weight, int dtype, int fmap, int B, int H, int L,
+                         int D, void* workspace, int64_t workspace_bytes, void* stream);
+int sla_linear_out_fwd(const void* q, const float* bias, const void* residual, void* out, int dtype, int fmap, int B,
+                       int H, int L, int D, void* workspace, int64_t workspace_bytes, void* stream);
+
 /* Linear branch backward.  d_out is the gradient of `out` above.  Writes dq, dk, dv in `dtype`
  * (gradients of the linear branch only; the residual's gradient is d_out itself) and the
  * fp32 gradients of weight (D,D) and bias (D).  With accumulate != 0, dq/dk/dv already hold

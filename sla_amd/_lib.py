@@ -33,6 +33,8 @@ SIGNATURES = {
     "sla_sparse_attn_bwd": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I,
                                  _I, _F, _P, _I64, _P]),
     "sla_linear_fwd": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I64, _P]),
+    "sla_linear_state_fwd": (_I, [_P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I64, _P]),
+    "sla_linear_out_fwd": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I64, _P]),
     "sla_linear_bwd": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P, _I64, _P]),
     "sage_quant_qk": (_I, [_P, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _I64, _P]),
     "sage_quant_v": (_I, [_P, _I, _I, _I, _I, _I, _P, _P, _P, _I64, _P]),

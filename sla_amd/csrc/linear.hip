@@ -139,18 +139,24 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 int64_t linear_fwd_workspace_bytes(int BH, int L, int D) { return (int64_t)lin_ws(BH, L, D).total; }
 
 template <typename Tag, int D>
-static int linear_fwd_impl(const void* q, const void* k, const void* v, const float* weight, const float* bias,
-                           const void* residual, void* out, int fmap, int BH, int L, char* ws, hipStream_t st) {
+static int linear_state_impl(const void* k, const void* v, const float* weight, int fmap, int BH, int L, char* ws,
+                             hipStream_t st) {
   const LinWs w = lin_ws(BH, L, D);
-  uint16_t* kvt = (uint16_t*)(ws + w.kvt);
-  uint16_t* kvwt = (uint16_t*)(ws + w.kvwt);
-  uint16_t* z = (uint16_t*)(ws + w.z);
   launch_state_build<Tag, D>(k, v, weight, fmap, BH, L, ws, w, st);
-  hipLaunchKernelGGL((linear_fold_kernel<Tag>), dim3(cdiv(D * D, 256), BH), dim3(256), 0, st, kvt, weight, kvwt, D);
+  hipLaunchKernelGGL((linear_fold_kernel<Tag>), dim3(cdiv(D * D, 256), BH), dim3(256), 0, st,
+                     (const uint16_t*)(ws + w.kvt), weight, (uint16_t*)(ws + w.kvwt), D);
+  return check_launch("linear_state_fwd");
+}
+
+template <typename Tag, int D>
+static int linear_out_impl(const void* q, const float* bias, const void* residual, void* out, int fmap, int BH, int L,
+                           char* ws, hipStream_t st) {
+  const LinWs w = lin_ws(BH, L, D);
   const int tiles = balanced_tiles(cdiv(L, 128), BH, 2);
-  hipLaunchKernelGGL((linear_out_kernel<Tag, D>), dim3(cdiv(L, 128 * tiles), BH), dim3(256), 0, st, (const uint16_t*)q, kvwt,
-                     z, bias, (const uint16_t*)residual, (uint16_t*)out, L, fmap, tiles);
-  return check_launch("linear_fwd");
+  hipLaunchKernelGGL((linear_out_kernel<Tag, D>), dim3(cdiv(L, 128 * tiles), BH), dim3(256), 0, st, (const uint16_t*)q,
+                     (const uint16_t*)(ws + w.kvwt), (const uint16_t*)(ws + w.z), bias, (const uint16_t*)residual,
+                     (uint16_t*)out, L, fmap, tiles);
+  return check_launch("linear_out_fwd");
 }
 
 int validate_linear(int dtype, int fmap, int B, int H, int L, int D) {
@@ -168,22 +174,27 @@ int validate_linear(int dtype, int fmap, int B, int H, int L, int D) {
 
 using namespace sla;
 
-extern "C" int sla_linear_fwd(const void* q, const void* k, const void* v, const float* weight, const float* bias,
-                              const void* residual, void* out, int dtype, int fmap, int B, int H, int L, int D,
-                              void* workspace, int64_t workspace_bytes, void* stream) {
-  int rc = validate_linear(dtype, fmap, B, H, L, D);
-  if (rc) return rc;
-  SLA_REQUIRE(q && k && v && weight && bias && out && workspace, SLA_ERR_BAD_ARG, "null pointer");
-  SLA_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out | (uintptr_t)residual | (uintptr_t)weight |
-               (uintptr_t)workspace) % 16 == 0,
-              SLA_ERR_BAD_ARG, "pointers must be 16-byte aligned");
-  const int BH = B * H;
+static int check_linear_ws(int BH, int L, int D, const void* workspace, int64_t workspace_bytes) {
+  SLA_REQUIRE(workspace && (uintptr_t)workspace % 16 == 0, SLA_ERR_BAD_ARG, "workspace null or not 16-byte aligned");
   const int64_t need = linear_fwd_workspace_bytes(BH, L, D);
   SLA_REQUIRE(workspace_bytes >= need, SLA_ERR_WORKSPACE, "workspace of %lld bytes, need %lld", (long long)workspace_bytes,
               (long long)need);
+  return SLA_OK;
+}
+
+extern "C" int sla_linear_state_fwd(const void* k, const void* v, const float* weight, int dtype, int fmap, int B, int H,
+                                    int L, int D, void* workspace, int64_t workspace_bytes, void* stream) {
+  int rc = validate_linear(dtype, fmap, B, H, L, D);
+  if (rc) return rc;
+  SLA_REQUIRE(k && v && weight, SLA_ERR_BAD_ARG, "null pointer");
+  SLA_REQUIRE(((uintptr_t)k | (uintptr_t)v | (uintptr_t)weight) % 16 == 0, SLA_ERR_BAD_ARG,
+              "pointers must be 16-byte aligned");
+  const int BH = B * H;
+  rc = check_linear_ws(BH, L, D, workspace, workspace_bytes);
+  if (rc) return rc;
   hipStream_t st = (hipStream_t)stream;
   char* ws = (char*)workspace;
-#define SLA_LIN_CASE(TAG, DD) return linear_fwd_impl<TAG, DD>(q, k, v, weight, bias, residual, out, fmap, BH, L, ws, st)
+#define SLA_LIN_CASE(TAG, DD) return linear_state_impl<TAG, DD>(k, v, weight, fmap, BH, L, ws, st)
   if (dtype == SLA_BF16) {
     if (D == 128) SLA_LIN_CASE(bf16_tag, 128);
     SLA_LIN_CASE(bf16_tag, 64);
@@ -191,4 +202,37 @@ extern "C" int sla_linear_fwd(const void* q, const void* k, const void* v, const
   if (D == 128) SLA_LIN_CASE(f16_tag, 128);
   SLA_LIN_CASE(f16_tag, 64);
 #undef SLA_LIN_CASE
+}
+
+extern "C" int sla_linear_out_fwd(const void* q, const float* bias, const void* residual, void* out, int dtype, int fmap,
+                                  int B, int H, int L, int D, void* workspace, int64_t workspace_bytes, void* stream) {
+  int rc = validate_linear(dtype, fmap, B, H, L, D);
+  if (rc) return rc;
+  SLA_REQUIRE(q && bias && out, SLA_ERR_BAD_ARG, "null pointer");
+  SLA_REQUIRE(((uintptr_t)q | (uintptr_t)out | (uintptr_t)residual) % 16 == 0, SLA_ERR_BAD_ARG,
+              "pointers must be 16-byte aligned");
+  const int BH = B * H;
+  rc = check_linear_ws(BH, L, D, workspace, workspace_bytes);
+  if (rc) return rc;
+  hipStream_t st = (hipStream_t)stream;
+  char* ws = (char*)workspace;
+#define SLA_LIN_CASE(TAG, DD) return linear_out_impl<TAG, DD>(q, bias, residual, out, fmap, BH, L, ws, st)
+  if (dtype == SLA_BF16) {
+    if (D == 128) SLA_LIN_CASE(bf16_tag, 128);
+    SLA_LIN_CASE(bf16_tag, 64);
+  }
+  if (D == 128) SLA_LIN_CASE(f16_tag, 128);
+  SLA_LIN_CASE(f16_tag, 64);
+#undef SLA_LIN_CASE
+}
+
+extern "C" int sla_linear_fwd(const void* q, const void* k, const void* v, const float* weight, const float* bias,
+                              const void* residual, void* out, int dtype, int fmap, int B, int H, int L, int D,
+                              void* workspace, int64_t workspace_bytes, void* stream) {
+  int rc = validate_linear(dtype, fmap, B, H, L, D);
+  if (rc) return rc;
+  SLA_REQUIRE(q && k && v && weight && bias && out && workspace, SLA_ERR_BAD_ARG, "null pointer");
+  rc = sla_linear_state_fwd(k, v, weight, dtype, fmap, B, H, L, D, workspace, workspace_bytes, stream);
+  if (rc) return rc;
+  return sla_linear_out_fwd(q, bias, residual, out, dtype, fmap, B, H, L, D, workspace, workspace_bytes, stream);
 }

@@ -24,6 +24,32 @@ def linear_fwd(q, k, v, weight, bias, residual, fmap: str):
     return out
 
 
+def linear_state_fwd(k, v, weight, fmap: str):
+    """First half of :func:`linear_fwd`: builds the per-head states from ``k`` and ``v`` on the current
+    stream and returns the workspace that :func:`linear_out_fwd` consumes."""
+    _lib.require_gpu(k, v, weight)
+    B, H, L, D = k.shape
+    dt = _lib.dtype_code(k.dtype)
+    ws = _lib.workspace(_lib.WS_LINEAR_FWD, dt, B, H, L, D, 64, 64, 0, k.device)
+    rc = _lib.load().sla_linear_state_fwd(k.data_ptr(), v.data_ptr(), weight.data_ptr(), dt, _lib.FMAP[fmap], B, H, L, D,
+                                          ws.data_ptr(), ws.numel(), _lib.stream_ptr(k.device))
+    _lib.check(rc)
+    return ws
+
+
+def linear_out_fwd(q, bias, residual, state_ws, fmap: str):
+    """Second half of :func:`linear_fwd`: ``residual + proj(phi(q) state / divisor)``."""
+    _lib.require_gpu(q, bias, state_ws)
+    B, H, L, D = q.shape
+    dt = _lib.dtype_code(q.dtype)
+    out = torch.empty_like(q)
+    rc = _lib.load().sla_linear_out_fwd(q.data_ptr(), bias.data_ptr(), 0 if residual is None else residual.data_ptr(),
+                                        out.data_ptr(), dt, _lib.FMAP[fmap], B, H, L, D, state_ws.data_ptr(),
+                                        state_ws.numel(), _lib.stream_ptr(q.device))
+    _lib.check(rc)
+    return out
+
+
 def linear_bwd(q, k, v, weight, bias, d_out, fmap: str, accumulate_into=None):
     """Gradients of the linear branch.  ``accumulate_into=(dq, dk, dv)`` adds them to existing
     gradient tensors (those of the sparse branch) instead of allocating new ones."""

@@ -6,7 +6,7 @@ import torch
 import torch.nn as nn
 
 from .block_map import get_block_map
-from .linear import linear_bwd, linear_fwd
+from .linear import linear_bwd, linear_out_fwd, linear_state_fwd
 from .sparse_attn import sparse_attn_bwd, sparse_attn_fwd
 
 FEATURE_MAPS = ("elu", "relu", "softmax")
@@ -20,16 +20,16 @@ class _sla_core(torch.autograd.Function):
     """
 
     @staticmethod
-    def forward(ctx, q, k, v, weight, bias, sparse_map, lut, topk, BLKQ, BLKK, fmap):
+    def forward(ctx, q, k, v, weight, bias, sparse_map, lut, topk, BLKQ, BLKK, fmap, state):
         assert q.is_contiguous() and k.is_contiguous() and v.is_contiguous()
         assert sparse_map.is_contiguous() and lut.is_contiguous()
         assert BLKQ == 64 or BLKQ == 128
         assert BLKK == 64
         qk_scale = q.shape[-1] ** -0.5
-        weight = weight.contiguous()
         bias = bias.contiguous()
         o_s, lse = sparse_attn_fwd(q, k, v, lut, topk, BLKQ, BLKK, qk_scale)
-        out = linear_fwd(q, k, v, weight, bias, o_s, fmap)
+        state_ws = state.join()
+        out = linear_out_fwd(q, bias, o_s, state_ws, fmap)
         ctx.save_for_backward(q, k, v, weight, bias, sparse_map, lut, lse, o_s)
         ctx.cfg = (topk, BLKQ, BLKK, fmap, qk_scale)
         return out
@@ -41,7 +41,39 @@ class _sla_core(torch.autograd.Function):
         d_out = d_out.contiguous()
         dq, dk, dv = sparse_attn_bwd(q, k, v, o_s, d_out, lse, sparse_map, lut, topk, BLKQ, BLKK, qk_scale)
         _, _, _, dw, db = linear_bwd(q, k, v, weight, bias, d_out, fmap, accumulate_into=(dq, dk, dv))
-        return dq, dk, dv, dw, db, None, None, None, None, None, None
+        return dq, dk, dv, dw, db, None, None, None, None, None, None, None
+
+
+class _StateBuild:
+    """The k/v-only half of the linear branch, started on a side stream so that it runs beside the mask
+    builder (both are short memory-bound kernels; neither fills the device on its own).  ``join`` makes
+    the calling stream wait for it and hands over the workspace it filled."""
+
+    _side = {}
+
+    def __init__(self, k, v, weight, fmap):
+        dev = k.device
+        cur = torch.cuda.current_stream(dev)
+        if torch.cuda.is_current_stream_capturing():
+            side = None          # inside a graph capture the work stays on the capturing stream
+        else:
+            side = self._side.get(dev.index)
+            if side is None:
+                side = self._side[dev.index] = torch.cuda.Stream(device=dev)
+        self.side = side
+        if side is None:
+            self.ws = linear_state_fwd(k, v, weight, fmap)
+            return
+        side.wait_stream(cur)    # k, v and the weight were produced on the calling stream
+        with torch.cuda.stream(side):
+            self.ws = linear_state_fwd(k, v, weight, fmap)
+
+    def join(self):
+        if self.side is not None:
+            torch.cuda.current_stream(self.ws.device).wait_stream(self.side)
+            # the workspace was allocated under the side stream; it is consumed on the calling one
+            self.ws.record_stream(torch.cuda.current_stream(self.ws.device))
+        return self.ws
 
 
 class SparseLinearAttention(nn.Module):
@@ -86,14 +118,18 @@ class SparseLinearAttention(nn.Module):
         k = k.contiguous()
         v = v.contiguous()
 
+        qc = q.to(self.dtype)
+        kc = k.to(self.dtype)
+        vc = v.to(self.dtype)
+        weight = self.proj_l.weight.contiguous()
+        with torch.no_grad():
+            state = _StateBuild(kc, vc, weight, self.feature_map)
+
         # the mask is built from the inputs in their own dtype (reference core.py:83)
         sparse_map, lut, real_topk = get_block_map(q, k, topk_ratio=self.topk, BLKQ=self.BLKQ, BLKK=self.BLKK)
 
-        q = q.to(self.dtype)
-        k = k.to(self.dtype)
-        v = v.to(self.dtype)
-        o = _sla_core.apply(q, k, v, self.proj_l.weight, self.proj_l.bias, sparse_map, lut, real_topk, self.BLKQ,
-                            self.BLKK, self.feature_map)
+        o = _sla_core.apply(qc, kc, vc, weight, self.proj_l.bias, sparse_map, lut, real_topk, self.BLKQ,
+                            self.BLKK, self.feature_map, state)
         o = o.to(dtype)
 
         if return_sparsity:

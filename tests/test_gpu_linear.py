@@ -5,7 +5,7 @@ import torch
 from conftest import cos_sim, max_abs
 from oracle import sla_oracle as O
 from sla_amd.inputs import CONFIGS, make_inputs, make_proj
-from sla_amd.linear import linear_fwd
+from sla_amd.linear import linear_fwd, linear_out_fwd, linear_state_fwd
 
 pytestmark = pytest.mark.gpu
 
@@ -81,3 +81,19 @@ def test_linear_branch_backward_vs_autograd_oracle(dev, fmap, L, D):
         scale = max(1.0, float(r.abs().max()))          # dW/db are sums over B*H*L rows
         assert max_abs(a, r) <= TOL_ABS * scale, (name, max_abs(a, r), scale)
         assert cos_sim(a, r) >= TOL_COS, (name, cos_sim(a, r))
+
+
+def test_split_entry_points_equal_the_fused_one(dev):
+    """state half on a side stream + output half on the main one == sla_linear_fwd, bit for bit."""
+    g = torch.Generator().manual_seed(7)
+    q, k, v, res = (torch.randn(1, 3, 700, 128, generator=g).to(torch.bfloat16).to(dev) for _ in range(4))
+    w, b = (t.to(dev) for t in make_proj(128))
+    ref = linear_fwd(q, k, v, w, b, res, "elu")
+    side = torch.cuda.Stream(device=dev)
+    side.wait_stream(torch.cuda.current_stream(dev))
+    with torch.cuda.stream(side):
+        ws = linear_state_fwd(k, v, w, "elu")
+    torch.cuda.current_stream(dev).wait_stream(side)
+    ws.record_stream(torch.cuda.current_stream(dev))
+    out = linear_out_fwd(q, b, res, ws, "elu")
+    assert torch.equal(out, ref)
