@@ -37,6 +37,7 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
 typedef __attribute__((__vector_size__(2 * sizeof(int)))) int i32x2_t;
 typedef __attribute__((__vector_size__(4 * sizeof(int)))) int i32x4_t;
+typedef __attribute__((__vector_size__(8 * sizeof(int)))) int i32x8_t;
 typedef __attribute__((__vector_size__(16 * sizeof(int)))) int i32x16_t;
 
 struct bf16_tag {};

@@ -108,12 +108,21 @@ __global__ __launch_bounds__(256) void v_amax_partial_kernel(const uint16_t* __r
   }
 }
 
-__global__ void v_scale_kernel(const float* __restrict__ part, float* __restrict__ v_scale, int nchunk, int D) {
-  const int bh = blockIdx.x, d = threadIdx.x;
-  if (d >= D) return;
+// grid (BH), 1024 threads: thread (cg, d) = (tid / D, tid % D) takes the maximum over chunks cg, cg + 1024/D, ...;
+// the 1024/D partial maxima per column meet in LDS.
+__global__ __launch_bounds__(1024) void v_scale_kernel(const float* __restrict__ part, float* __restrict__ v_scale, int nchunk,
+                                                      int D) {
+  __shared__ float sm[1024];
+  const int bh = blockIdx.x, tid = threadIdx.x;
+  const int d = tid % D, cg = tid / D, ncg = 1024 / D;
   float a = 0.f;
-  for (int c = 0; c < nchunk; ++c) a = fmaxf(a, part[((size_t)bh * nchunk + c) * D + d]);
-  v_scale[(size_t)bh * D + d] = fmaxf(a, 1e-30f) / 448.0f;
+  for (int c = cg; c < nchunk; c += ncg) a = fmaxf(a, part[((size_t)bh * nchunk + c) * D + d]);
+  sm[tid] = a;
+  __syncthreads();
+  if (tid < D) {
+    for (int j = 1; j < ncg; ++j) a = fmaxf(a, sm[j * D + tid]);
+    v_scale[(size_t)bh * D + tid] = fmaxf(a, 1e-30f) / 448.0f;
+  }
 }
 
 static __device__ __forceinline__ uint32_t cvt4_fp8(float a, float b, float c, float d) {
@@ -145,12 +154,22 @@ __global__ __launch_bounds__(256) void v_quant_fp8_kernel(const uint16_t* __rest
 // ---- quantised block-sparse attention ----------------------------------------------------------
 typedef __attribute__((address_space(3))) i32x2_t lds_i32x2_t;
 
+// One workgroup per query block of BLKQ rows, one wave per 32 queries, two waves per SIMD.
+// S^T = K8 Q8^T with v_mfma_i32_32x32x32_i8 (exact), dequantised by sq*sk*scale*log2(e) inside the exponent's
+// FMA.  Both 32-key halves of a tile are exponentiated against one reference maximum and packed to e4m3: the
+// 32 probabilities a lane then holds are, as they stand, its B operand of ONE v_mfma_f32_32x32x64_f8f6f4 per
+// 32 output channels (O^T += V8^T P^T, contraction over all 64 keys of the tile); V^T fragments come from the
+// row-major V tile with the transposing 8-bit LDS read, whose row addresses follow the accumulator's key order.
+// The reference maximum only moves when a tile's maximum exceeds it by more than TAU = 2 (log2 units), so
+// probabilities are at most 4; they are scaled by 112 = 448/4 to use the e4m3 range.
+// K/V tiles: global -> registers -> LDS, double-buffered in LDS: the next tile is in flight during the whole
+// current one and there is one barrier per tile.
 template <typename OutTag, int D, int BLKQ>
-__global__ __launch_bounds__(BLKQ * 2) void sage_fwd_kernel(const int8_t* __restrict__ q8, const float* __restrict__ q_scale,
-                                                            const int8_t* __restrict__ k8, const float* __restrict__ k_scale,
-                                                            const uint8_t* __restrict__ v8, const float* __restrict__ v_scale,
-                                                            const void* __restrict__ lut, int lut64, uint16_t* __restrict__ o,
-                                                            int L, int Mblk, int Nblk, int topk, float scale_log2e, int total) {
+__global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))) void sage_fwd_kernel(
+    const int8_t* __restrict__ q8, const float* __restrict__ q_scale, const int8_t* __restrict__ k8,
+    const float* __restrict__ k_scale, const uint8_t* __restrict__ v8, const float* __restrict__ v_scale,
+    const void* __restrict__ lut, int lut64, uint16_t* __restrict__ o, int L, int Mblk, int Nblk, int topk,
+    float scale_log2e, int total) {
   using EO = Elem<OutTag>;
   constexpr int BLKK = 64;
   constexpr int NT = BLKQ * 2;
@@ -159,9 +178,12 @@ __global__ __launch_bounds__(BLKQ * 2) void sage_fwd_kernel(const int8_t* __rest
   constexpr int STR = D + 16;               // bytes per LDS row
   constexpr int CPR = D / 16;               // 16-byte chunks per row
   constexpr int NLD = (BLKK * CPR + NT - 1) / NT;
+  constexpr float TAU = 2.0f;
+  // probabilities are scaled by 112 = 448 / 2^TAU, applied as an offset of the exponent
+  constexpr float LOG2_P_SCALE = 6.807354922057604f;
 
-  __shared__ __attribute__((aligned(16))) uint8_t sK[BLKK * STR];
-  __shared__ __attribute__((aligned(16))) uint8_t sV[BLKK * STR];
+  __shared__ __attribute__((aligned(16))) uint8_t sK[2][BLKK * STR];
+  __shared__ __attribute__((aligned(16))) uint8_t sV[2][BLKK * STR];
 
   const int logical = xcd_remap(blockIdx.x, gridDim.x, total);
   if (logical < 0) return;
@@ -171,13 +193,15 @@ __global__ __launch_bounds__(BLKQ * 2) void sage_fwd_kernel(const int8_t* __rest
   const int g = lane >> 5, r = lane & 31;
 
   const size_t head_off = (size_t)bh * L * D;
+  const uint32_t head_bytes = (uint32_t)L * D;
+  const __amdgpu_buffer_rsrc_t qh = make_rsrc(q8 + head_off, head_bytes);
+  const __amdgpu_buffer_rsrc_t kh = make_rsrc(k8 + head_off, head_bytes);
+  const __amdgpu_buffer_rsrc_t vh = make_rsrc(v8 + head_off, head_bytes);
   const int qrow = mb * BLKQ + wave * 32 + r;
   i32x4_t qf[QC];
 #pragma unroll
-  for (int c = 0; c < QC; ++c) {
-    qf[c] = i32x4_t{0, 0, 0, 0};
-    if (qrow < L) qf[c] = *reinterpret_cast<const i32x4_t*>(q8 + head_off + (size_t)qrow * D + 32 * c + 16 * g);
-  }
+  for (int c = 0; c < QC; ++c)
+    qf[c] = __builtin_bit_cast(i32x4_t, buf_load_b128(qh, (uint32_t)qrow * D + 32 * c + 16 * g));   // rows past L: 0
   const float qs = q_scale[(size_t)bh * Mblk + mb] * scale_log2e;
   const float* ksc = k_scale + (size_t)bh * Nblk;
 
@@ -186,29 +210,26 @@ __global__ __launch_bounds__(BLKQ * 2) void sage_fwd_kernel(const int8_t* __rest
     return lut64 ? (int)reinterpret_cast<const long long*>(lut)[lut_row + i]
                  : reinterpret_cast<const int*>(lut)[lut_row + i];
   };
-  i32x4_t kreg[NLD], vreg[NLD];
+  i16x8_t kreg[NLD], vreg[NLD];
   auto load_tile = [&](int nb) {
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
       const int idx = tid + i * NT;
       const int row = idx / CPR, col = (idx % CPR) * 16;
-      const int grow = nb * BLKK + row;
-      kreg[i] = i32x4_t{0, 0, 0, 0};
-      vreg[i] = i32x4_t{0, 0, 0, 0};
-      if (idx < BLKK * CPR && grow < L) {
-        kreg[i] = *reinterpret_cast<const i32x4_t*>(k8 + head_off + (size_t)grow * D + col);
-        vreg[i] = *reinterpret_cast<const i32x4_t*>(v8 + head_off + (size_t)grow * D + col);
-      }
+      // chunks past the tile (when the tile does not divide among the threads) and rows past L read as zero
+      const uint32_t off = idx < BLKK * CPR ? (uint32_t)(nb * BLKK + row) * D + col : 0xfffffff0u;
+      kreg[i] = buf_load_b128(kh, off);
+      vreg[i] = buf_load_b128(vh, off);
     }
   };
-  auto store_tile = [&]() {
+  auto store_tile = [&](int stage) {
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
       const int idx = tid + i * NT;
       if (idx < BLKK * CPR) {
         const int row = idx / CPR, col = (idx % CPR) * 16;
-        *reinterpret_cast<i32x4_t*>(&sK[row * STR + col]) = kreg[i];
-        *reinterpret_cast<i32x4_t*>(&sV[row * STR + col]) = vreg[i];
+        *reinterpret_cast<i16x8_t*>(&sK[stage][row * STR + col]) = kreg[i];
+        *reinterpret_cast<i16x8_t*>(&sV[stage][row * STR + col]) = vreg[i];
       }
     }
   };
@@ -218,7 +239,16 @@ __global__ __launch_bounds__(BLKQ * 2) void sage_fwd_kernel(const int8_t* __rest
   for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
     for (int i = 0; i < 16; ++i) oacc[dt][i] = 0.f;
-  float m_run = -INFINITY, l_run = 0.f;
+  float m_used = -INFINITY;   // reference maximum (log2 units)
+  // Row sums of the e4m3 probabilities come from the matrix core as well: an A operand of ones makes every
+  // row of this accumulator the sum over all 64 keys of a tile, so each lane holds l of its query column
+  // (numerator and denominator then see the same rounded probabilities, and no vector-ALU adds are spent).
+  f32x16_t lacc;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) lacc[i] = 0.f;
+  i32x8_t ones;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) ones[i] = 0x38383838;   // e4m3 1.0 in every byte
 
   // transposed 8-bit read: lane i of a 16-lane group passes the address of (row i/2, 8 bytes at
   // column 8*(i%2)) and receives column i of the 8x16 tile.  Row i/2 is mapped to the key that
@@ -229,77 +259,101 @@ __global__ __launch_bounds__(BLKQ * 2) void sage_fwd_kernel(const int8_t* __rest
   const int tr_col = 16 * ((lane >> 4) & 1) + 8 * (li & 1);
 
   int nb = topk > 0 ? lut_at(0) : 0;
-  if (topk > 0) load_tile(nb);
+  int nb_next = topk > 1 ? lut_at(1) : 0;
+  if (topk > 0) {
+    load_tile(nb);
+    store_tile(0);
+  }
+  __syncthreads();
   for (int it = 0; it < topk; ++it) {
-    __syncthreads();
-    store_tile();
-    __syncthreads();
+    const int cur = it & 1;
     const int kv_valid = L - nb * BLKK;
-    const float sc = qs * ksc[nb];
-    if (it + 1 < topk) {
-      nb = lut_at(it + 1);
+    // an all-zero block has scale 1e-30/127; the floor keeps -inf * sc = -inf (never NaN) for masked rows
+    const float sc = fmaxf(qs * ksc[nb], 1e-37f);
+    const bool more = it + 1 < topk;
+    if (more) {
+      nb = nb_next;
+      nb_next = it + 2 < topk ? lut_at(it + 2) : 0;
       load_tile(nb);
+    }
+    // ---- S^T, both halves ----
+    i32x16_t acc[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[t][i] = 0;
+#pragma unroll
+      for (int c = 0; c < QC; ++c) {
+        const i32x4_t a = *reinterpret_cast<const i32x4_t*>(&sK[cur][(32 * t + r) * STR + 32 * c + 16 * g]);
+        acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, qf[c], acc[t], 0, 0, 0);
+      }
     }
     float s[2][16];
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      i32x16_t acc;
+    for (int t = 0; t < 2; ++t)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) acc[i] = 0;
+      for (int i = 0; i < 16; ++i) s[t][i] = (float)acc[t][i];
+    if (kv_valid < BLKK) {                 // ragged last key block: missing rows take no part
+      const int lim = kv_valid - 4 * g;    // key index of register i is 32t + 8(i/4) + i%4 + 4g
 #pragma unroll
-      for (int c = 0; c < QC; ++c) {
-        const i32x4_t a = *reinterpret_cast<const i32x4_t*>(&sK[(32 * t + r) * STR + 32 * c + 16 * g]);
-        acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, qf[c], acc, 0, 0, 0);
-      }
+      for (int t = 0; t < 2; ++t)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int key = 32 * t + 8 * (i >> 2) + 4 * g + (i & 3);
-        s[t][i] = key < kv_valid ? (float)acc[i] * sc : -INFINITY;
-      }
+        for (int i = 0; i < 16; ++i)
+          if (32 * t + 8 * (i >> 2) + (i & 3) >= lim) s[t][i] = -INFINITY;
     }
+    // raw maximum of this lane's 32 scores (sc >= 0, so the maximum commutes with the scaling)
     float mx = s[0][0];
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[t][i]);
-    mx = fmaxf(mx, __shfl_xor(mx, 32));
-    const float m_new = fmaxf(m_run, mx);
-    const float alpha = fast_exp2(m_run - m_new);
-    float psum = 0.f;
+    if (__any(mx * sc > m_used + TAU)) {   // rare: move the reference and rescale what is accumulated
+      float m_new = fmaxf(mx, __shfl_xor(mx, 32)) * sc;
+      m_new = fmaxf(m_used, m_new);
+      const float f = fast_exp2(m_used - m_new);     // 0 on the first tile
+      m_used = m_new;
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const float p = fast_exp2(s[t][i] - m_new);
-        psum += p;
-        s[t][i] = p * 448.0f;
-      }
-    l_run = l_run * alpha + psum;
-    m_run = m_new;
-    if (__any(alpha != 1.0f)) {
+      for (int i = 0; i < 16; ++i) lacc[i] *= f;
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) oacc[dt][i] *= alpha;
+        for (int i = 0; i < 16; ++i) oacc[dt][i] *= f;
     }
+    // P_SCALE * p = exp2(s*sc - (m_used - log2 P_SCALE)); -inf scores give exactly 0
+    const float m_off = m_used - LOG2_P_SCALE;
+    i32x8_t pb;
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
-      for (int c2 = 0; c2 < 2; ++c2) {
-        i32x2_t pw;
-        pw[0] = (int)cvt4_fp8(s[t][8 * c2 + 0], s[t][8 * c2 + 1], s[t][8 * c2 + 2], s[t][8 * c2 + 3]);
-        pw[1] = (int)cvt4_fp8(s[t][8 * c2 + 4], s[t][8 * c2 + 5], s[t][8 * c2 + 6], s[t][8 * c2 + 7]);
-        const long pb = __builtin_bit_cast(long, pw);
-        const int key = 32 * t + 16 * c2 + tr_key;
+      for (int i4 = 0; i4 < 4; ++i4) {
+        float pv[4];
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-          const i32x2_t a = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_i32x2_t*)&sV[key * STR + 32 * dt + tr_col]);
-          oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(__builtin_bit_cast(long, a), pb, oacc[dt], 0, 0, 0);
+        for (int j = 0; j < 4; ++j) {
+          pv[j] = fast_exp2(__builtin_fmaf(s[t][4 * i4 + j], sc, -m_off));
         }
+        pb[4 * t + i4] = (int)cvt4_fp8(pv[0], pv[1], pv[2], pv[3]);
       }
+    lacc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pb, lacc, 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
+    // ---- O^T += V8^T P^T: one 64-key product per 32 output channels ----
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      i32x8_t a;
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int c2 = 0; c2 < 2; ++c2) {
+          const int key = 32 * t + 16 * c2 + tr_key;
+          const i32x2_t x = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_i32x2_t*)&sV[cur][key * STR + 32 * dt + tr_col]);
+          a[4 * t + 2 * c2] = x[0];
+          a[4 * t + 2 * c2 + 1] = x[1];
+        }
+      // formats 0/0 = e4m3 for both operands, block scales 2^0
+      oacc[dt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, pb, oacc[dt], 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
+    }
+    if (more) store_tile(cur ^ 1);
+    __syncthreads();                       // next tile visible; this one fully consumed
   }
-  const float l_tot = l_run + __shfl_xor(l_run, 32);
-  const float inv = 1.0f / (448.0f * l_tot);
+  const float inv = 1.0f / lacc[0];        // P_SCALE cancels: numerator and l carry the same factor
   if (qrow < L) {
     uint16_t* orow = o + head_off + (size_t)qrow * D;
     const float* vs = v_scale + (size_t)bh * D;
@@ -364,7 +418,7 @@ static int quant_v_impl(const void* v, int BH, int L, uint8_t* v8, float* vs, ch
   float* part = (float*)(ws + w.v_part);
   hipLaunchKernelGGL((v_amax_partial_kernel<Tag, D>), dim3(w.nchunk_v, BH), dim3(256), 0, st, (const uint16_t*)v, part, L,
                      w.rows_per_chunk_v);
-  hipLaunchKernelGGL(v_scale_kernel, dim3(BH), dim3(D), 0, st, part, vs, w.nchunk_v, D);
+  hipLaunchKernelGGL(v_scale_kernel, dim3(BH), dim3(1024), 0, st, part, vs, w.nchunk_v, D);
   constexpr int RPP = 256 / (D / 8);
   hipLaunchKernelGGL((v_quant_fp8_kernel<Tag, D>), dim3(cdiv(L, RPP), BH), dim3(256), 0, st, (const uint16_t*)v, vs, v8, L);
   return check_launch("sage_quant_v");

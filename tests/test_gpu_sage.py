@@ -44,8 +44,12 @@ def test_attention_vs_fp32_and_vs_quantised_oracle(dev, L, D, ratio):
     v8, vs = quant_v(v.to(dev))
     o = sage_attn_fwd(q8, qs, k8, ks, v8, vs, lut.to(dev), T, torch.bfloat16).cpu()
     assert cos_sim(o, ref) >= TOL_COS
-    assert cos_sim(o, ref_q) >= 0.9995          # same quantised arithmetic, only summation order differs
-    assert float((o.float() - ref_q).abs().max()) <= 2e-2
+    # Same quantised scheme as the oracle.  The kernel rounds P to e4m3 against a reference maximum that may
+    # lag the running maximum by up to 2 (log2 units) and uses 448/4 as P scale; the oracle rounds against the
+    # running maximum with scale 448: equal up to e4m3 rounding of P at slightly different points.
+    assert cos_sim(o, ref_q) >= 0.9995
+    assert float((o.float() - ref_q).abs().max()) <= 3e-2
+    assert float((o.float() - ref).abs().max()) <= float((ref_q - ref).abs().max()) * 1.5 + 5e-3
 
 
 def test_full_selection_vs_sdpa(dev):
