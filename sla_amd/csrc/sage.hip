@@ -182,8 +182,8 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
   // probabilities are scaled by 112 = 448 / 2^TAU, applied as an offset of the exponent
   constexpr float LOG2_P_SCALE = 6.807354922057604f;
 
-  __shared__ __attribute__((aligned(16))) uint8_t sK[2][BLKK * STR];
-  __shared__ __attribute__((aligned(16))) uint8_t sV[2][BLKK * STR];
+  __shared__ __attribute__((aligned(16))) uint8_t sK[2][BLKK * STR];   // K of tile i lives in slot i % 2
+  __shared__ __attribute__((aligned(16))) uint8_t sV[3][BLKK * STR];   // V of tile i lives in slot i % 3
 
   const int logical = xcd_remap(blockIdx.x, gridDim.x, total);
   if (logical < 0) return;
@@ -222,14 +222,14 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
       vreg[i] = buf_load_b128(vh, off);
     }
   };
-  auto store_tile = [&](int stage) {
+  auto store_tile = [&](int kslot, int vslot) {
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
       const int idx = tid + i * NT;
       if (idx < BLKK * CPR) {
         const int row = idx / CPR, col = (idx % CPR) * 16;
-        *reinterpret_cast<i16x8_t*>(&sK[stage][row * STR + col]) = kreg[i];
-        *reinterpret_cast<i16x8_t*>(&sV[stage][row * STR + col]) = vreg[i];
+        *reinterpret_cast<i16x8_t*>(&sK[kslot][row * STR + col]) = kreg[i];
+        *reinterpret_cast<i16x8_t*>(&sV[vslot][row * STR + col]) = vreg[i];
       }
     }
   };
@@ -258,36 +258,22 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
   const int tr_key = 8 * (slot >> 2) + 4 * g + (slot & 3);
   const int tr_col = 16 * ((lane >> 4) & 1) + 8 * (li & 1);
 
-  int nb = topk > 0 ? lut_at(0) : 0;
-  int nb_next = topk > 1 ? lut_at(1) : 0;
-  if (topk > 0) {
-    load_tile(nb);
-    store_tile(0);
-  }
-  __syncthreads();
-  for (int it = 0; it < topk; ++it) {
-    const int cur = it & 1;
-    const int kv_valid = L - nb * BLKK;
-    // an all-zero block has scale 1e-30/127; the floor keeps -inf * sc = -inf (never NaN) for masked rows
-    const float sc = fmaxf(qs * ksc[nb], 1e-37f);
-    const bool more = it + 1 < topk;
-    if (more) {
-      nb = nb_next;
-      nb_next = it + 2 < topk ? lut_at(it + 2) : 0;
-      load_tile(nb);
-    }
-    // ---- S^T, both halves ----
-    i32x16_t acc[2];
+  // S^T of one tile: raw int32 products of both 32-key halves
+  auto scores = [&](int kslot, i32x16_t (&acc)[2]) {
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[t][i] = 0;
 #pragma unroll
       for (int c = 0; c < QC; ++c) {
-        const i32x4_t a = *reinterpret_cast<const i32x4_t*>(&sK[cur][(32 * t + r) * STR + 32 * c + 16 * g]);
+        const i32x4_t a = *reinterpret_cast<const i32x4_t*>(&sK[kslot][(32 * t + r) * STR + 32 * c + 16 * g]);
         acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, qf[c], acc[t], 0, 0, 0);
       }
     }
+  };
+  // softmax numerators of one tile (scores acc, dequantisation factor sc, kv_valid existing key rows),
+  // packed to e4m3 in the B-operand order of the 64-key product
+  auto probabilities = [&](const i32x16_t (&acc)[2], float sc, int kv_valid) -> i32x8_t {
     float s[2][16];
 #pragma unroll
     for (int t = 0; t < 2; ++t)
@@ -301,7 +287,7 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
         for (int i = 0; i < 16; ++i)
           if (32 * t + 8 * (i >> 2) + (i & 3) >= lim) s[t][i] = -INFINITY;
     }
-    // raw maximum of this lane's 32 scores (sc >= 0, so the maximum commutes with the scaling)
+    // raw maximum of this lane's 32 scores (sc > 0, so the maximum commutes with the scaling)
     float mx = s[0][0];
 #pragma unroll
     for (int t = 0; t < 2; ++t)
@@ -319,7 +305,7 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
 #pragma unroll
         for (int i = 0; i < 16; ++i) oacc[dt][i] *= f;
     }
-    // P_SCALE * p = exp2(s*sc - (m_used - log2 P_SCALE)); -inf scores give exactly 0
+    // 112 p = exp2(s*sc - (m_used - log2 112)); -inf scores give exactly 0
     const float m_off = m_used - LOG2_P_SCALE;
     i32x8_t pb;
 #pragma unroll
@@ -328,13 +314,15 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
       for (int i4 = 0; i4 < 4; ++i4) {
         float pv[4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          pv[j] = fast_exp2(__builtin_fmaf(s[t][4 * i4 + j], sc, -m_off));
-        }
+        for (int j = 0; j < 4; ++j) pv[j] = fast_exp2(__builtin_fmaf(s[t][4 * i4 + j], sc, -m_off));
         pb[4 * t + i4] = (int)cvt4_fp8(pv[0], pv[1], pv[2], pv[3]);
       }
+    return pb;
+  };
+  // l += sum_keys P ; O^T += V8^T P^T: one 64-key product per 32 output channels
+  auto accumulate = [&](int vslot, const i32x8_t& pb) {
+    // formats 0/0 = e4m3 for both operands, block scales 2^0
     lacc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pb, lacc, 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
-    // ---- O^T += V8^T P^T: one 64-key product per 32 output channels ----
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
       i32x8_t a;
@@ -343,15 +331,62 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
 #pragma unroll
         for (int c2 = 0; c2 < 2; ++c2) {
           const int key = 32 * t + 16 * c2 + tr_key;
-          const i32x2_t x = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_i32x2_t*)&sV[cur][key * STR + 32 * dt + tr_col]);
+          const i32x2_t x = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_i32x2_t*)&sV[vslot][key * STR + 32 * dt + tr_col]);
           a[4 * t + 2 * c2] = x[0];
           a[4 * t + 2 * c2 + 1] = x[1];
         }
-      // formats 0/0 = e4m3 for both operands, block scales 2^0
       oacc[dt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, pb, oacc[dt], 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
     }
-    if (more) store_tile(cur ^ 1);
-    __syncthreads();                       // next tile visible; this one fully consumed
+  };
+
+  // Software pipeline over the selected tiles: step i issues the int8 products of tile i, then does the
+  // exponentials of tile i-1 on the vector ALU while the matrix core works, then issues the fp8 products
+  // of tile i-1.  Tile i+1 is in flight from global memory during the whole step.
+  int nb = topk > 0 ? lut_at(0) : 0;
+  int nb_next = topk > 1 ? lut_at(1) : 0;
+  if (topk > 0) {
+    load_tile(nb);
+    store_tile(0, 0);
+  }
+  __syncthreads();
+  i32x16_t acc_a[2], acc_b[2];              // scores of even / odd steps (ping-pong, no copies)
+  float sc_prev = 0.f;
+  int valid_prev = BLKK;
+  int vslot_prev = 0, vslot = 0;
+  auto step = [&](int it, i32x16_t (&acc)[2], const i32x16_t (&acc_prev)[2]) {
+    const int kv_valid = L - nb * BLKK;
+    // an all-zero block has scale 1e-30/127; the floor keeps -inf * sc = -inf (never NaN) for masked rows
+    const float sc = fmaxf(qs * ksc[nb], 1e-37f);
+    const bool more = it + 1 < topk;
+    if (more) {
+      nb = nb_next;
+      nb_next = it + 2 < topk ? lut_at(it + 2) : 0;
+      load_tile(nb);
+    }
+    scores(it & 1, acc);
+    if (it > 0) {
+      const i32x8_t pb = probabilities(acc_prev, sc_prev, valid_prev);
+      accumulate(vslot_prev, pb);
+    }
+    sc_prev = sc;
+    valid_prev = kv_valid;
+    vslot_prev = vslot;
+    vslot = vslot == 2 ? 0 : vslot + 1;
+    if (more) store_tile((it + 1) & 1, vslot);
+    __syncthreads();                       // next tile visible; K of this step and V of the previous one consumed
+  };
+  int it = 0;
+  for (; it + 1 < topk; it += 2) {
+    step(it, acc_a, acc_b);
+    step(it + 1, acc_b, acc_a);
+  }
+  if (it < topk) {                         // odd count: one more step, its scores land in acc_a
+    step(it, acc_a, acc_b);
+    const i32x8_t pb = probabilities(acc_a, sc_prev, valid_prev);
+    accumulate(vslot_prev, pb);
+  } else if (topk > 0) {
+    const i32x8_t pb = probabilities(acc_b, sc_prev, valid_prev);
+    accumulate(vslot_prev, pb);
   }
   const float inv = 1.0f / lacc[0];        // P_SCALE cancels: numerator and l carry the same factor
   if (qrow < L) {
