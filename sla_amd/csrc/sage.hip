@@ -7,8 +7,8 @@
 //   q_int8 = rint(q / sq), sq = max|q| / 127 over each block of BLKQ rows;
 //   k_int8 = rint((k - mean_L k) / sk), sk per block of BLKK rows;
 //   v_fp8  = e4m3(v / sv), sv[d] = max_L |v[:, d]| / 448;
-//   S = (q_int8 . k_int8) * sq * sk * scale ; P = softmax over the selected blocks ;
-//   O = (e4m3(448 P) . v_fp8) * sv / (448 l).
+//   S = (q_int8 . k_int8) * sq * sk * scale ; P = softmax numerators over the selected blocks ;
+//   O = (e4m3(c P) . v_fp8) * sv / sum(e4m3(c P)), c = 112 with P <= 4 (reference maximum lagging by <= 2).
 // The look-up table of the bf16 path is used as is (no delta encoding is needed here).
 #include "common.h"
 
