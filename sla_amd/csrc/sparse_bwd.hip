@@ -189,7 +189,6 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
   }
   __syncthreads();
   for (int it = 0; it < topk; ++it) {
-    const int kv_valid = L - nb * BLKK;
     const bool more = it + 1 < topk;
     if (more) {
       nb = nb_next;
@@ -211,12 +210,11 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
         const i16x8_t b = *reinterpret_cast<const i16x8_t*>(&sV[(32 * t + r) * VSTR + 16 * c + 8 * g]);
         dp = E::mfma32(b, dof[c], dp);
       }
-      // dS^T = P^T * (dP^T - delta), zero on key rows past L
-      const int lim = kv_valid - 4 * g;      // key index of register i is 32t + 8(i/4) + i%4 + 4g
+      // dS^T = P^T * (dP^T - delta).  Key rows past L need no masking: their K rows are zero in LDS, so
+      // whatever (finite) dS they get is multiplied by zero in dQ^T += K^T dS^T.
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        float p = fast_exp2(__builtin_fmaf(s[i], c_log2e, -lse_q));
-        if (32 * t + 8 * (i >> 2) + (i & 3) >= lim) p = 0.f;
+        const float p = fast_exp2(__builtin_fmaf(s[i], c_log2e, -lse_q));
         s[i] = p * (dp[i] - delta_q);
       }
 #pragma unroll
@@ -390,8 +388,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int i = 4 * i4 + j;
-        float p = fast_exp2(__builtin_fmaf(s[i], c_log2e, -l4[j]));
-        if (!kok) p = 0.f;
+        // (a key row past L only ever feeds its own, never stored, column of dK^T / dV^T: no masking needed)
+        const float p = fast_exp2(__builtin_fmaf(s[i], c_log2e, -l4[j]));
         s[i] = p;
         dp[i] = p * (dp[i] - d4[j]);
       }
