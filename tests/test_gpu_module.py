@@ -75,3 +75,38 @@ def test_cfg3_three_heads_forward(dev):
     o_ref, *_ = O.sla_forward(d["q"], d["k"], d["v"], w, b, cfg.topk, cfg.feature_map, linear_dtype=torch.float32)
     o = mod(d["q"].to(dev), d["k"].to(dev), d["v"].to(dev)).cpu()
     assert max_abs(o, o_ref) <= TOL_ABS and cos_sim(o, o_ref) >= TOL_COS
+
+
+def test_forward_in_a_hip_graph(dev):
+    """The whole forward (mask builder, attention, linear branch) is capturable: the library allocates
+    nothing, clears nothing with memset nodes, and under capture the module keeps all work on the capturing
+    stream.  Every replay is checked against the eager result, with eager work between the replays."""
+    cfg = CONFIGS["cfg2"]
+    d = make_inputs(cfg, H=2)
+    mod, _, _ = _module(cfg, dev)
+    q, k, v = (d[x].to(dev) for x in "qkv")
+    with torch.no_grad():
+        ref = mod(q, k, v)
+        torch.cuda.synchronize()
+        s = torch.cuda.Stream(device=dev)
+        s.wait_stream(torch.cuda.current_stream(dev))
+        with torch.cuda.stream(s):
+            mod(q, k, v)                      # warm-up on the capture stream
+        torch.cuda.current_stream(dev).wait_stream(s)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            out = mod(q, k, v)
+        for i in range(3):
+            out.zero_()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out, ref), f"replay {i}"
+            assert torch.equal(mod(q, k, v), ref)   # eager work between the replays
+            torch.cuda.synchronize()
+        # new inputs in the captured buffers
+        q2 = torch.roll(q, 3, dims=2)
+        ref2 = mod(q2, k, v)
+        q.copy_(q2)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, ref2)
