@@ -180,6 +180,16 @@ def main():
         except (ImportError, AssertionError, RuntimeError) as e:
             extra["sage_fwd_ms"] = None
             extra["sage_note"] = str(e)[:200]
+        try:
+            cmod = SparseLinearAttention(cfg.D, cfg.topk, cfg.feature_map, cfg.BLKQ, cfg.BLKK,
+                                         linear_mode="complement").to(dev)
+            with torch.no_grad():
+                cmod.proj_l.weight.copy_(w)
+                cmod.proj_l.bias.copy_(b)
+                extra["sla_fwd_complement_mode_ms"] = time_region(torch, lambda: cmod(q, k, v), args.steps, args.warmup)
+        except (AssertionError, RuntimeError, NotImplementedError) as e:
+            extra["sla_fwd_complement_mode_ms"] = None
+            extra["complement_note"] = str(e)[:200]
     if args.pmc_calibration:
         x = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
         y = torch.empty_like(x)

@@ -49,6 +49,7 @@ extern "C" {
 #define SLA_WS_LINEAR_FWD 2
 #define SLA_WS_LINEAR_BWD 3
 #define SLA_WS_SAGE_QUANT 4
+#define SLA_WS_LINEAR_COMPLEMENT 5
 
 int sla_version(void);
 const char* sla_last_error(void);
@@ -106,6 +107,16 @@ int sla_linear_state_fwd(const void* k, const void* v, const float* weight, int 
                          int D, void* workspace, int64_t workspace_bytes, void* stream);
 int sla_linear_out_fwd(const void* q, const float* bias, const void* residual, void* out, int dtype, int fmap, int B,
                        int H, int L, int D, void* workspace, int64_t workspace_bytes, void* stream);
+
+/* Linear branch in "complement" mode (opt-in; forward only): query block i attends linearly only to the key
+ * blocks (of 64 rows) that its look-up row did NOT select; projection, bias and residual as in
+ * sla_linear_fwd.  out = residual + proj(o_l).  lut as produced by sla_block_map_fwd; BLKK must be 64.
+ * The mounted reference has no code for this variant (its README.md:8 names it; core.py:92-96 computes
+ * the global one): the definition is the brute-force one stated in the oracle. */
+int sla_linear_complement_fwd(const void* q, const void* k, const void* v, const void* lut, int lut_elem_bytes,
+                              const float* weight, const float* bias, const void* residual, void* out, int dtype,
+                              int fmap, int B, int H, int L, int D, int BLKQ, int BLKK, int topk, void* workspace,
+                              int64_t workspace_bytes, void* stream);
 
 /* Linear branch backward.  d_out is the gradient of `out` above.  Writes dq, dk, dv in `dtype`
  * (gradients of the linear branch only; the residual's gradient is d_out itself) and the

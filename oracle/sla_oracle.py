@@ -17,6 +17,7 @@ Reference lines followed (paths are inside the reference checkout):
   sparse_attn_bwd          sparse_linear_attention/kernel.py:85-237, 277-320
   feature maps             sparse_linear_attention/core.py:43-60
   calc_linear / proj / sum sparse_linear_attention/core.py:77-105
+  complement linear mode   no reference code (README.md:8 names the variant); brute-force definition
   SageSLA orchestration    SageSLA/core.py:75-163
 
 Two things are fixed here that the reference leaves open, because without them
@@ -343,6 +344,44 @@ def linear_branch(q, k, v, weight, bias, fmap: str, dtype):
     fk = phi(k.to(dtype)).contiguous().to(dtype)
     o_l = calc_linear(fq, fk, v.to(dtype))
     return F.linear(o_l, weight.to(dtype), bias.to(dtype))
+
+
+def linear_branch_complement(q, k, v, lut, weight, bias, fmap: str, BLKQ: int, BLKK: int, dtype=torch.float32):
+    """Linear branch restricted, per query block, to the key blocks it did NOT select, then proj_l.
+
+    This is the formulation of the SLA paper (linear attention over the non-critical blocks); the mounted
+    reference computes the global variant instead (core.py:92-96) and has no code for this one, so the
+    definition here is the brute-force one: for query block i with selected set S_i,
+
+        o_l[rows of i] = phi(Q_i) (sum_{j not in S_i} phi(K_j)^T V_j) / (1e-5 + phi(Q_i) . sum_{j not in S_i} sum_rows phi(K_j))
+
+    evaluated with per-key-block states in fp32.  ``dtype`` is the dtype of phi(q), phi(k), v and of the
+    result; everything in between is fp32 (the kernel rounds its states to ``dtype`` as the global path does).
+    """
+    B, H, L, D = q.shape
+    phi = feature_map(fmap)
+    fq = phi(q.to(dtype)).to(dtype).float()
+    fk = phi(k.to(dtype)).to(dtype).float()
+    vf = v.to(dtype).float()
+    N = (L + BLKK - 1) // BLKK
+    M = (L + BLKQ - 1) // BLKQ
+    pad = N * BLKK - L
+    fkp = F.pad(fk, (0, 0, 0, pad)).view(B, H, N, BLKK, D)      # padded rows are zero: they add nothing
+    vp = F.pad(vf, (0, 0, 0, pad)).view(B, H, N, BLKK, D)
+    h = fkp.transpose(-1, -2) @ vp                               # (B,H,N,D,D)
+    z = fkp.sum(dim=-2)                                          # (B,H,N,D)
+    h_all, z_all = h.sum(dim=2), z.sum(dim=2)
+    out = torch.empty(B, H, L, D, dtype=torch.float32)
+    for b in range(B):
+        for hh in range(H):
+            for i in range(M):
+                sel = lut[b, hh, i].long()
+                hc = h_all[b, hh] - h[b, hh, sel].sum(dim=0)
+                zc = z_all[b, hh] - z[b, hh, sel].sum(dim=0)
+                rows = slice(i * BLKQ, min(L, (i + 1) * BLKQ))
+                fqi = fq[b, hh, rows]
+                out[b, hh, rows] = (fqi @ hc) / (1e-5 + (fqi * zc).sum(dim=-1, keepdim=True))
+    return F.linear(out.to(dtype).float(), weight.to(dtype).float(), bias.to(dtype).float()).to(dtype)
 
 
 def sla_forward(q, k, v, weight, bias, topk_ratio, fmap="softmax", BLKQ=64, BLKK=64,

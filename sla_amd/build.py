@@ -16,7 +16,8 @@ CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIBPATH = os.path.join(LIBDIR, "libsla_hip.so")
 
-SOURCES = ["capi.hip", "block_map.hip", "sparse_fwd.hip", "linear.hip", "linear_bwd.hip", "sparse_bwd.hip", "sage.hip"]
+SOURCES = ["capi.hip", "block_map.hip", "sparse_fwd.hip", "linear.hip", "linear_bwd.hip", "sparse_bwd.hip", "sage.hip",
+           "linear_complement.hip"]
 
 COMMON_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",

@@ -6,9 +6,10 @@ namespace sla {
 
 // ---- kernel 1: partial states -----------------------------------------------------------
 // grid (nsplit, BH), 256 threads.  Thread t moves 16-byte chunk (t%CPR) of rows t/CPR + i*RPP.
-template <typename Tag, int D>
+// OUT16: the D x D partial is written rounded to 16 bit (per-key-block states of the complement mode).
+template <typename Tag, int D, bool OUT16 = false>
 __global__ __launch_bounds__(256) void linear_state_partial_kernel(const uint16_t* __restrict__ k,
-                                                                   const uint16_t* __restrict__ v, float* __restrict__ kv_part,
+                                                                   const uint16_t* __restrict__ v, void* __restrict__ kv_part_,
                                                                    float* __restrict__ z_part, int L, int rows_per_split,
                                                                    int fmap) {
   using E = Elem<Tag>;
@@ -113,7 +114,7 @@ __global__ __launch_bounds__(256) void linear_state_partial_kernel(const uint16_
   }
 
   // partial KV, stored transposed: kv_part[bh][split][d2][d1]
-  float* out = kv_part + ((size_t)bh * nsplit + split) * D * D;
+  const size_t part_off = ((size_t)bh * nsplit + split) * D * D;
 #pragma unroll
   for (int t = 0; t < WPT; ++t) {
     const int tile = wave * WPT + t;
@@ -121,8 +122,16 @@ __global__ __launch_bounds__(256) void linear_state_partial_kernel(const uint16_
     const int d2 = 32 * d2t + (lane & 31);
 #pragma unroll
     for (int i4 = 0; i4 < 4; ++i4) {
-      f32x4_t w = {acc[t][4 * i4], acc[t][4 * i4 + 1], acc[t][4 * i4 + 2], acc[t][4 * i4 + 3]};
-      *reinterpret_cast<f32x4_t*>(out + (size_t)d2 * D + 32 * d1t + 8 * i4 + 4 * g) = w;
+      const size_t o = part_off + (size_t)d2 * D + 32 * d1t + 8 * i4 + 4 * g;
+      if (OUT16) {
+        i32x2_t w;
+        w[0] = (int)E::pack2(acc[t][4 * i4], acc[t][4 * i4 + 1]);
+        w[1] = (int)E::pack2(acc[t][4 * i4 + 2], acc[t][4 * i4 + 3]);
+        *reinterpret_cast<i32x2_t*>(reinterpret_cast<uint16_t*>(kv_part_) + o) = w;
+      } else {
+        f32x4_t w = {acc[t][4 * i4], acc[t][4 * i4 + 1], acc[t][4 * i4 + 2], acc[t][4 * i4 + 3]};
+        *reinterpret_cast<f32x4_t*>(reinterpret_cast<float*>(kv_part_) + o) = w;
+      }
     }
   }
   // partial z: reduce the RPP row groups through LDS

@@ -50,6 +50,27 @@ def linear_out_fwd(q, bias, residual, state_ws, fmap: str):
     return out
 
 
+def linear_complement_fwd(q, k, v, lut, topk, weight, bias, residual, fmap: str, BLKQ: int = 64, BLKK: int = 64):
+    """Linear branch over the key blocks each query block did NOT select, + projection + ``residual``.
+
+    Opt-in variant (the paper's formulation); the reference module computes the global branch
+    (``core.py:92-96``).  Forward only."""
+    _lib.require_gpu(q, k, v, lut, weight, bias)
+    B, H, L, D = q.shape
+    dt = _lib.dtype_code(q.dtype)
+    if lut.dtype not in (torch.int32, torch.int64):
+        raise TypeError(f"lut must be int32 or int64, got {lut.dtype}")
+    ws = _lib.workspace(_lib.WS_LINEAR_COMPLEMENT, dt, B, H, L, D, BLKQ, BLKK, topk, q.device)
+    out = torch.empty_like(q)
+    rc = _lib.load().sla_linear_complement_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), lut.data_ptr(),
+                                               lut.element_size(), weight.data_ptr(), bias.data_ptr(),
+                                               0 if residual is None else residual.data_ptr(), out.data_ptr(), dt,
+                                               _lib.FMAP[fmap], B, H, L, D, BLKQ, BLKK, topk, ws.data_ptr(),
+                                               ws.numel(), _lib.stream_ptr(q.device))
+    _lib.check(rc)
+    return out
+
+
 def linear_bwd(q, k, v, weight, bias, d_out, fmap: str, accumulate_into=None):
     """Gradients of the linear branch.  ``accumulate_into=(dq, dk, dv)`` adds them to existing
     gradient tensors (those of the sparse branch) instead of allocating new ones."""

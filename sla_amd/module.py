@@ -6,7 +6,7 @@ import torch
 import torch.nn as nn
 
 from .block_map import get_block_map
-from .linear import linear_bwd, linear_out_fwd, linear_state_fwd
+from .linear import linear_bwd, linear_complement_fwd, linear_out_fwd, linear_state_fwd
 from .sparse_attn import sparse_attn_bwd, sparse_attn_fwd
 
 FEATURE_MAPS = ("elu", "relu", "softmax")
@@ -78,7 +78,7 @@ class _StateBuild:
 
 class SparseLinearAttention(nn.Module):
     def __init__(self, head_dim, topk, feature_map="softmax", BLKQ=64, BLKK=64, use_bf16=True,
-                 tie_feature_map_qk=True):
+                 tie_feature_map_qk=True, linear_mode="global"):
         r"""
         Args:
             head_dim: dimension of each head.
@@ -89,6 +89,9 @@ class SparseLinearAttention(nn.Module):
             use_bf16: bfloat16 (default) or float16 compute; inputs are converted inside the module.
             tie_feature_map_qk: kept for signature compatibility; q and k always use the same map
                 (as in the reference, core.py:43-60).
+            linear_mode: "global" (default, what the reference computes: the linear branch sees every key)
+                or "complement" (extension: it sees only the key blocks the query block did not select;
+                forward only).
         """
         super().__init__()
         self.dtype = torch.bfloat16 if use_bf16 else torch.float16
@@ -100,6 +103,9 @@ class SparseLinearAttention(nn.Module):
             raise NotImplementedError(f"Not supported feature map {feature_map}.")
         self.feature_map = feature_map
         self.tie_feature_map_qk = tie_feature_map_qk
+        if linear_mode not in ("global", "complement"):
+            raise NotImplementedError(f"Not supported linear mode {linear_mode}.")
+        self.linear_mode = linear_mode
         self.init_weights_()
 
     def init_weights_(self):
@@ -121,6 +127,8 @@ class SparseLinearAttention(nn.Module):
         qc = q.to(self.dtype)
         kc = k.to(self.dtype)
         vc = v.to(self.dtype)
+        if self.linear_mode == "complement":
+            return self._forward_complement(q, k, qc, kc, vc, dtype, return_sparsity)
         weight = self.proj_l.weight.contiguous()
         with torch.no_grad():
             state = _StateBuild(kc, vc, weight, self.feature_map)
@@ -132,6 +140,18 @@ class SparseLinearAttention(nn.Module):
                             self.BLKK, self.feature_map, state)
         o = o.to(dtype)
 
+        if return_sparsity:
+            return o, real_topk / sparse_map.shape[-1]
+        return o
+
+    def _forward_complement(self, q, k, qc, kc, vc, dtype, return_sparsity):
+        if torch.is_grad_enabled() and any(t.requires_grad for t in (qc, kc, vc, self.proj_l.weight, self.proj_l.bias)):
+            raise NotImplementedError("linear_mode='complement' has no backward; call it under torch.no_grad()")
+        sparse_map, lut, real_topk = get_block_map(q, k, topk_ratio=self.topk, BLKQ=self.BLKQ, BLKK=self.BLKK)
+        assert self.BLKQ in (64, 128) and self.BLKK == 64
+        o_s, _ = sparse_attn_fwd(qc, kc, vc, lut, real_topk, self.BLKQ, self.BLKK, qc.shape[-1] ** -0.5)
+        o = linear_complement_fwd(qc, kc, vc, lut, real_topk, self.proj_l.weight.contiguous(),
+                                  self.proj_l.bias.contiguous(), o_s, self.feature_map, self.BLKQ, self.BLKK).to(dtype)
         if return_sparsity:
             return o, real_topk / sparse_map.shape[-1]
         return o

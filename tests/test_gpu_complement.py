@@ -1,0 +1,63 @@
+"""Complement-mode linear branch (linear attention over the non-selected key blocks) vs the brute-force oracle."""
+import pytest
+import torch
+
+from conftest import cos_sim, max_abs
+from oracle import sla_oracle as O
+from sla_amd import SparseLinearAttention
+from sla_amd.inputs import CONFIGS, make_inputs, make_proj
+from sla_amd.linear import linear_complement_fwd, linear_fwd
+
+pytestmark = pytest.mark.gpu
+
+TOL_ABS = 2e-2
+TOL_COS = 0.999
+
+
+@pytest.mark.parametrize("fmap", ["elu", "relu", "softmax"])
+@pytest.mark.parametrize("L,D,BLKQ,ratio", [(512, 128, 64, 0.25), (1000, 128, 128, 0.3), (333, 64, 64, 0.5), (700, 64, 128, 0.2)])
+def test_complement_vs_oracle(dev, fmap, L, D, BLKQ, ratio):
+    g = torch.Generator().manual_seed(L + D)
+    q, k, v, res = (torch.randn(1, 2, L, D, generator=g).to(torch.bfloat16) for _ in range(4))
+    w, b = make_proj(D)
+    m, lut, T = O.get_block_map(q, k, ratio, BLKQ, 64)
+    ref = O.linear_branch_complement(q, k, v, lut, w, b, fmap, BLKQ, 64, torch.float32).float() + res.float()
+    out = linear_complement_fwd(q.to(dev), k.to(dev), v.to(dev), lut.to(dev), T, w.to(dev), b.to(dev), res.to(dev), fmap,
+                                BLKQ, 64).cpu()
+    assert out.dtype == torch.bfloat16
+    assert max_abs(out, ref) <= TOL_ABS and cos_sim(out, ref) >= TOL_COS
+
+
+def test_empty_selection_equals_global_branch(dev):
+    """With nothing selected the complement is everything: same result as the global linear branch up to the
+    16-bit rounding of the per-block states and of the unfolded projection."""
+    g = torch.Generator().manual_seed(11)
+    q, k, v = (torch.randn(1, 2, 640, 128, generator=g).to(torch.bfloat16).to(dev) for _ in range(3))
+    w, b = (t.to(dev) for t in make_proj(128))
+    lut = torch.zeros((1, 2, 10, 0), dtype=torch.int64, device=dev)
+    out = linear_complement_fwd(q, k, v, lut, 0, w, b, None, "elu")
+    ref = linear_fwd(q, k, v, w, b, None, "elu")
+    assert max_abs(out.cpu(), ref.cpu()) <= TOL_ABS and cos_sim(out.cpu(), ref.cpu()) >= TOL_COS
+
+
+def test_int32_lut_and_module_option(dev):
+    cfg = CONFIGS["cfg2"]
+    d = make_inputs(cfg, H=2)
+    q, k, v = (d[x] for x in "qkv")
+    w, b = make_proj(cfg.D)
+    mod = SparseLinearAttention(cfg.D, cfg.topk, "relu", cfg.BLKQ, cfg.BLKK, linear_mode="complement").to(dev)
+    with torch.no_grad():
+        mod.proj_l.weight.copy_(w)
+        mod.proj_l.bias.copy_(b)
+        o = mod(q.to(dev), k.to(dev), v.to(dev)).cpu()
+    m, lut, T = O.get_block_map(q, k, cfg.topk, cfg.BLKQ, cfg.BLKK)
+    o_s, _ = O.sparse_attn_fwd_gather(q, k, v, lut, cfg.BLKQ, cfg.BLKK)
+    ref = o_s.float() + O.linear_branch_complement(q, k, v, lut, w, b, "relu", cfg.BLKQ, cfg.BLKK, torch.float32).float()
+    assert max_abs(o, ref) <= TOL_ABS and cos_sim(o, ref) >= TOL_COS
+    out32 = linear_complement_fwd(q.to(dev), k.to(dev), v.to(dev), lut.to(dev).int(), T, w.to(dev), b.to(dev), None, "relu")
+    out64 = linear_complement_fwd(q.to(dev), k.to(dev), v.to(dev), lut.to(dev), T, w.to(dev), b.to(dev), None, "relu")
+    assert torch.equal(out32, out64)
+    with pytest.raises(NotImplementedError):
+        mod(q.to(dev), k.to(dev), v.to(dev))          # gradients enabled: no backward for this mode
+    with pytest.raises(NotImplementedError):
+        SparseLinearAttention(cfg.D, cfg.topk, "relu", linear_mode="selected")

@@ -82,3 +82,43 @@ def test_module_forward_is_sum_of_branches():
     o, o_s, o_l, m, lut, T = O.sla_forward(q, k, v, w, b, 0.5, "elu", compute_dtype=torch.float32)
     ref, ref_s, ref_l = O.sla_forward_autograd(q, k, v, w, b, m, "elu", 64, 64)
     assert (o.double() - ref).abs().max() < 1e-4
+
+
+# ---- complement mode (linear branch over the non-selected key blocks) ----------------------------------
+def _complement_case(L=300, D=16, BLKQ=64, BLKK=64, ratio=0.4, seed=3):
+    g = torch.Generator().manual_seed(seed)
+    q, k, v = (torch.randn(1, 2, L, D, generator=g) for _ in range(3))
+    m, lut, T = O.get_block_map(q, k, ratio, BLKQ, BLKK)
+    w = torch.randn(D, D, generator=g) / D ** 0.5
+    b = torch.randn(D, generator=g)
+    return q, k, v, m, lut, T, w, b
+
+
+@pytest.mark.parametrize("fmap", ["elu", "relu", "softmax"])
+def test_complement_equals_masked_dense_linear_attention(fmap):
+    """Independent restatement: dense (L x L) kernelised attention with the selected blocks masked out."""
+    q, k, v, m, lut, T, w, b = _complement_case()
+    L = q.shape[2]
+    phi = O.feature_map(fmap)
+    a = phi(q.double()) @ phi(k.double()).transpose(-1, -2)              # (B,H,L,L)
+    keep = ~O.expand_block_map(m, L, 64, 64)
+    a = a * keep
+    o = (a @ v.double()) / (1e-5 + a.sum(dim=-1, keepdim=True))
+    ref = torch.nn.functional.linear(o, w.double(), b.double())
+    got = O.linear_branch_complement(q, k, v, lut, w, b, fmap, 64, 64, torch.float32)
+    assert float((got.double() - ref).abs().max()) < 1e-4
+
+
+def test_complement_with_nothing_selected_is_the_global_branch():
+    q, k, v, m, lut, T, w, b = _complement_case()
+    empty = lut[..., :0]
+    got = O.linear_branch_complement(q, k, v, empty, w, b, "elu", 64, 64, torch.float32)
+    ref = O.linear_branch(q, k, v, w, b, "elu", torch.float32)
+    assert float((got - ref).abs().max()) < 1e-4
+
+
+def test_complement_with_everything_selected_is_the_bias():
+    q, k, v, m, lut, T, w, b = _complement_case(ratio=1.0)
+    got = O.linear_branch_complement(q, k, v, lut, w, b, "relu", 64, 64, torch.float32)
+    # numerator and divisor state are (numerically) zero: o_l = 0 / 1e-5, so only the bias is left
+    assert float((got - b).abs().max()) < 1e-2
