@@ -1,0 +1,39 @@
+"""A DiT-style self-attention block around ``SparseLinearAttention``: the caller either side of the path.
+
+The reference README (``README.md:2``, usage at ``README.md:30-50``) motivates SLA as a replacement of the
+attention call inside a video-diffusion transformer block that is then fine-tuned; its benchmark moves between
+the ``(B, L, H, D)`` layout of such blocks and the operator's ``(B, H, L, D)`` (``evaluate/bench_kernel.py:68-71``).
+This module is that caller: QKV projection -> head split -> SLA -> head merge -> output projection.  The two
+projections are plain library GEMMs; the layout changes are single fused copies (``unbind`` of one permuted
+``(3, B, H, L, D)`` tensor), after which the operator sees the contiguous ``(B, H, L, D)`` it requires.
+"""
+from __future__ import annotations
+
+import torch
+import torch.nn as nn
+
+from .module import SparseLinearAttention
+
+
+class SLASelfAttention(nn.Module):
+    def __init__(self, dim, num_heads, topk, feature_map="softmax", BLKQ=64, BLKK=64, use_bf16=True, qkv_bias=True,
+                 linear_mode="global"):
+        super().__init__()
+        if dim % num_heads != 0:
+            raise ValueError(f"dim {dim} is not a multiple of num_heads {num_heads}")
+        self.num_heads = num_heads
+        self.head_dim = dim // num_heads
+        self.qkv = nn.Linear(dim, 3 * dim, bias=qkv_bias)
+        self.attn = SparseLinearAttention(self.head_dim, topk, feature_map, BLKQ, BLKK, use_bf16=use_bf16,
+                                          linear_mode=linear_mode)
+        self.proj = nn.Linear(dim, dim)
+
+    def forward(self, x):
+        """x: (B, L, dim) -> (B, L, dim)."""
+        B, L, C = x.shape
+        H, D = self.num_heads, self.head_dim
+        # one copy: (B, L, 3, H, D) -> (3, B, H, L, D) contiguous; q, k, v are then contiguous views of it
+        qkv = self.qkv(x).view(B, L, 3, H, D).permute(2, 0, 3, 1, 4).contiguous()
+        q, k, v = qkv.unbind(0)
+        o = self.attn(q, k, v)                                  # (B, H, L, D)
+        return self.proj(o.transpose(1, 2).reshape(B, L, C))
