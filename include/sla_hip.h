@@ -79,6 +79,18 @@ int sla_sparse_attn_fwd(const void* q, const void* k, const void* v, const void*
                         void* o, float* lse, int dtype, int B, int H, int L, int D, int BLKQ, int BLKK,
                         int topk, float qk_scale, void* stream);
 
+/* The attention forward with the module's linear branch and final sum fused into its epilogue:
+ *   out = o_s + proj(o_l),  o_l = phi(q) KV / (1e-5 + phi(q) z)
+ * for callers that own both branches.  `linear_workspace` is the workspace sla_linear_state_fwd filled for
+ * the same k, v, weight, fmap (size SLA_WS_LINEAR_FWD); bias (D) fp32.  o_s (optional, may be NULL) receives
+ * the attention output alone, which the backward needs; out and o_s in `dtype`.  Equal bit for bit to
+ * sla_sparse_attn_fwd followed by sla_linear_out_fwd with residual = o_s.
+ * Replaces kernel.py:21-82, 242-274 and core.py:90-100 (q feature map, rest of calc_linear, proj_l, sum). */
+int sla_sparse_attn_linear_fwd(const void* q, const void* k, const void* v, const void* lut, int lut_elem_bytes,
+                               const void* linear_workspace, int64_t linear_workspace_bytes, const float* bias,
+                               void* o_s, void* out, float* lse, int dtype, int fmap, int B, int H, int L, int D,
+                               int BLKQ, int BLKK, int topk, float qk_scale, void* stream);
+
 /* Block-sparse FlashAttention backward: delta, dQ over the look-up table, dK/dV
  * over per-key-block lists built from the int8 map.
  * Replaces _attention.backward + _attn_bwd_preprocess/_dq/_dkdv,

@@ -30,6 +30,8 @@ SIGNATURES = {
     "sla_mean_pool": (_I, [_P, _P, _I, _I, _I, _I, _I, _P]),
     "sla_block_map_fwd": (_I, [_P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _I64, _P, _P, _I, _P]),
     "sla_sparse_attn_fwd": (_I, [_P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _P]),
+    "sla_sparse_attn_linear_fwd": (_I, [_P, _P, _P, _P, _I, _P, _I64, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I,
+                                        _F, _P]),
     "sla_sparse_attn_bwd": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I,
                                  _I, _F, _P, _I64, _P]),
     "sla_linear_fwd": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I64, _P]),

@@ -219,6 +219,14 @@ static __device__ __forceinline__ void store_acc_tile(uint16_t* stage, const flo
   wave_lds_fence();   // the staging area may be rewritten right after
 }
 
+// Keeps an fp32 value as it is: stops the compiler from merging the operation that produced it with a
+// following conversion to 16 bit (a mixed-precision fma rounds once, fp32-then-16-bit rounds twice), so
+// that two kernels evaluating the same expression agree bit for bit.
+static __device__ __forceinline__ float pin_f32(float x) {
+  asm volatile("" : "+v"(x));
+  return x;
+}
+
 static __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 static __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 

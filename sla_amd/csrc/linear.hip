@@ -129,7 +129,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         acc = E::mfma32(a, qf[c], acc);
       }
 #pragma unroll
-      for (int i = 0; i < 16; ++i) val[t][i] = acc[i] * inv_den + sBias[32 * t + 8 * (i >> 2) + 4 * g + (i & 3)];
+      for (int i = 0; i < 16; ++i) val[t][i] = pin_f32(__builtin_fmaf(acc[i], inv_den, sBias[32 * t + 8 * (i >> 2) + 4 * g + (i & 3)]));   // as in the fused epilogue
     }
     store_acc_tile<E, D>(stage, val, out + off, residual ? &res : nullptr, rows_valid, lane);
   }

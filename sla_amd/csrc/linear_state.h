@@ -8,7 +8,7 @@ namespace sla {
 // grid (nsplit, BH), 256 threads.  Thread t moves 16-byte chunk (t%CPR) of rows t/CPR + i*RPP.
 // OUT16: the D x D partial is written rounded to 16 bit (per-key-block states of the complement mode).
 template <typename Tag, int D, bool OUT16 = false>
-__global__ __launch_bounds__(256) void linear_state_partial_kernel(const uint16_t* __restrict__ k,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void linear_state_partial_kernel(const uint16_t* __restrict__ k,
                                                                    const uint16_t* __restrict__ v, void* __restrict__ kv_part_,
                                                                    float* __restrict__ z_part, int L, int rows_per_split,
                                                                    int fmap) {
@@ -49,18 +49,29 @@ __global__ __launch_bounds__(256) void linear_state_partial_kernel(const uint16_
   const int tr_row = (lane & 15) >> 2;
   const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
 
+  // rows of the next tile are fetched into registers while the current tile is multiplied
+  i16x8_t kreg[NP], vreg[NP];
+  auto fetch = [&](int r0) {
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
+      const int grow = r0 + lrow + p * RPP;
+      kreg[p] = i16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+      vreg[p] = i16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+      if (grow < row_end) {
+        kreg[p] = *reinterpret_cast<const i16x8_t*>(kh + (size_t)grow * D + lcol);
+        vreg[p] = *reinterpret_cast<const i16x8_t*>(vh + (size_t)grow * D + lcol);
+      }
+    }
+  };
+  if (row_begin < row_end) fetch(row_begin);
   for (int r0 = row_begin; r0 < row_end; r0 += TR) {
     __syncthreads();
 #pragma unroll
     for (int p = 0; p < NP; ++p) {
       const int row = lrow + p * RPP;
       const int grow = r0 + row;
-      i16x8_t kk = {0, 0, 0, 0, 0, 0, 0, 0}, vv = {0, 0, 0, 0, 0, 0, 0, 0};
+      const i16x8_t kk = kreg[p], vv = vreg[p];
       const bool ok = grow < row_end;
-      if (ok) {
-        kk = *reinterpret_cast<const i16x8_t*>(kh + (size_t)grow * D + lcol);
-        vv = *reinterpret_cast<const i16x8_t*>(vh + (size_t)grow * D + lcol);
-      }
       float f[8];
 #pragma unroll
       for (int e = 0; e < 8; ++e) f[e] = E::to_float((uint16_t)kk[e]);
@@ -96,6 +107,7 @@ __global__ __launch_bounds__(256) void linear_state_partial_kernel(const uint16_
       *reinterpret_cast<i16x8_t*>(&sK[row * STR + lcol]) = fk;
       *reinterpret_cast<i16x8_t*>(&sV[row * STR + lcol]) = vv;
     }
+    if (r0 + TR < row_end) fetch(r0 + TR);
     __syncthreads();
 #pragma unroll
     for (int c = 0; c < TR / 16; ++c) {

@@ -12,17 +12,26 @@
 // K/V tiles go global -> registers -> LDS; the next tile's K is in flight during QK^T and
 // softmax, its V during PV.  Register use is held to 256 so two waves share a SIMD and one
 // wave's softmax (vector ALU) overlaps the other's MFMAs.
-#include "common.h"
+#include "linear_state.h"
 
 namespace sla {
 
-template <typename Tag, int D, int BLKQ>
+// What the fused variant (FUSED = true) adds after the loop: the linear branch of the same query rows,
+// out = o_s + (phi(q) KVW / divisor + bias), from the per-head state the linear state kernels left in
+// their workspace (kvwt: KVW^T in 16 bit, zst: sum phi(k) in 16 bit).  The state is staged in the LDS the
+// K/V tiles no longer need, the raw q fragments are still in registers, and the product costs as many
+// MFMAs as one more key tile.  o then receives the sum; o_s (optional) the attention output alone.
+template <typename Tag, int D, int BLKQ, bool FUSED>
 __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))) void sparse_fwd_kernel(const uint16_t* __restrict__ q,
                                                               const uint16_t* __restrict__ k,
                                                               const uint16_t* __restrict__ v,
                                                               const void* __restrict__ lut, int lut64,
                                                               uint16_t* __restrict__ o, float* __restrict__ lse, int L,
-                                                              int Mblk, int topk, float scale_log2e, int total) {
+                                                              int Mblk, int topk, float scale_log2e, int total,
+                                                              const uint16_t* __restrict__ kvwt,
+                                                              const uint16_t* __restrict__ zst,
+                                                              const float* __restrict__ bias, int fmap,
+                                                              uint16_t* __restrict__ o_s) {
   using E = Elem<Tag>;
   constexpr int BLKK = 64;
   constexpr int NT = BLKQ * 2;              // threads
@@ -34,8 +43,10 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
   constexpr int NLD = BLKK * CPR / NT;      // 16-byte chunks each thread moves per tile
   static_assert(BLKK * CPR % NT == 0, "tile does not divide among the threads");
 
-  __shared__ __attribute__((aligned(16))) uint16_t sK[BLKK * KSTR];
-  __shared__ __attribute__((aligned(16))) uint16_t sV[BLKK * VSTR];
+  __shared__ __attribute__((aligned(16))) uint16_t smem[BLKK * KSTR + BLKK * VSTR];
+  uint16_t* const sK = smem;
+  uint16_t* const sV = smem + BLKK * KSTR;
+  static_assert(D * (D + 8) <= BLKK * KSTR + BLKK * VSTR, "the folded state must fit where the K/V tiles were");
 
   const int logical = xcd_remap(blockIdx.x, gridDim.x, total);
   if (logical < 0) return;
@@ -277,34 +288,122 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
   // ---- epilogue ----
   const float l_tot = l_run + __shfl_xor(l_run, 32);
   const float inv = 1.0f / l_tot;
-  if (qrow < L) {
-    uint16_t* orow = o + head_off + (size_t)qrow * D;
+  if (!FUSED) {
+    if (qrow < L) {
+      uint16_t* orow = o + head_off + (size_t)qrow * D;
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
+      for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-      for (int i4 = 0; i4 < 4; ++i4) {
-        i32x2_t w;
-        w[0] = (int)E::pack2(oacc[dt][4 * i4 + 0] * inv, oacc[dt][4 * i4 + 1] * inv);
-        w[1] = (int)E::pack2(oacc[dt][4 * i4 + 2] * inv, oacc[dt][4 * i4 + 3] * inv);
-        *reinterpret_cast<i32x2_t*>(orow + 32 * dt + 8 * i4 + 4 * g) = w;
+        for (int i4 = 0; i4 < 4; ++i4) {
+          i32x2_t w;
+          w[0] = (int)E::pack2(oacc[dt][4 * i4 + 0] * inv, oacc[dt][4 * i4 + 1] * inv);
+          w[1] = (int)E::pack2(oacc[dt][4 * i4 + 2] * inv, oacc[dt][4 * i4 + 3] * inv);
+          *reinterpret_cast<i32x2_t*>(orow + 32 * dt + 8 * i4 + 4 * g) = w;
+        }
+      if (g == 0) lse[(size_t)bh * L + qrow] = m_run + fast_log2(l_tot);
+    }
+  } else {
+    // ---- linear branch of the same rows (the loop's last barrier has freed the tile buffers) ----
+    constexpr int SSTR = D + 8;
+    __shared__ float sZ[D];
+    __shared__ float sBias[D];
+    {
+      const uint16_t* src = kvwt + (size_t)bh * D * D;
+      for (int idx = tid; idx < D * D / 8; idx += NT) {
+        const int row = idx / (D / 8), col = (idx % (D / 8)) * 8;
+        *reinterpret_cast<i16x8_t*>(&smem[row * SSTR + col]) = *reinterpret_cast<const i16x8_t*>(src + (size_t)row * D + col);
       }
-    if (g == 0) lse[(size_t)bh * L + qrow] = m_run + fast_log2(l_tot);
+      for (int d = tid; d < D; d += NT) {
+        sZ[d] = E::to_float(zst[(size_t)bh * D + d]);
+        sBias[d] = round16<Tag>(bias[d]);
+      }
+    }
+    __syncthreads();
+    // phi(q) from the resident raw q fragments: this lane holds d = 16c + 8g + j of its row
+    float f[DC][8];
+#pragma unroll
+    for (int c = 0; c < DC; ++c)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) f[c][j] = E::to_float((uint16_t)qf[c][j]);
+    float row_mx, row_inv;
+    phi_row_pair<Tag, DC>(fmap, f, row_mx, row_inv);
+    float den = 0.f;
+#pragma unroll
+    for (int c = 0; c < DC; ++c) {
+      i32x4_t pw;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) den += round16<Tag>(f[c][j] * sZ[16 * c + 8 * g + j]);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) pw[j] = (int)E::pack2(f[c][2 * j], f[c][2 * j + 1]);
+      qf[c] = __builtin_bit_cast(i16x8_t, pw);
+    }
+    den += __shfl_xor(den, 32);
+    den = round16<Tag>(1e-5f + round16<Tag>(den));
+    const float inv_den = 1.0f / den;
+    const bool ok = qrow < L;
+    const size_t off = head_off + (size_t)qrow * D;
+#pragma unroll
+    for (int et = 0; et < DT; ++et) {
+      f32x16_t acc;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+#pragma unroll
+      for (int c = 0; c < DC; ++c) {
+        const i16x8_t a = *reinterpret_cast<const i16x8_t*>(&smem[(32 * et + r) * SSTR + 16 * c + 8 * g]);
+        acc = E::mfma32(a, qf[c], acc);
+      }
+      if (ok) {
+#pragma unroll
+        for (int i4 = 0; i4 < 4; ++i4) {
+          const int e0 = 32 * et + 8 * i4 + 4 * g;
+          i32x2_t ws, wo;
+          ws[0] = (int)E::pack2(oacc[et][4 * i4 + 0] * inv, oacc[et][4 * i4 + 1] * inv);
+          ws[1] = (int)E::pack2(oacc[et][4 * i4 + 2] * inv, oacc[et][4 * i4 + 3] * inv);
+          if (o_s) *reinterpret_cast<i32x2_t*>(o_s + off + e0) = ws;
+          // the sum as the reference's tensor addition forms it: both summands in 16 bit, one rounded add
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            const uint32_t x = (uint32_t)ws[h];
+            const float l0 = round16<Tag>(pin_f32(__builtin_fmaf(acc[4 * i4 + 2 * h], inv_den, sBias[e0 + 2 * h])));
+            const float l1 = round16<Tag>(pin_f32(__builtin_fmaf(acc[4 * i4 + 2 * h + 1], inv_den, sBias[e0 + 2 * h + 1])));
+            wo[h] = (int)E::pack2(E::to_float((uint16_t)(x & 0xffff)) + l0, E::to_float((uint16_t)(x >> 16)) + l1);
+          }
+          *reinterpret_cast<i32x2_t*>(o + off + e0) = wo;
+        }
+      }
+    }
+    if (ok && g == 0) lse[(size_t)bh * L + qrow] = m_run + fast_log2(l_tot);
   }
 }
 
+struct FusedLinear {        // state of the linear branch for the fused epilogue (all null / 0 when not fused)
+  const uint16_t* kvwt;
+  const uint16_t* zst;
+  const float* bias;
+  int fmap;
+  uint16_t* o_s;
+};
+
 template <typename Tag>
 static int launch_fwd(const void* q, const void* k, const void* v, const void* lut, int lut64, void* o, float* lse, int BH,
-                      int L, int D, int BLKQ, int topk, float qk_scale, hipStream_t st) {
+                      int L, int D, int BLKQ, int topk, float qk_scale, const FusedLinear* fl, hipStream_t st) {
   const int Mblk = cdiv(L, BLKQ);
   const int64_t total64 = (int64_t)BH * Mblk;
   const int total = (int)total64;
   const int grid = xcd_grid(total);
   const float c = qk_scale * 1.4426950408889634f;
-#define SLA_FWD_CASE(DD, BQ)                                                                                         \
-  if (D == DD && BLKQ == BQ) {                                                                                       \
-    hipLaunchKernelGGL((sparse_fwd_kernel<Tag, DD, BQ>), dim3(grid), dim3(BQ * 2), 0, st, (const uint16_t*)q,       \
-                       (const uint16_t*)k, (const uint16_t*)v, lut, lut64, (uint16_t*)o, lse, L, Mblk, topk, c, total); \
-    return check_launch("sparse_attn_fwd");                                                                          \
+#define SLA_FWD_CASE(DD, BQ)                                                                                          \
+  if (D == DD && BLKQ == BQ) {                                                                                        \
+    if (fl)                                                                                                           \
+      hipLaunchKernelGGL((sparse_fwd_kernel<Tag, DD, BQ, true>), dim3(grid), dim3(BQ * 2), 0, st, (const uint16_t*)q, \
+                         (const uint16_t*)k, (const uint16_t*)v, lut, lut64, (uint16_t*)o, lse, L, Mblk, topk, c,    \
+                         total, fl->kvwt, fl->zst, fl->bias, fl->fmap, fl->o_s);                                      \
+    else                                                                                                              \
+      hipLaunchKernelGGL((sparse_fwd_kernel<Tag, DD, BQ, false>), dim3(grid), dim3(BQ * 2), 0, st,                   \
+                         (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, lut, lut64, (uint16_t*)o, lse,  \
+                         L, Mblk, topk, c, total, (const uint16_t*)nullptr, (const uint16_t*)nullptr,                 \
+                         (const float*)nullptr, 0, (uint16_t*)nullptr);                                               \
+    return check_launch("sparse_attn_fwd");                                                                           \
   }
   SLA_FWD_CASE(128, 64)
   SLA_FWD_CASE(128, 128)
@@ -346,6 +445,30 @@ extern "C" int sla_sparse_attn_fwd(const void* q, const void* k, const void* v, 
   hipStream_t st = (hipStream_t)stream;
   const int BH = B * H;
   if (dtype == SLA_BF16)
-    return launch_fwd<bf16_tag>(q, k, v, lut, lut_elem_bytes == 8, o, lse, BH, L, D, BLKQ, topk, qk_scale, st);
-  return launch_fwd<f16_tag>(q, k, v, lut, lut_elem_bytes == 8, o, lse, BH, L, D, BLKQ, topk, qk_scale, st);
+    return launch_fwd<bf16_tag>(q, k, v, lut, lut_elem_bytes == 8, o, lse, BH, L, D, BLKQ, topk, qk_scale, nullptr, st);
+  return launch_fwd<f16_tag>(q, k, v, lut, lut_elem_bytes == 8, o, lse, BH, L, D, BLKQ, topk, qk_scale, nullptr, st);
+}
+
+extern "C" int sla_sparse_attn_linear_fwd(const void* q, const void* k, const void* v, const void* lut, int lut_elem_bytes,
+                                          const void* linear_workspace, int64_t linear_workspace_bytes, const float* bias,
+                                          void* o_s, void* out, float* lse, int dtype, int fmap, int B, int H, int L, int D,
+                                          int BLKQ, int BLKK, int topk, float qk_scale, void* stream) {
+  int rc = validate_attn_shape(dtype, B, H, L, D, BLKQ, BLKK, topk, lut_elem_bytes);
+  if (rc) return rc;
+  rc = validate_linear(dtype, fmap, B, H, L, D);
+  if (rc) return rc;
+  SLA_REQUIRE(q && k && v && out && lse && bias && linear_workspace && (lut || topk == 0), SLA_ERR_BAD_ARG, "null pointer");
+  SLA_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out | (uintptr_t)o_s | (uintptr_t)linear_workspace) %
+                      16 == 0,
+              SLA_ERR_BAD_ARG, "q, k, v, out, o_s, workspace must be 16-byte aligned");
+  const int BH = B * H;
+  const LinWs w = lin_ws(BH, L, D);
+  SLA_REQUIRE(linear_workspace_bytes >= (int64_t)w.total, SLA_ERR_WORKSPACE, "workspace of %lld bytes, need %lld",
+              (long long)linear_workspace_bytes, (long long)w.total);
+  const char* ws = (const char*)linear_workspace;
+  FusedLinear fl{(const uint16_t*)(ws + w.kvwt), (const uint16_t*)(ws + w.z), bias, fmap, (uint16_t*)o_s};
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == SLA_BF16)
+    return launch_fwd<bf16_tag>(q, k, v, lut, lut_elem_bytes == 8, out, lse, BH, L, D, BLKQ, topk, qk_scale, &fl, st);
+  return launch_fwd<f16_tag>(q, k, v, lut, lut_elem_bytes == 8, out, lse, BH, L, D, BLKQ, topk, qk_scale, &fl, st);
 }

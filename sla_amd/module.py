@@ -7,7 +7,7 @@ import torch.nn as nn
 
 from .block_map import get_block_map
 from .linear import linear_bwd, linear_complement_fwd, linear_out_fwd, linear_state_fwd
-from .sparse_attn import sparse_attn_bwd, sparse_attn_fwd
+from .sparse_attn import sparse_attn_bwd, sparse_attn_fwd, sparse_attn_linear_fwd
 
 FEATURE_MAPS = ("elu", "relu", "softmax")
 
@@ -20,16 +20,19 @@ class _sla_core(torch.autograd.Function):
     """
 
     @staticmethod
-    def forward(ctx, q, k, v, weight, bias, sparse_map, lut, topk, BLKQ, BLKK, fmap, state):
+    def forward(ctx, q, k, v, weight, bias, sparse_map, lut, topk, BLKQ, BLKK, fmap, state, needs_grad=True):
         assert q.is_contiguous() and k.is_contiguous() and v.is_contiguous()
         assert sparse_map.is_contiguous() and lut.is_contiguous()
         assert BLKQ == 64 or BLKQ == 128
         assert BLKK == 64
         qk_scale = q.shape[-1] ** -0.5
         bias = bias.contiguous()
-        o_s, lse = sparse_attn_fwd(q, k, v, lut, topk, BLKQ, BLKK, qk_scale)
-        state_ws = state.join()
-        out = linear_out_fwd(q, bias, o_s, state_ws, fmap)
+        # one kernel: attention over the selected blocks, then the linear branch of the same rows from the
+        # per-head state, projection and sum in its epilogue; o_s is only written when a backward will need it
+        out, o_s, lse = sparse_attn_linear_fwd(q, k, v, lut, topk, BLKQ, BLKK, qk_scale, state.join(), bias, fmap,
+                                               want_o_s=needs_grad)
+        if not needs_grad:
+            return out
         ctx.save_for_backward(q, k, v, weight, bias, sparse_map, lut, lse, o_s)
         ctx.cfg = (topk, BLKQ, BLKK, fmap, qk_scale)
         return out
@@ -41,7 +44,7 @@ class _sla_core(torch.autograd.Function):
         d_out = d_out.contiguous()
         dq, dk, dv = sparse_attn_bwd(q, k, v, o_s, d_out, lse, sparse_map, lut, topk, BLKQ, BLKK, qk_scale)
         _, _, _, dw, db = linear_bwd(q, k, v, weight, bias, d_out, fmap, accumulate_into=(dq, dk, dv))
-        return dq, dk, dv, dw, db, None, None, None, None, None, None, None
+        return dq, dk, dv, dw, db, None, None, None, None, None, None, None, None
 
 
 class _StateBuild:
@@ -136,8 +139,10 @@ class SparseLinearAttention(nn.Module):
         # the mask is built from the inputs in their own dtype (reference core.py:83)
         sparse_map, lut, real_topk = get_block_map(q, k, topk_ratio=self.topk, BLKQ=self.BLKQ, BLKK=self.BLKK)
 
+        needs_grad = torch.is_grad_enabled() and any(
+            t.requires_grad for t in (qc, kc, vc, weight, self.proj_l.bias))
         o = _sla_core.apply(qc, kc, vc, weight, self.proj_l.bias, sparse_map, lut, real_topk, self.BLKQ,
-                            self.BLKK, self.feature_map, state)
+                            self.BLKK, self.feature_map, state, needs_grad)
         o = o.to(dtype)
 
         if return_sparsity:

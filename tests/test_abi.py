@@ -73,6 +73,12 @@ def test_other_entry_points_validate():
     assert lib.sla_block_map_fwd(FAKE, FAKE, 1, 1, 1, 128, 64, 64, 64, 1, FAKE, 16, FAKE, FAKE, 8, None) == _lib.ERR_WORKSPACE
     assert lib.sla_linear_fwd(FAKE, FAKE, FAKE, FAKE, FAKE, None, FAKE, 1, 9, 1, 1, 64, 128, FAKE, 1 << 30, None) == _lib.ERR_BAD_ARG
     assert lib.sla_linear_fwd(FAKE, FAKE, FAKE, FAKE, FAKE, None, FAKE, 1, 0, 1, 1, 64, 96, FAKE, 1 << 30, None) == _lib.ERR_UNSUPPORTED
+    assert lib.sla_sparse_attn_linear_fwd(FAKE, FAKE, FAKE, FAKE, 8, FAKE, 8, FAKE, None, FAKE, FAKE, 1, 0, 1, 1, 128, 128,
+                                          64, 64, 1, 0.1, None) == _lib.ERR_WORKSPACE
+    assert lib.sla_sparse_attn_linear_fwd(FAKE, FAKE, FAKE, FAKE, 8, FAKE, 1 << 30, FAKE, None, FAKE, FAKE, 1, 7, 1, 1, 128,
+                                          128, 64, 64, 1, 0.1, None) == _lib.ERR_BAD_ARG
+    assert lib.sla_linear_complement_fwd(FAKE, FAKE, FAKE, FAKE, 8, FAKE, FAKE, None, FAKE, 1, 0, 1, 1, 128, 128, 64, 32, 1,
+                                         FAKE, 1 << 30, None) == _lib.ERR_UNSUPPORTED
     assert lib.sla_linear_state_fwd(FAKE, FAKE, FAKE, 1, 0, 1, 1, 64, 128, FAKE, 8, None) == _lib.ERR_WORKSPACE
     assert lib.sla_linear_state_fwd(FAKE, None, FAKE, 1, 0, 1, 1, 64, 128, FAKE, 1 << 30, None) == _lib.ERR_BAD_ARG
     assert lib.sla_linear_out_fwd(FAKE, FAKE, None, FAKE, 0, 0, 1, 1, 64, 128, FAKE, 1 << 30, None) == _lib.ERR_UNSUPPORTED

@@ -110,3 +110,27 @@ def test_forward_in_a_hip_graph(dev):
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(out, ref2)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("L,D,BLKQ,fmap", [(1000, 128, 64, "elu"), (700, 128, 128, "softmax"), (333, 64, 64, "relu"),
+                                            (512, 64, 128, "elu")])
+def test_fused_epilogue_equals_the_two_kernel_path(dev, dtype, L, D, BLKQ, fmap):
+    """sla_sparse_attn_linear_fwd == sla_sparse_attn_fwd followed by sla_linear_out_fwd(residual = o_s),
+    bit for bit, for out, o_s and lse (ragged L, both block sizes, both head dims, all feature maps)."""
+    from sla_amd import get_block_map
+    from sla_amd.linear import linear_out_fwd, linear_state_fwd
+    from sla_amd.sparse_attn import sparse_attn_fwd, sparse_attn_linear_fwd
+    g = torch.Generator().manual_seed(L)
+    q, k, v = (torch.randn(1, 3, L, D, generator=g).to(dtype).to(dev) for _ in range(3))
+    w, b = (t.to(dev) for t in make_proj(D))
+    m, lut, T = get_block_map(q, k, 0.3, BLKQ, 64)
+    ws = linear_state_fwd(k, v, w, fmap)
+    o_s, lse = sparse_attn_fwd(q, k, v, lut, T, BLKQ, 64, D ** -0.5)
+    ref = linear_out_fwd(q, b, o_s, ws, fmap)
+    out, o_s2, lse2 = sparse_attn_linear_fwd(q, k, v, lut, T, BLKQ, 64, D ** -0.5, ws, b, fmap, want_o_s=True)
+    bits = lambda t: t.view(torch.int16)            # bit patterns: equal also where float16 overflowed to inf/nan
+    assert torch.equal(o_s2, o_s) and torch.equal(lse2, lse)
+    assert torch.equal(bits(out), bits(ref))
+    out3, none, _ = sparse_attn_linear_fwd(q, k, v, lut, T, BLKQ, 64, D ** -0.5, ws, b, fmap, want_o_s=False)
+    assert none is None and torch.equal(bits(out3), bits(ref))
