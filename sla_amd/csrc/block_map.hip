@@ -53,15 +53,14 @@ struct alignas(16) Vec16 {
 // MODE 2: block mean of round(x - colmean)     -> out     (BH, nblk, D)
 // One thread owns VEC adjacent columns of one block and walks its rows in order.
 template <typename IO, int MODE>
-__global__ __launch_bounds__(256) void pool_kernel(const typename IO::raw* __restrict__ x,
-                                                   const typename IO::raw* __restrict__ colmean,
-                                                   void* __restrict__ out, int L, int D, int BLK, int nblk) {
+static __device__ __forceinline__ void pool_body(const typename IO::raw* __restrict__ x,
+                                                 const typename IO::raw* __restrict__ colmean, void* __restrict__ out, int L,
+                                                 int D, int BLK, int nblk, int bx, int bh) {
   constexpr int VEC = IO::VEC;
   const int tpr = D / VEC;
   const int bpw = 256 / tpr;
-  const int bh = blockIdx.y;
   const int sub = threadIdx.x / tpr;
-  const int blk = blockIdx.x * bpw + sub;
+  const int blk = bx * bpw + sub;
   const int c = (threadIdx.x - sub * tpr) * VEC;
   if (sub >= bpw || blk >= nblk) return;
   const int row0 = blk * BLK;
@@ -76,8 +75,23 @@ __global__ __launch_bounds__(256) void pool_kernel(const typename IO::raw* __res
     for (int e = 0; e < VEC; ++e) cm[e] = IO::ld(m.e[e]);
   }
   const typename IO::raw* p = x + ((size_t)bh * L + row0) * D + c;
-#pragma unroll 8
-  for (int r = 0; r < nrows; ++r) {
+  // rows are fetched sixteen at a time (all loads of a batch in flight together), then added in row order
+  constexpr int BATCH = 16;
+  int r = 0;
+  for (; r + BATCH <= nrows; r += BATCH) {
+    Vec16<IO> v[BATCH];
+#pragma unroll
+    for (int i = 0; i < BATCH; ++i) v[i] = *reinterpret_cast<const Vec16<IO>*>(p + (size_t)(r + i) * D);
+#pragma unroll
+    for (int i = 0; i < BATCH; ++i)
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        float f = IO::ld(v[i].e[e]);
+        if (MODE == 2) f = IO::ld(IO::st(f - cm[e]));
+        acc[e] = acc[e] + f;
+      }
+  }
+  for (; r < nrows; ++r) {
     Vec16<IO> v = *reinterpret_cast<const Vec16<IO>*>(p + (size_t)r * D);
 #pragma unroll
     for (int e = 0; e < VEC; ++e) {
@@ -98,6 +112,25 @@ __global__ __launch_bounds__(256) void pool_kernel(const typename IO::raw* __res
     for (int e = 0; e < VEC; ++e) r.e[e] = IO::st(acc[e] / cnt);
     *reinterpret_cast<Vec16<IO>*>(reinterpret_cast<typename IO::raw*>(out) + o) = r;
   }
+}
+
+template <typename IO, int MODE>
+__global__ __launch_bounds__(256) void pool_kernel(const typename IO::raw* __restrict__ x,
+                                                   const typename IO::raw* __restrict__ colmean,
+                                                   void* __restrict__ out, int L, int D, int BLK, int nblk) {
+  pool_body<IO, MODE>(x, colmean, out, L, D, BLK, nblk, blockIdx.x, blockIdx.y);
+}
+
+// The two independent first passes of the mask builder in one launch (neither fills the memory system alone):
+// blockIdx.z == 0: fp32 chunk sums of k (MODE 0, chunks of KMEAN_CHUNK rows); z == 1: block means of q (MODE 1).
+template <typename IO>
+__global__ __launch_bounds__(256) void pool_pair_kernel(const typename IO::raw* __restrict__ k, float* __restrict__ chunk_sums,
+                                                        int nchunk, const typename IO::raw* __restrict__ q,
+                                                        typename IO::raw* __restrict__ pq, int BLKQ, int nblkq, int L, int D) {
+  if (blockIdx.z == 0)
+    pool_body<IO, 0>(k, nullptr, chunk_sums, L, D, KMEAN_CHUNK, nchunk, blockIdx.x, blockIdx.y);
+  else
+    pool_body<IO, 1>(q, nullptr, pq, L, D, BLKQ, nblkq, blockIdx.x, blockIdx.y);
 }
 
 // Column mean of K, levels 2 and 3 of the fixed summation order:
@@ -128,6 +161,33 @@ __global__ __launch_bounds__(128) void colmean_kernel(const float* __restrict__ 
 #pragma unroll 8
   for (int i = 0; i < ngroup; ++i) acc = acc + p[(size_t)i * D];
   colmean[(size_t)bh * D + d] = IO::st(acc / (float)L);
+}
+
+// Levels 2 and 3 in one workgroup per head when the group sums fit in LDS: thread (gi, d) = (tid / D, tid % D)
+// forms group sums gi, gi + 1024/D, ...; thread d < D then adds the groups in ascending order.
+constexpr int COLMEAN_LDS_FLOATS = 12288;
+template <typename IO>
+__global__ __launch_bounds__(1024) void colmean_fused_kernel(const float* __restrict__ chunk_sums,
+                                                             typename IO::raw* __restrict__ colmean, int nchunk, int ngroup,
+                                                             int D, int L) {
+  __shared__ float gs[COLMEAN_LDS_FLOATS];
+  const int bh = blockIdx.x, tid = threadIdx.x;
+  const int d = tid % D, gstep = 1024 / D;
+  for (int g = tid / D; g < ngroup; g += gstep) {
+    const int c0 = g * KMEAN_GROUP;
+    const int n = min(KMEAN_GROUP, nchunk - c0);
+    const float* p = chunk_sums + ((size_t)bh * nchunk + c0) * D + d;
+    float acc = 0.f;
+#pragma unroll 8
+    for (int i = 0; i < n; ++i) acc = acc + p[(size_t)i * D];
+    gs[g * D + d] = acc;
+  }
+  __syncthreads();
+  if (tid < D) {
+    float acc = 0.f;
+    for (int g = 0; g < ngroup; ++g) acc = acc + gs[g * D + tid];
+    colmean[(size_t)bh * D + tid] = IO::st(acc / (float)L);
+  }
 }
 
 // score[bh][m][n] = round_dtype( sum_d pq[m][d]*pk[n][d] ), d ascending, mul and add rounded separately.
@@ -340,13 +400,24 @@ static void launch_pool(const void* x, const void* colmean, void* out, int BH, i
                      (const typename IO::raw*)colmean, out, L, D, BLK, nblk);
 }
 
+// levels 2 and 3 of the K column mean from the chunk sums
+template <typename IO>
+static void launch_colmean_reduce(float* chunk_sums, float* group_sums, typename IO::raw* colmean, int BH, int L, int D,
+                                  hipStream_t st) {
+  const int nchunk = cdiv(L, KMEAN_CHUNK), ngroup = cdiv(nchunk, KMEAN_GROUP);
+  if (D <= 1024 && 1024 % D == 0 && ngroup * D <= COLMEAN_LDS_FLOATS) {
+    hipLaunchKernelGGL((colmean_fused_kernel<IO>), dim3(BH), dim3(1024), 0, st, chunk_sums, colmean, nchunk, ngroup, D, L);
+    return;
+  }
+  hipLaunchKernelGGL(colmean_group_kernel, dim3(ngroup, BH), dim3(128), 0, st, chunk_sums, group_sums, nchunk, ngroup, D);
+  hipLaunchKernelGGL((colmean_kernel<IO>), dim3(cdiv(D, 128), BH), dim3(128), 0, st, group_sums, colmean, ngroup, D, L);
+}
+
 template <typename IO>
 static void launch_k_colmean_t(const void* k, int BH, int L, int D, float* chunk_sums, float* group_sums,
                                typename IO::raw* colmean, hipStream_t st) {
-  const int nchunk = cdiv(L, KMEAN_CHUNK), ngroup = cdiv(nchunk, KMEAN_GROUP);
   launch_pool<IO, 0>(k, nullptr, chunk_sums, BH, L, D, KMEAN_CHUNK, st);
-  hipLaunchKernelGGL(colmean_group_kernel, dim3(ngroup, BH), dim3(128), 0, st, chunk_sums, group_sums, nchunk, ngroup, D);
-  hipLaunchKernelGGL((colmean_kernel<IO>), dim3(cdiv(D, 128), BH), dim3(128), 0, st, group_sums, colmean, ngroup, D, L);
+  launch_colmean_reduce<IO>(chunk_sums, group_sums, colmean, BH, L, D, st);
 }
 
 template <typename IO>
@@ -359,8 +430,15 @@ static int block_map_impl(const void* q, const void* k, int dtype, int BH, int L
   typename IO::raw* pq = (typename IO::raw*)(ws + w.pq);
   typename IO::raw* pk = (typename IO::raw*)(ws + w.pk);
   typename IO::raw* score = (typename IO::raw*)(ws + w.score);
-  launch_k_colmean_t<IO>(k, BH, L, D, chunk_sums, (float*)(ws + w.group_sums), colmean, st);
-  launch_pool<IO, 1>(q, nullptr, pq, BH, L, D, BLKQ, st);
+  {
+    // k chunk sums and q block means share one launch
+    const int nchunk = cdiv(L, KMEAN_CHUNK);
+    const int bpw = 256 / (D / IO::VEC);
+    dim3 grid(cdiv(max(nchunk, M), bpw), BH, 2);
+    hipLaunchKernelGGL((pool_pair_kernel<IO>), grid, dim3(256), 0, st, (const typename IO::raw*)k, chunk_sums, nchunk,
+                       (const typename IO::raw*)q, pq, BLKQ, M, L, D);
+  }
+  launch_colmean_reduce<IO>(chunk_sums, (float*)(ws + w.group_sums), colmean, BH, L, D, st);
   launch_pool<IO, 2>(k, colmean, pk, BH, L, D, BLKK, st);
   hipLaunchKernelGGL((score_kernel<IO>), dim3(cdiv(N, 64), cdiv(M, 64), BH), dim3(256), 0, st, pq, pk, score, M, N, D);
   // topk == 0 selects nothing: the kernel then only clears the map row.
