@@ -31,7 +31,7 @@ PEAK_HBM_GBS = 8000.0
 # the 1 GiB-read / 1 GiB-write elementwise kernel of --pmc-calibration (FETCH_SIZE x2.0, WRITE_SIZE x1.0).
 # It is a property of the kernel and the workload, not re-measured by a plain bench run.
 MEASURED_TRAFFIC_BYTES = {
-    "cfg3": {"kernel": "sparse_fwd_kernel", "fetch": 201962.4 * 1024 * 2.0, "write": 100071.1 * 1024 * 1.0},
+    "cfg3": {"kernel": "sparse_fwd_kernel<FUSED>", "fetch": 211642.1 * 1024 * 2.0, "write": 100080.5 * 1024 * 1.0},
 }
 
 
@@ -104,7 +104,8 @@ def main():
     from sla_amd import SparseLinearAttention, get_block_map
     from sla_amd.inputs import CONFIGS, make_inputs, make_proj
     from sla_amd.linear import linear_fwd
-    from sla_amd.sparse_attn import sparse_attn_fwd
+    from sla_amd.linear import linear_state_fwd
+    from sla_amd.sparse_attn import sparse_attn_fwd, sparse_attn_linear_fwd
 
     cfg = CONFIGS[args.workload]
     dev = torch.device("cuda:0")
@@ -125,12 +126,16 @@ def main():
     dense_flops = 4.0 * B * H * L * L * D
     eff_tflops = dense_flops / ms_fwd / 1e9
 
-    # ---- dominant kernel: block-sparse forward, timed alone with events on its stream ----
+    # ---- dominant kernel: the attention kernel the module launches (block-sparse forward with the linear
+    # branch, projection and sum in its epilogue), timed alone with events on its stream ----
     m, lut, T = get_block_map(q, k, cfg.topk, cfg.BLKQ, cfg.BLKK)
     scale = D ** -0.5
-    ms_sparse = time_region(torch, lambda: sparse_attn_fwd(q, k, v, lut, T, cfg.BLKQ, cfg.BLKK, scale), args.steps,
-                            args.warmup)
-    sparse_flops = 4.0 * B * H * M * T * cfg.BLKQ * cfg.BLKK * D
+    wdev, bdev = mod.proj_l.weight.detach().contiguous(), mod.proj_l.bias.detach().contiguous()
+    state_ws = linear_state_fwd(k, v, wdev, cfg.feature_map)
+    ms_sparse = time_region(torch, lambda: sparse_attn_linear_fwd(q, k, v, lut, T, cfg.BLKQ, cfg.BLKK, scale, state_ws,
+                                                                  bdev, cfg.feature_map, False), args.steps, args.warmup)
+    # executed MFMA work: QK^T and PV over the selected tiles + phi(q) KVW of the epilogue
+    sparse_flops = 4.0 * B * H * M * T * cfg.BLKQ * cfg.BLKK * D + 2.0 * B * H * L * D * D
     achieved = sparse_flops / ms_sparse / 1e9
     out = {
         "metric": "sla_forward_effective_tflops",
@@ -145,19 +150,23 @@ def main():
                      "frac": achieved / PEAK_BF16_TFLOPS,
                      "traffic": (sum(v for k_, v in MEASURED_TRAFFIC_BYTES[cfg.name].items() if k_ != "kernel")
                                  if cfg.name in MEASURED_TRAFFIC_BYTES else None),
-                     "traffic_unit": "HBM bytes per launch (fetch + write)", "kernel": "sparse_fwd_kernel",
+                     "traffic_unit": "HBM bytes per launch (fetch + write)", "kernel": "sparse_fwd_kernel<FUSED=true>",
                      "flops_per_launch": sparse_flops, "ms_per_launch": ms_sparse},
     }
-    extra = {"sla_fwd_ms": ms_fwd, "sparse_fwd_ms": ms_sparse}
+    extra = {"sla_fwd_ms": ms_fwd, "attention_fused_ms": ms_sparse}
     if not args.no_extras:
         extra["mask_ms"] = time_region(torch, lambda: get_block_map(q, k, cfg.topk, cfg.BLKQ, cfg.BLKK), args.steps,
                                        args.warmup)
         extra["mask_hbm_gbs"] = 2.0 * q.numel() * 2 / extra["mask_ms"] / 1e6
+        extra["sparse_fwd_alone_ms"] = time_region(torch, lambda: sparse_attn_fwd(q, k, v, lut, T, cfg.BLKQ, cfg.BLKK, scale),
+                                                   args.steps, args.warmup)
+        extra["linear_state_ms"] = time_region(torch, lambda: linear_state_fwd(k, v, wdev, cfg.feature_map), args.steps,
+                                               args.warmup)
+        extra["state_hbm_gbs"] = 2.0 * q.numel() * 2 / extra["linear_state_ms"] / 1e6
         o_s, _ = sparse_attn_fwd(q, k, v, lut, T, cfg.BLKQ, cfg.BLKK, scale)
-        wd, bd = mod.proj_l.weight.detach(), mod.proj_l.bias.detach()
-        extra["linear_proj_sum_ms"] = time_region(torch, lambda: linear_fwd(q, k, v, wd, bd, o_s, cfg.feature_map),
-                                                  args.steps, args.warmup)
-        extra["mfma_frac_module_fwd"] = (sparse_flops + 6.0 * B * H * L * D * D) / ms_fwd / 1e9 / PEAK_BF16_TFLOPS
+        extra["linear_proj_sum_unfused_ms"] = time_region(torch, lambda: linear_fwd(q, k, v, wdev, bdev, o_s, cfg.feature_map),
+                                                          args.steps, args.warmup)
+        extra["mfma_frac_module_fwd"] = (sparse_flops + 2.0 * B * H * L * D * D) / ms_fwd / 1e9 / PEAK_BF16_TFLOPS
         try:
             qg, kg, vg = (t.clone().requires_grad_(True) for t in (q, k, v))
 

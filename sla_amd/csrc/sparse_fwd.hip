@@ -18,9 +18,9 @@ namespace sla {
 
 // What the fused variant (FUSED = true) adds after the loop: the linear branch of the same query rows,
 // out = o_s + (phi(q) KVW / divisor + bias), from the per-head state the linear state kernels left in
-// their workspace (kvwt: KVW^T in 16 bit, zst: sum phi(k) in 16 bit).  The state is staged in the LDS the
-// K/V tiles no longer need, the raw q fragments are still in registers, and the product costs as many
-// MFMAs as one more key tile.  o then receives the sum; o_s (optional) the attention output alone.
+// their workspace (kvwt: KVW^T in 16 bit, zst: sum phi(k) in 16 bit).  The state is read from L2 in
+// operand order, the raw q fragments are still in registers, and the product costs as many MFMAs as one
+// more key tile.  o then receives the sum; o_s (optional) the attention output alone.
 template <typename Tag, int D, int BLKQ, bool FUSED>
 __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))) void sparse_fwd_kernel(const uint16_t* __restrict__ q,
                                                               const uint16_t* __restrict__ k,
@@ -46,7 +46,6 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
   __shared__ __attribute__((aligned(16))) uint16_t smem[BLKK * KSTR + BLKK * VSTR];
   uint16_t* const sK = smem;
   uint16_t* const sV = smem + BLKK * KSTR;
-  static_assert(D * (D + 8) <= BLKK * KSTR + BLKK * VSTR, "the folded state must fit where the K/V tiles were");
 
   const int logical = xcd_remap(blockIdx.x, gridDim.x, total);
   if (logical < 0) return;
@@ -303,22 +302,12 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
       if (g == 0) lse[(size_t)bh * L + qrow] = m_run + fast_log2(l_tot);
     }
   } else {
-    // ---- linear branch of the same rows (the loop's last barrier has freed the tile buffers) ----
-    constexpr int SSTR = D + 8;
-    __shared__ float sZ[D];
-    __shared__ float sBias[D];
-    {
-      const uint16_t* src = kvwt + (size_t)bh * D * D;
-      for (int idx = tid; idx < D * D / 8; idx += NT) {
-        const int row = idx / (D / 8), col = (idx % (D / 8)) * 8;
-        *reinterpret_cast<i16x8_t*>(&smem[row * SSTR + col]) = *reinterpret_cast<const i16x8_t*>(src + (size_t)row * D + col);
-      }
-      for (int d = tid; d < D; d += NT) {
-        sZ[d] = E::to_float(zst[(size_t)bh * D + d]);
-        sBias[d] = round16<Tag>(bias[d]);
-      }
-    }
-    __syncthreads();
+    // ---- linear branch of the same rows ----
+    // The per-head state (32 KB) is read straight from L2 in MFMA A-operand order (row 32et + r, 16-byte
+    // chunk 2c + g): no staging, no barrier, so the other workgroups of the compute unit keep running
+    // their loops while this wave waits for its loads.
+    const uint16_t* st_h = kvwt + (size_t)bh * D * D;
+    const uint16_t* z_h = zst + (size_t)bh * D;
     // phi(q) from the resident raw q fragments: this lane holds d = 16c + 8g + j of its row
     float f[DC][8];
 #pragma unroll
@@ -330,9 +319,10 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
     float den = 0.f;
 #pragma unroll
     for (int c = 0; c < DC; ++c) {
+      const i16x8_t zc = *reinterpret_cast<const i16x8_t*>(z_h + 16 * c + 8 * g);
       i32x4_t pw;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) den += round16<Tag>(f[c][j] * sZ[16 * c + 8 * g + j]);
+      for (int j = 0; j < 8; ++j) den += round16<Tag>(f[c][j] * E::to_float((uint16_t)zc[j]));
 #pragma unroll
       for (int j = 0; j < 4; ++j) pw[j] = (int)E::pack2(f[c][2 * j], f[c][2 * j + 1]);
       qf[c] = __builtin_bit_cast(i16x8_t, pw);
@@ -344,18 +334,19 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
     const size_t off = head_off + (size_t)qrow * D;
 #pragma unroll
     for (int et = 0; et < DT; ++et) {
+      i16x8_t a[DC];
+#pragma unroll
+      for (int c = 0; c < DC; ++c) a[c] = *reinterpret_cast<const i16x8_t*>(st_h + (size_t)(32 * et + r) * D + 16 * c + 8 * g);
       f32x16_t acc;
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[i] = 0.f;
 #pragma unroll
-      for (int c = 0; c < DC; ++c) {
-        const i16x8_t a = *reinterpret_cast<const i16x8_t*>(&smem[(32 * et + r) * SSTR + 16 * c + 8 * g]);
-        acc = E::mfma32(a, qf[c], acc);
-      }
+      for (int c = 0; c < DC; ++c) acc = E::mfma32(a[c], qf[c], acc);
       if (ok) {
 #pragma unroll
         for (int i4 = 0; i4 < 4; ++i4) {
           const int e0 = 32 * et + 8 * i4 + 4 * g;
+          const f32x4_t b4 = *reinterpret_cast<const f32x4_t*>(bias + e0);
           i32x2_t ws, wo;
           ws[0] = (int)E::pack2(oacc[et][4 * i4 + 0] * inv, oacc[et][4 * i4 + 1] * inv);
           ws[1] = (int)E::pack2(oacc[et][4 * i4 + 2] * inv, oacc[et][4 * i4 + 3] * inv);
@@ -364,8 +355,8 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
 #pragma unroll
           for (int h = 0; h < 2; ++h) {
             const uint32_t x = (uint32_t)ws[h];
-            const float l0 = round16<Tag>(pin_f32(__builtin_fmaf(acc[4 * i4 + 2 * h], inv_den, sBias[e0 + 2 * h])));
-            const float l1 = round16<Tag>(pin_f32(__builtin_fmaf(acc[4 * i4 + 2 * h + 1], inv_den, sBias[e0 + 2 * h + 1])));
+            const float l0 = round16<Tag>(pin_f32(__builtin_fmaf(acc[4 * i4 + 2 * h], inv_den, round16<Tag>(b4[2 * h]))));
+            const float l1 = round16<Tag>(pin_f32(__builtin_fmaf(acc[4 * i4 + 2 * h + 1], inv_den, round16<Tag>(b4[2 * h + 1]))));
             wo[h] = (int)E::pack2(E::to_float((uint16_t)(x & 0xffff)) + l0, E::to_float((uint16_t)(x >> 16)) + l1);
           }
           *reinterpret_cast<i32x2_t*>(o + off + e0) = wo;
