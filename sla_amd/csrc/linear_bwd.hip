@@ -248,6 +248,29 @@ __global__ __launch_bounds__(256) void linear_bwd_states_kernel(
   const int tr_row = (lane & 15) >> 2;
   const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
 
+  // rows of the next tile are fetched into registers while the current tile is multiplied
+  i16x8_t rq[NP], rdn[NP], rg[NP], ry[NP];
+  float rdd[NP];
+  auto fetch = [&](int r0) {
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
+      const int grow = r0 + lrow + p * RPP;
+      rq[p] = i16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+      rdn[p] = rq[p];
+      rg[p] = rq[p];
+      ry[p] = rq[p];
+      rdd[p] = 0.f;
+      if (grow < row_end) {
+        const size_t off = head_off + (size_t)grow * D + lcol;
+        rq[p] = *reinterpret_cast<const i16x8_t*>(q + off);
+        rdn[p] = *reinterpret_cast<const i16x8_t*>(dn + off);
+        rg[p] = *reinterpret_cast<const i16x8_t*>(gout + off);
+        ry[p] = *reinterpret_cast<const i16x8_t*>(y + off);
+        rdd[p] = dden[(size_t)bh * L + grow];
+      }
+    }
+  };
+  if (row_begin < row_end) fetch(row_begin);
   for (int r0 = row_begin; r0 < row_end; r0 += TR) {
     __syncthreads();
 #pragma unroll
@@ -255,16 +278,8 @@ __global__ __launch_bounds__(256) void linear_bwd_states_kernel(
       const int row = lrow + p * RPP;
       const int grow = r0 + row;
       const bool ok = grow < row_end;
-      i16x8_t xq = {0, 0, 0, 0, 0, 0, 0, 0}, xdn = xq, xg = xq, xy = xq;
-      float dd = 0.f;
-      if (ok) {
-        const size_t off = head_off + (size_t)grow * D + lcol;
-        xq = *reinterpret_cast<const i16x8_t*>(q + off);
-        xdn = *reinterpret_cast<const i16x8_t*>(dn + off);
-        xg = *reinterpret_cast<const i16x8_t*>(gout + off);
-        xy = *reinterpret_cast<const i16x8_t*>(y + off);
-        dd = dden[(size_t)bh * L + grow];
-      }
+      const i16x8_t xq = rq[p], xdn = rdn[p], xg = rg[p], xy = ry[p];
+      const float dd = rdd[p];
       float f[8];
 #pragma unroll
       for (int e = 0; e < 8; ++e) f[e] = E::to_float((uint16_t)xq[e]);
@@ -303,6 +318,7 @@ __global__ __launch_bounds__(256) void linear_bwd_states_kernel(
       *reinterpret_cast<i16x8_t*>(&sY[row * STR + lcol]) = xy;
     }
     __syncthreads();
+    if (r0 + TR < row_end) fetch(r0 + TR);     // after the barrier: its fence would wait for these loads
 #pragma unroll
     for (int c = 0; c < TR / 16; ++c) {
       const int l0 = 16 * c + 8 * g + tr_row;

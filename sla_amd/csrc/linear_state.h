@@ -107,8 +107,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
       *reinterpret_cast<i16x8_t*>(&sK[row * STR + lcol]) = fk;
       *reinterpret_cast<i16x8_t*>(&sV[row * STR + lcol]) = vv;
     }
-    if (r0 + TR < row_end) fetch(r0 + TR);
     __syncthreads();
+    if (r0 + TR < row_end) fetch(r0 + TR);     // after the barrier: its fence would wait for these loads
 #pragma unroll
     for (int c = 0; c < TR / 16; ++c) {
       const int l0 = 16 * c + 8 * g + tr_row;
