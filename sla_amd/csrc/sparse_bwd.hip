@@ -203,6 +203,8 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
         s[i] = 0.f;
         dp[i] = 0.f;
       }
+      // (the group barriers fix the issue order: LDS reads run two fragments ahead of the MFMAs that use them)
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int c = 0; c < DC; ++c) {
         const i16x8_t a = *reinterpret_cast<const i16x8_t*>(&sK[(32 * t + r) * KSTR + 16 * c + 8 * g]);
@@ -210,6 +212,14 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
         const i16x8_t b = *reinterpret_cast<const i16x8_t*>(&sV[(32 * t + r) * VSTR + 16 * c + 8 * g]);
         dp = E::mfma32(b, dof[c], dp);
       }
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+#pragma unroll
+      for (int i = 0; i < 2 * DC - 2; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+      __builtin_amdgcn_sched_barrier(0);
       // dS^T = P^T * (dP^T - delta).  Key rows past L need no masking: their K rows are zero in LDS, so
       // whatever (finite) dS they get is multiplied by zero in dQ^T += K^T dS^T.
 #pragma unroll
@@ -217,19 +227,32 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
         const float p = fast_exp2(__builtin_fmaf(s[i], c_log2e, -lse_q));
         s[i] = p * (dp[i] - delta_q);
       }
+      i16x8_t dsb[2];
 #pragma unroll
       for (int c2 = 0; c2 < 2; ++c2) {
         i32x4_t pw;
 #pragma unroll
         for (int j = 0; j < 4; ++j) pw[j] = (int)E::pack2(s[8 * c2 + 2 * j], s[8 * c2 + 2 * j + 1]);
-        const i16x8_t dsb = __builtin_bit_cast(i16x8_t, pw);
+        dsb[c2] = __builtin_bit_cast(i16x8_t, pw);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int c2 = 0; c2 < 2; ++c2) {
         const int key0 = 32 * t + 16 * c2 + 4 * g + tr_row;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
           const uint16_t* p0 = &sK[key0 * KSTR + 32 * dt + tr_col];
-          dqacc[dt] = E::mfma32(concat4(lds_read_tr16(p0), lds_read_tr16(p0 + 8 * KSTR)), dsb, dqacc[dt]);
+          dqacc[dt] = E::mfma32(concat4(lds_read_tr16(p0), lds_read_tr16(p0 + 8 * KSTR)), dsb[c2], dqacc[dt]);
         }
       }
+      __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+      for (int i = 0; i < 2 * DT - 2; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+      __builtin_amdgcn_sched_barrier(0);
     }
     __syncthreads();                       // both tiles fully consumed
     if (more) store_tile();
@@ -373,6 +396,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       s[i] = 0.f;
       dp[i] = 0.f;
     }
+    // (the group barriers fix the issue order: LDS reads run a few fragments ahead of the MFMAs that use them)
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int c = 0; c < DC; ++c) {
       const i16x8_t a = *reinterpret_cast<const i16x8_t*>(&sQ[(32 * dh + r) * STR + 16 * c + 8 * g]);
@@ -380,6 +405,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       const i16x8_t b = *reinterpret_cast<const i16x8_t*>(&sDO[(32 * dh + r) * STR + 16 * c + 8 * g]);
       dp = E::mfma32(b, vf[c], dp);
     }
+    __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+    for (int i = 0; i < 2 * DC - 4; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+    __builtin_amdgcn_sched_barrier(0);
     // accumulator rows are queries 32dh + 8*(i/4) + 4g + i%4; this lane's column is its key
 #pragma unroll
     for (int i4 = 0; i4 < 4; ++i4) {
@@ -421,6 +454,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           dsb = sXS[wave ^ 2][c2][lane];
         }
         const int q0 = 32 * h + 16 * c2 + 4 * g + tr_row;
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int dt = 0; dt < DH; ++dt) {
           const int dcol = 32 * (DH * dh + dt) + tr_col;
@@ -429,6 +463,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           const uint16_t* pq = &sQ[q0 * STR + dcol];
           dkacc[dt] = E::mfma32(concat4(lds_read_tr16(pq), lds_read_tr16(pq + 8 * STR)), dsb, dkacc[dt]);
         }
+        // all eight transposing reads of this 16-row group first, then its four MFMAs
+        __builtin_amdgcn_sched_group_barrier(0x100, 4 * DH, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 2 * DH, 0);
+        __builtin_amdgcn_sched_barrier(0);
       }
     __syncthreads();                       // tile and exchange buffers fully consumed
     if (ti + 1 < ntile) store_tile();
