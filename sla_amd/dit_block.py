@@ -9,7 +9,6 @@ projections are plain library GEMMs; the layout changes are single fused copies 
 """
 from __future__ import annotations
 
-import torch
 import torch.nn as nn
 
 from .module import SparseLinearAttention

@@ -6,7 +6,7 @@ import torch
 import torch.nn as nn
 
 from .block_map import get_block_map
-from .linear import linear_bwd, linear_complement_fwd, linear_out_fwd, linear_state_fwd
+from .linear import linear_bwd, linear_complement_fwd, linear_state_fwd
 from .sparse_attn import sparse_attn_bwd, sparse_attn_fwd, sparse_attn_linear_fwd
 
 FEATURE_MAPS = ("elu", "relu", "softmax")
