@@ -60,15 +60,19 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
 
   const size_t head_off = (size_t)bh * L * D;
   const uint32_t head_bytes = (uint32_t)L * D * 2;
-  const __amdgpu_buffer_rsrc_t qh = make_rsrc(q + head_off, head_bytes);
   const __amdgpu_buffer_rsrc_t kh = make_rsrc(k + head_off, head_bytes);
   const __amdgpu_buffer_rsrc_t vh = make_rsrc(v + head_off, head_bytes);
 
-  // Q^T fragments (B operand), resident for the whole loop.
-  const int qrow = mb * BLKQ + wave * 32 + r;
-  i16x8_t qf[DC];
-#pragma unroll
-  for (int c = 0; c < DC; ++c) qf[c] = buf_load_b128(qh, ((uint32_t)qrow * D + 16 * c + 8 * g) * 2);   // rows past L: 0
+  // This wave's 32 query rows.  Q comes in and O goes out as whole 256-byte rows (16 adjacent lanes per
+  // row) through a wave-private staging tile in LDS: a lane-per-row access pattern would touch 32 memory
+  // lines with every instruction.
+  const int qrow0 = mb * BLKQ + wave * 32;
+  const int qrow = qrow0 + r;
+  const int qrows_valid = min(32, L - qrow0);
+  uint16_t* const stage = smem + wave * 32 * TileRows<D>::SSTR;
+  static_assert(BLKQ / 32 * 32 * TileRows<D>::SSTR <= BLKK * KSTR + BLKK * VSTR, "staging tiles exceed the K/V buffers");
+  TileRows<D> qt;
+  qt.fetch(q + head_off + (size_t)qrow0 * D, qrows_valid, lane);   // rows past L: 0
 
   const size_t lut_row = ((size_t)bh * Mblk + mb) * topk;
   auto lut_at = [&](int i) -> int {
@@ -79,23 +83,25 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
   // One set of staging registers carries K of the next tile during the QK^T phase and V of the
   // next tile during the PV phase (each LDS buffer is free while the other one is being read).
   i16x8_t stg[NLD];
-  auto load_rows = [&](const __amdgpu_buffer_rsrc_t& base, int nb) {
+  auto load_rows_to = [&](i16x8_t (&dst)[NLD], const __amdgpu_buffer_rsrc_t& base, int nb) {
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
       const int idx = tid + i * NT;
       const int row = idx / CPR, col = (idx % CPR) * 8;
       // rows past L lie beyond the buffer range and read as zero (0 * garbage could be NaN)
-      stg[i] = buf_load_b128(base, ((uint32_t)(nb * BLKK + row) * D + col) * 2);
+      dst[i] = buf_load_b128(base, ((uint32_t)(nb * BLKK + row) * D + col) * 2);
     }
   };
-  auto store_rows = [&](uint16_t* dst, int stride) {
+  auto store_rows_from = [&](const i16x8_t (&src)[NLD], uint16_t* dst, int stride) {
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
       const int idx = tid + i * NT;
       const int row = idx / CPR, col = (idx % CPR) * 8;
-      *reinterpret_cast<i16x8_t*>(&dst[row * stride + col]) = stg[i];
+      *reinterpret_cast<i16x8_t*>(&dst[row * stride + col]) = src[i];
     }
   };
+  auto load_rows = [&](const __amdgpu_buffer_rsrc_t& base, int nb) { load_rows_to(stg, base, nb); };
+  auto store_rows = [&](uint16_t* dst, int stride) { store_rows_from(stg, dst, stride); };
 
   f32x16_t oacc[DT];
 #pragma unroll
@@ -111,11 +117,17 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
   // the address computation of the K/V loads
   int nb = topk > 0 ? lut_at(0) : 0;
   int nb_next = topk > 1 ? lut_at(1) : 0;
-  if (topk > 0) {
-    load_rows(kh, nb);
-    store_rows(sK, KSTR);
-    load_rows(vh, nb);
-  }
+  // Q and K of the first tile are in flight together; V follows as soon as Q has been parked
+  i16x8_t stg_first[NLD];
+  if (topk > 0) load_rows_to(stg_first, kh, nb);
+  // Q^T fragments (B operand), resident for the whole loop
+  qt.park(stage, lane);
+  i16x8_t qf[DC];
+#pragma unroll
+  for (int c = 0; c < DC; ++c) qf[c] = *reinterpret_cast<const i16x8_t*>(&stage[r * TileRows<D>::SSTR + 16 * c + 8 * g]);
+  if (topk > 0) load_rows(vh, nb);
+  __syncthreads();                         // the staging tiles overlap the K buffer
+  if (topk > 0) store_rows_from(stg_first, sK, KSTR);
   __syncthreads();
 
   // Reference maximum of the online softmax.  It is only moved when a sub-tile's maximum exceeds it
@@ -287,20 +299,32 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
   // ---- epilogue ----
   const float l_tot = l_run + __shfl_xor(l_run, 32);
   const float inv = 1.0f / l_tot;
+  // (the loop ended with a barrier: every wave is done with the K/V buffers, the staging tiles are free)
+  constexpr int SSTR = TileRows<D>::SSTR;
+  const size_t tile_off = head_off + (size_t)qrow0 * D;
+  if (qrow < L && g == 0) lse[(size_t)bh * L + qrow] = m_run + fast_log2(l_tot);
+  // normalised attention output of this lane, packed, into its row of the staging tile
+  auto park_attention = [&]() {
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; ++i4) {
+        i32x2_t w;
+        w[0] = (int)E::pack2(oacc[dt][4 * i4 + 0] * inv, oacc[dt][4 * i4 + 1] * inv);
+        w[1] = (int)E::pack2(oacc[dt][4 * i4 + 2] * inv, oacc[dt][4 * i4 + 3] * inv);
+        *reinterpret_cast<i32x2_t*>(&stage[r * SSTR + 32 * dt + 8 * i4 + 4 * g]) = w;
+      }
+    wave_lds_fence();
+  };
+  auto flush_rows = [&](uint16_t* dst) {   // staging tile -> global rows
+    TileRows<D> t;
+    t.unpark(stage, lane);
+    t.store(dst + tile_off, qrows_valid, lane);
+    wave_lds_fence();
+  };
   if (!FUSED) {
-    if (qrow < L) {
-      uint16_t* orow = o + head_off + (size_t)qrow * D;
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-        for (int i4 = 0; i4 < 4; ++i4) {
-          i32x2_t w;
-          w[0] = (int)E::pack2(oacc[dt][4 * i4 + 0] * inv, oacc[dt][4 * i4 + 1] * inv);
-          w[1] = (int)E::pack2(oacc[dt][4 * i4 + 2] * inv, oacc[dt][4 * i4 + 3] * inv);
-          *reinterpret_cast<i32x2_t*>(orow + 32 * dt + 8 * i4 + 4 * g) = w;
-        }
-      if (g == 0) lse[(size_t)bh * L + qrow] = m_run + fast_log2(l_tot);
-    }
+    park_attention();
+    flush_rows(o);
   } else {
     // ---- linear branch of the same rows ----
     // The per-head state (32 KB) is read straight from L2 in MFMA A-operand order (row 32et + r, 16-byte
@@ -330,8 +354,6 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
     den += __shfl_xor(den, 32);
     den = round16<Tag>(1e-5f + round16<Tag>(den));
     const float inv_den = 1.0f / den;
-    const bool ok = qrow < L;
-    const size_t off = head_off + (size_t)qrow * D;
 #pragma unroll
     for (int et = 0; et < DT; ++et) {
       i16x8_t a[DC];
@@ -342,28 +364,30 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
       for (int i = 0; i < 16; ++i) acc[i] = 0.f;
 #pragma unroll
       for (int c = 0; c < DC; ++c) acc = E::mfma32(a[c], qf[c], acc);
-      if (ok) {
 #pragma unroll
-        for (int i4 = 0; i4 < 4; ++i4) {
-          const int e0 = 32 * et + 8 * i4 + 4 * g;
-          const f32x4_t b4 = *reinterpret_cast<const f32x4_t*>(bias + e0);
-          i32x2_t ws, wo;
-          ws[0] = (int)E::pack2(oacc[et][4 * i4 + 0] * inv, oacc[et][4 * i4 + 1] * inv);
-          ws[1] = (int)E::pack2(oacc[et][4 * i4 + 2] * inv, oacc[et][4 * i4 + 3] * inv);
-          if (o_s) *reinterpret_cast<i32x2_t*>(o_s + off + e0) = ws;
-          // the sum as the reference's tensor addition forms it: both summands in 16 bit, one rounded add
+      for (int i4 = 0; i4 < 4; ++i4) {
+        const int e0 = 32 * et + 8 * i4 + 4 * g;
+        const f32x4_t b4 = *reinterpret_cast<const f32x4_t*>(bias + e0);
+        i32x2_t ws, wo;
+        ws[0] = (int)E::pack2(oacc[et][4 * i4 + 0] * inv, oacc[et][4 * i4 + 1] * inv);
+        ws[1] = (int)E::pack2(oacc[et][4 * i4 + 2] * inv, oacc[et][4 * i4 + 3] * inv);
+        // the sum as the reference's tensor addition forms it: both summands in 16 bit, one rounded add
 #pragma unroll
-          for (int h = 0; h < 2; ++h) {
-            const uint32_t x = (uint32_t)ws[h];
-            const float l0 = round16<Tag>(pin_f32(__builtin_fmaf(acc[4 * i4 + 2 * h], inv_den, round16<Tag>(b4[2 * h]))));
-            const float l1 = round16<Tag>(pin_f32(__builtin_fmaf(acc[4 * i4 + 2 * h + 1], inv_den, round16<Tag>(b4[2 * h + 1]))));
-            wo[h] = (int)E::pack2(E::to_float((uint16_t)(x & 0xffff)) + l0, E::to_float((uint16_t)(x >> 16)) + l1);
-          }
-          *reinterpret_cast<i32x2_t*>(o + off + e0) = wo;
+        for (int h = 0; h < 2; ++h) {
+          const uint32_t x = (uint32_t)ws[h];
+          const float l0 = round16<Tag>(pin_f32(__builtin_fmaf(acc[4 * i4 + 2 * h], inv_den, round16<Tag>(b4[2 * h]))));
+          const float l1 = round16<Tag>(pin_f32(__builtin_fmaf(acc[4 * i4 + 2 * h + 1], inv_den, round16<Tag>(b4[2 * h + 1]))));
+          wo[h] = (int)E::pack2(E::to_float((uint16_t)(x & 0xffff)) + l0, E::to_float((uint16_t)(x >> 16)) + l1);
         }
+        *reinterpret_cast<i32x2_t*>(&stage[r * SSTR + e0]) = wo;
       }
     }
-    if (ok && g == 0) lse[(size_t)bh * L + qrow] = m_run + fast_log2(l_tot);
+    wave_lds_fence();
+    flush_rows(o);
+    if (o_s) {
+      park_attention();
+      flush_rows(o_s);
+    }
   }
 }
 
