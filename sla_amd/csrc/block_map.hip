@@ -190,7 +190,7 @@ __global__ __launch_bounds__(1024) void colmean_fused_kernel(const float* __rest
   }
 }
 
-// score[bh][m][n] = round_dtype( sum_d pq[m][d]*pk[n][d] ), d ascending, mul and add rounded separately.
+// score[bh][m][n] = round_dtype( sum_d pq[m][d]*pk[n][d] ), d ascending, every product and every sum rounded to fp32.
 // 64x64 outputs per workgroup, 4x4 per thread, operands staged through LDS 32 columns at a time.
 template <typename IO>
 __global__ __launch_bounds__(256) void score_kernel(const typename IO::raw* __restrict__ pq,
@@ -227,8 +227,14 @@ __global__ __launch_bounds__(256) void score_kernel(const typename IO::raw* __re
       for (int i = 0; i < 4; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          const float prod = a[i] * b[j];
-          acc[i][j] = acc[i][j] + prod;
+          if (sizeof(typename IO::raw) == 2) {
+            // the product of two 16-bit values is exact in fp32 (above the subnormal range), so the fused
+            // form rounds the same sum once, exactly as the separate addition does, in half the instructions
+            acc[i][j] = __builtin_fmaf(a[i], b[j], acc[i][j]);
+          } else {
+            const float prod = a[i] * b[j];
+            acc[i][j] = acc[i][j] + prod;
+          }
         }
     }
   }

@@ -297,12 +297,22 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
   const float m_run = m_used;
 
   // ---- epilogue ----
+  // (lane-derived indices are formed again from an opaque copy of the thread id, so that none of them is
+  //  kept in a register, or spilled, across the loop)
+  int tid_e = tid;
+  asm volatile("" : "+v"(tid_e));
+  const int lane_e = tid_e & 63, wave_e = tid_e >> 6;
+  const int g_e = lane_e >> 5, r_e = lane_e & 31;
+  uint16_t* const stage_e = smem + wave_e * 32 * TileRows<D>::SSTR;
+  const int qrow0_e = mb * BLKQ + wave_e * 32;
+  const int qrow_e = qrow0_e + r_e;
+  const int qrows_valid_e = min(32, L - qrow0_e);
   const float l_tot = l_run + __shfl_xor(l_run, 32);
   const float inv = 1.0f / l_tot;
   // (the loop ended with a barrier: every wave is done with the K/V buffers, the staging tiles are free)
   constexpr int SSTR = TileRows<D>::SSTR;
-  const size_t tile_off = head_off + (size_t)qrow0 * D;
-  if (qrow < L && g == 0) lse[(size_t)bh * L + qrow] = m_run + fast_log2(l_tot);
+  const size_t tile_off = head_off + (size_t)qrow0_e * D;
+  if (qrow_e < L && g_e == 0) lse[(size_t)bh * L + qrow_e] = m_run + fast_log2(l_tot);
   // normalised attention output of this lane, packed, into its row of the staging tile
   auto park_attention = [&]() {
 #pragma unroll
@@ -312,14 +322,14 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
         i32x2_t w;
         w[0] = (int)E::pack2(oacc[dt][4 * i4 + 0] * inv, oacc[dt][4 * i4 + 1] * inv);
         w[1] = (int)E::pack2(oacc[dt][4 * i4 + 2] * inv, oacc[dt][4 * i4 + 3] * inv);
-        *reinterpret_cast<i32x2_t*>(&stage[r * SSTR + 32 * dt + 8 * i4 + 4 * g]) = w;
+        *reinterpret_cast<i32x2_t*>(&stage_e[r_e * SSTR + 32 * dt + 8 * i4 + 4 * g_e]) = w;
       }
     wave_lds_fence();
   };
   auto flush_rows = [&](uint16_t* dst) {   // staging tile -> global rows
     TileRows<D> t;
-    t.unpark(stage, lane);
-    t.store(dst + tile_off, qrows_valid, lane);
+    t.unpark(stage_e, lane_e);
+    t.store(dst + tile_off, qrows_valid_e, lane_e);
     wave_lds_fence();
   };
   if (!FUSED) {
@@ -343,7 +353,7 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
     float den = 0.f;
 #pragma unroll
     for (int c = 0; c < DC; ++c) {
-      const i16x8_t zc = *reinterpret_cast<const i16x8_t*>(z_h + 16 * c + 8 * g);
+      const i16x8_t zc = *reinterpret_cast<const i16x8_t*>(z_h + 16 * c + 8 * g_e);
       i32x4_t pw;
 #pragma unroll
       for (int j = 0; j < 8; ++j) den += round16<Tag>(f[c][j] * E::to_float((uint16_t)zc[j]));
@@ -358,7 +368,7 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
     for (int et = 0; et < DT; ++et) {
       i16x8_t a[DC];
 #pragma unroll
-      for (int c = 0; c < DC; ++c) a[c] = *reinterpret_cast<const i16x8_t*>(st_h + (size_t)(32 * et + r) * D + 16 * c + 8 * g);
+      for (int c = 0; c < DC; ++c) a[c] = *reinterpret_cast<const i16x8_t*>(st_h + (size_t)(32 * et + r_e) * D + 16 * c + 8 * g_e);
       f32x16_t acc;
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[i] = 0.f;
@@ -366,7 +376,7 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
       for (int c = 0; c < DC; ++c) acc = E::mfma32(a[c], qf[c], acc);
 #pragma unroll
       for (int i4 = 0; i4 < 4; ++i4) {
-        const int e0 = 32 * et + 8 * i4 + 4 * g;
+        const int e0 = 32 * et + 8 * i4 + 4 * g_e;
         const f32x4_t b4 = *reinterpret_cast<const f32x4_t*>(bias + e0);
         i32x2_t ws, wo;
         ws[0] = (int)E::pack2(oacc[et][4 * i4 + 0] * inv, oacc[et][4 * i4 + 1] * inv);
@@ -379,7 +389,7 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
           const float l1 = round16<Tag>(pin_f32(__builtin_fmaf(acc[4 * i4 + 2 * h + 1], inv_den, round16<Tag>(b4[2 * h + 1]))));
           wo[h] = (int)E::pack2(E::to_float((uint16_t)(x & 0xffff)) + l0, E::to_float((uint16_t)(x >> 16)) + l1);
         }
-        *reinterpret_cast<i32x2_t*>(&stage[r * SSTR + e0]) = wo;
+        *reinterpret_cast<i32x2_t*>(&stage_e[r_e * SSTR + e0]) = wo;
       }
     }
     wave_lds_fence();
