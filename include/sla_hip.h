@@ -50,6 +50,7 @@ extern "C" {
 #define SLA_WS_LINEAR_BWD 3
 #define SLA_WS_SAGE_QUANT 4
 #define SLA_WS_LINEAR_COMPLEMENT 5
+#define SLA_WS_SAGE_PREPARE 6
 
 int sla_version(void);
 const char* sla_last_error(void);
@@ -154,6 +155,17 @@ int sage_quant_qk(const void* q, const void* k, int dtype, int B, int H, int L, 
  * SageSLA/core.py:123-129. */
 int sage_quant_v(const void* v, int dtype, int B, int H, int L, int D, uint8_t* v_fp8, float* v_scale,
                  void* workspace, int64_t workspace_bytes, void* stream);
+
+/* SageSLA: everything the quantised attention kernel needs, in one call: the block map of
+ * sla_block_map_fwd (BLKQ 128, BLKK 64), the INT8 q / k of sage_quant_qk and the FP8 v of sage_quant_v,
+ * with outputs identical to those three calls on the same q, k, v (which must already be in the compute
+ * dtype).  The column mean of k is formed once and the quantisers emit the block means the scores are
+ * made of, so q is read once and k twice.
+ * Replaces get_block_map + k.mean + get_vanilla_qk_quant + the v quantisation, SageSLA/core.py:96-129. */
+int sage_prepare(const void* q, const void* k, const void* v, int dtype, int B, int H, int L, int D, int BLKQ,
+                 int BLKK, int topk, int8_t* sparse_map, void* lut, int lut_elem_bytes, int8_t* q_int8, float* q_scale,
+                 int8_t* k_int8, float* k_scale, uint8_t* v_fp8, float* v_scale, void* workspace,
+                 int64_t workspace_bytes, void* stream);
 
 /* SageSLA: quantised block-sparse attention, INT8 QK^T and FP8 PV on the matrix cores.
  * Replaces spas_sage_attn.utils.block_map_lut_triton + _qattn.qk_int8_sv_f8_*,

@@ -15,7 +15,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libsla_hip.so")
 
 SLA_F32, SLA_BF16, SLA_F16 = 0, 1, 2
 FMAP = {"elu": 0, "relu": 1, "softmax": 2}
-WS_BLOCK_MAP, WS_SPARSE_BWD, WS_LINEAR_FWD, WS_LINEAR_BWD, WS_SAGE_QUANT, WS_LINEAR_COMPLEMENT = range(6)
+WS_BLOCK_MAP, WS_SPARSE_BWD, WS_LINEAR_FWD, WS_LINEAR_BWD, WS_SAGE_QUANT, WS_LINEAR_COMPLEMENT, WS_SAGE_PREPARE = range(7)
 
 ERR_BAD_ARG, ERR_UNSUPPORTED, ERR_LAUNCH, ERR_WORKSPACE = -1, -2, -3, -4
 
@@ -41,6 +41,7 @@ SIGNATURES = {
                                        _P]),
     "sla_linear_bwd": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P, _I64, _P]),
     "sage_quant_qk": (_I, [_P, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _I64, _P]),
+    "sage_prepare": (_I, [_P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I64, _P]),
     "sage_quant_v": (_I, [_P, _I, _I, _I, _I, _I, _P, _P, _P, _I64, _P]),
     "sage_sparse_attn_fwd": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _P]),
 }

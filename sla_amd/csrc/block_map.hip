@@ -470,6 +470,22 @@ void launch_k_colmean(const void* k, int dtype, int BH, int L, int D, float* scr
     launch_k_colmean_t<IoF16>(k, BH, L, D, chunk_sums, group_sums, (uint16_t*)colmean, st);
 }
 
+// Scores and top-k selection from block means computed elsewhere (the quantisers of the SageSLA path
+// produce them on the way): pq (BH, M, D), pk (BH, N, D) in `dtype`; score: (BH, M, N) elements of `dtype`.
+void launch_map_from_pooled(int dtype, const void* pq, const void* pk, void* score, int BH, int M, int N, int D, int topk,
+                            int8_t* sparse_map, void* lut, int lut64, hipStream_t st) {
+  const dim3 grid(cdiv(N, 64), cdiv(M, 64), BH);
+  if (dtype == SLA_BF16) {
+    hipLaunchKernelGGL((score_kernel<IoBf16>), grid, dim3(256), 0, st, (const uint16_t*)pq, (const uint16_t*)pk,
+                       (uint16_t*)score, M, N, D);
+    launch_topk<IoBf16>((const uint16_t*)score, sparse_map, lut, lut64, N, topk, (size_t)BH * M, st);
+  } else {
+    hipLaunchKernelGGL((score_kernel<IoF16>), grid, dim3(256), 0, st, (const uint16_t*)pq, (const uint16_t*)pk,
+                       (uint16_t*)score, M, N, D);
+    launch_topk<IoF16>((const uint16_t*)score, sparse_map, lut, lut64, N, topk, (size_t)BH * M, st);
+  }
+}
+
 }  // namespace sla
 
 using namespace sla;

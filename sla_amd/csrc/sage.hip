@@ -16,17 +16,25 @@ namespace sla {
 
 int64_t k_colmean_scratch_floats(int BH, int L, int D);
 void launch_k_colmean(const void* k, int dtype, int BH, int L, int D, float* scratch, void* colmean, hipStream_t st);
+void launch_map_from_pooled(int dtype, const void* pq, const void* pk, void* score, int BH, int M, int N, int D, int topk,
+                            int8_t* sparse_map, void* lut, int lut64, hipStream_t st);
 
 // ---- INT8 block quantisation ----------------------------------------------------------------
 // One workgroup per (block, bh).  SUB_MEAN: subtract the per-head column mean first.
-template <typename Tag, int D, int BLK, bool SUB_MEAN>
+// POOL: also write the block mean the mask builder needs (of x, or of x - colmean rounded to 16 bit, as
+// get_block_map pools it: utils.py:55-58 of the reference), summed row by row in fp32 and divided once,
+// exactly as the pooling kernel of the mask builder does, so the block is read from memory once for both.
+template <typename Tag, int D, int BLK, bool SUB_MEAN, bool POOL>
 __global__ __launch_bounds__(256) void quant_int8_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ colmean,
-                                                         int8_t* __restrict__ xq, float* __restrict__ scale, int L, int nblk) {
+                                                         int8_t* __restrict__ xq, float* __restrict__ scale,
+                                                         uint16_t* __restrict__ pooled, int L, int nblk) {
   using E = Elem<Tag>;
   constexpr int CPR = D / 8;
   constexpr int RPP = 256 / CPR;
   constexpr int NP = BLK / RPP;
+  constexpr int TSTR = D + 8;
   __shared__ float sred[4];
+  __shared__ __attribute__((aligned(16))) uint16_t tile[POOL ? BLK * TSTR : 8];
   const int blk = blockIdx.x, bh = blockIdx.y;
   const int tid = threadIdx.x;
   const int lrow = tid / CPR, lcol = (tid % CPR) * 8;
@@ -51,6 +59,13 @@ __global__ __launch_bounds__(256) void quant_int8_kernel(const uint16_t* __restr
       val[p][e] = ok ? E::to_float((uint16_t)v[e]) - cm[e] : 0.f;
       amax = fmaxf(amax, fabsf(val[p][e]));
     }
+    if (POOL) {
+      if (SUB_MEAN) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = (short)E::from_float(val[p][e]);
+      }
+      *reinterpret_cast<i16x8_t*>(&tile[(lrow + p * RPP) * TSTR + lcol]) = v;
+    }
   }
 #pragma unroll
   for (int s = 1; s < 64; s <<= 1) amax = fmaxf(amax, __shfl_xor(amax, s));
@@ -59,6 +74,22 @@ __global__ __launch_bounds__(256) void quant_int8_kernel(const uint16_t* __restr
   amax = fmaxf(fmaxf(sred[0], sred[1]), fmaxf(sred[2], sred[3]));
   const float sc = fmaxf(amax, 1e-30f) / 127.0f;
   if (tid == 0) scale[(size_t)bh * nblk + blk] = sc;
+  if (POOL && tid < D) {   // one column per thread (the barrier above also covers the tile)
+    const int nrows = min(BLK, L - blk * BLK);
+    float acc = 0.f;
+    // rows are read sixteen at a time (all reads of a batch in flight together), then added in row order
+    constexpr int BATCH = 16;
+    int r = 0;
+    for (; r + BATCH <= nrows; r += BATCH) {
+      uint16_t t[BATCH];
+#pragma unroll
+      for (int i = 0; i < BATCH; ++i) t[i] = tile[(r + i) * TSTR + tid];
+#pragma unroll
+      for (int i = 0; i < BATCH; ++i) acc = acc + E::to_float(t[i]);
+    }
+    for (; r < nrows; ++r) acc = acc + E::to_float(tile[r * TSTR + tid]);
+    pooled[((size_t)bh * nblk + blk) * D + tid] = E::from_float(acc / (float)nrows);
+  }
 #pragma unroll
   for (int p = 0; p < NP; ++p) {
     const int grow = blk * BLK + lrow + p * RPP;
@@ -424,6 +455,22 @@ static SageWs sage_ws(int BH, int L, int D) {
 }
 int64_t sage_quant_workspace_bytes(int BH, int L, int D) { return (int64_t)sage_ws(BH, L, D).total; }
 
+// workspace of the one-call preparation: the quantisers' workspace, then block means and scores
+struct SagePrepWs {
+  size_t pq, pk, score, total;
+};
+static SagePrepWs sage_prep_ws(int BH, int L, int D) {
+  const int64_t M = cdiv(L, 128), N = cdiv(L, 64);
+  SagePrepWs w;
+  size_t off = sage_ws(BH, L, D).total;
+  w.pq = off;    off += align_up((int64_t)BH * M * D * 2, 256);
+  w.pk = off;    off += align_up((int64_t)BH * N * D * 2, 256);
+  w.score = off; off += align_up((int64_t)BH * M * N * 2, 256);
+  w.total = off;
+  return w;
+}
+int64_t sage_prepare_workspace_bytes(int BH, int L, int D) { return (int64_t)sage_prep_ws(BH, L, D).total; }
+
 static int validate_sage(int dtype, int B, int H, int L, int D, int BLKQ, int BLKK) {
   SLA_REQUIRE(B > 0 && H > 0 && L > 0, SLA_ERR_BAD_ARG, "non-positive size (B=%d H=%d L=%d)", B, H, L);
   SLA_REQUIRE((int64_t)B * H <= 65535, SLA_ERR_UNSUPPORTED, "B*H exceeds 65535");
@@ -440,11 +487,37 @@ static int quant_qk_impl(const void* q, const void* k, int dtype, int BH, int L,
   const SageWs w = sage_ws(BH, L, D);
   const int M = cdiv(L, 128), N = cdiv(L, 64);
   launch_k_colmean(k, dtype, BH, L, D, (float*)(ws + w.chunk_sums), ws + w.colmean, st);
-  hipLaunchKernelGGL((quant_int8_kernel<Tag, D, 128, false>), dim3(M, BH), dim3(256), 0, st, (const uint16_t*)q, nullptr, q8,
-                     qs, L, M);
-  hipLaunchKernelGGL((quant_int8_kernel<Tag, D, 64, true>), dim3(N, BH), dim3(256), 0, st, (const uint16_t*)k,
-                     (const uint16_t*)(ws + w.colmean), k8, ks, L, N);
+  hipLaunchKernelGGL((quant_int8_kernel<Tag, D, 128, false, false>), dim3(M, BH), dim3(256), 0, st, (const uint16_t*)q, nullptr,
+                     q8, qs, nullptr, L, M);
+  hipLaunchKernelGGL((quant_int8_kernel<Tag, D, 64, true, false>), dim3(N, BH), dim3(256), 0, st, (const uint16_t*)k,
+                     (const uint16_t*)(ws + w.colmean), k8, ks, nullptr, L, N);
   return check_launch("sage_quant_qk");
+}
+
+// Mask, INT8 q/k and FP8 v in one pass structure: the column mean of k is formed once (the mask builder
+// and the quantiser both subtract it) and the quantisers emit the block means the scores are made of, so
+// q is read once and k twice instead of q twice and k four times.
+template <typename Tag, int D>
+static int quant_v_impl(const void* v, int BH, int L, uint8_t* v8, float* vs, char* ws, hipStream_t st);
+
+template <typename Tag, int D>
+static int prepare_impl(const void* q, const void* k, const void* v, int dtype, int BH, int L, int topk, int8_t* sparse_map,
+                        void* lut, int lut64, int8_t* q8, float* qs, int8_t* k8, float* ks, uint8_t* v8, float* vs, char* ws,
+                        hipStream_t st) {
+  const SageWs w = sage_ws(BH, L, D);
+  const SagePrepWs p = sage_prep_ws(BH, L, D);
+  const int M = cdiv(L, 128), N = cdiv(L, 64);
+  uint16_t* pq = (uint16_t*)(ws + p.pq);
+  uint16_t* pk = (uint16_t*)(ws + p.pk);
+  launch_k_colmean(k, dtype, BH, L, D, (float*)(ws + w.chunk_sums), ws + w.colmean, st);
+  hipLaunchKernelGGL((quant_int8_kernel<Tag, D, 128, false, true>), dim3(M, BH), dim3(256), 0, st, (const uint16_t*)q, nullptr,
+                     q8, qs, pq, L, M);
+  hipLaunchKernelGGL((quant_int8_kernel<Tag, D, 64, true, true>), dim3(N, BH), dim3(256), 0, st, (const uint16_t*)k,
+                     (const uint16_t*)(ws + w.colmean), k8, ks, pk, L, N);
+  launch_map_from_pooled(dtype, pq, pk, ws + p.score, BH, M, N, D, topk, sparse_map, lut, lut64, st);
+  int rc = check_launch("sage_prepare");
+  if (rc) return rc;
+  return quant_v_impl<Tag, D>(v, BH, L, v8, vs, ws, st);
 }
 
 template <typename Tag, int D>
@@ -481,6 +554,41 @@ extern "C" int sage_quant_qk(const void* q, const void* k, int dtype, int B, int
   }
   if (D == 128) return quant_qk_impl<f16_tag, 128>(q, k, dtype, BH, L, q_int8, q_scale, k_int8, k_scale, ws, st);
   return quant_qk_impl<f16_tag, 64>(q, k, dtype, BH, L, q_int8, q_scale, k_int8, k_scale, ws, st);
+}
+
+extern "C" int sage_prepare(const void* q, const void* k, const void* v, int dtype, int B, int H, int L, int D, int BLKQ,
+                            int BLKK, int topk, int8_t* sparse_map, void* lut, int lut_elem_bytes, int8_t* q_int8,
+                            float* q_scale, int8_t* k_int8, float* k_scale, uint8_t* v_fp8, float* v_scale, void* workspace,
+                            int64_t workspace_bytes, void* stream) {
+  int rc = validate_sage(dtype, B, H, L, D, BLKQ, BLKK);
+  if (rc) return rc;
+  const int N = cdiv(L, 64);
+  SLA_REQUIRE(topk >= 0 && topk <= N, SLA_ERR_BAD_ARG, "topk=%d outside [0, %d]", topk, N);
+  SLA_REQUIRE(N <= 8192, SLA_ERR_UNSUPPORTED, "more than 8192 key blocks (%d)", N);
+  SLA_REQUIRE(lut_elem_bytes == 4 || lut_elem_bytes == 8, SLA_ERR_BAD_ARG, "lut_elem_bytes must be 4 or 8, got %d",
+              lut_elem_bytes);
+  SLA_REQUIRE(q && k && v && sparse_map && (lut || topk == 0) && q_int8 && q_scale && k_int8 && k_scale && v_fp8 && v_scale &&
+                  workspace,
+              SLA_ERR_BAD_ARG, "null pointer");
+  SLA_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)lut | (uintptr_t)q_int8 | (uintptr_t)k_int8 |
+               (uintptr_t)v_fp8 | (uintptr_t)workspace) % 16 == 0,
+              SLA_ERR_BAD_ARG, "pointers must be 16-byte aligned");
+  const int BH = B * H;
+  SLA_REQUIRE(workspace_bytes >= sage_prepare_workspace_bytes(BH, L, D), SLA_ERR_WORKSPACE, "workspace of %lld bytes, need %lld",
+              (long long)workspace_bytes, (long long)sage_prepare_workspace_bytes(BH, L, D));
+  hipStream_t st = (hipStream_t)stream;
+  char* ws = (char*)workspace;
+  const int lut64 = lut_elem_bytes == 8;
+#define SLA_PREP_CASE(TAG, DD) \
+  return prepare_impl<TAG, DD>(q, k, v, dtype, BH, L, topk, sparse_map, lut, lut64, q_int8, q_scale, k_int8, k_scale, v_fp8, \
+                               v_scale, ws, st)
+  if (dtype == SLA_BF16) {
+    if (D == 128) SLA_PREP_CASE(bf16_tag, 128);
+    SLA_PREP_CASE(bf16_tag, 64);
+  }
+  if (D == 128) SLA_PREP_CASE(f16_tag, 128);
+  SLA_PREP_CASE(f16_tag, 64);
+#undef SLA_PREP_CASE
 }
 
 extern "C" int sage_quant_v(const void* v, int dtype, int B, int H, int L, int D, uint8_t* v_fp8, float* v_scale,

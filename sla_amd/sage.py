@@ -10,7 +10,7 @@ import torch
 import torch.nn as nn
 
 from . import _lib
-from .block_map import get_block_map
+from .block_map import get_block_map, topk_count
 from .linear import linear_fwd
 from .module import FEATURE_MAPS
 
@@ -47,6 +47,38 @@ def quant_v(v):
                                   _lib.stream_ptr(v.device))
     _lib.check(rc)
     return v8, vs
+
+
+def sage_prepare(q, k, v, topk_ratio):
+    """Block map, INT8 q / k and FP8 v in one library call (q, k, v already in the compute dtype).
+
+    Returns ``(sparse_map, lut, T, q_int8, q_scale, k_int8, k_scale, v_fp8, v_scale)``, identical to
+    ``get_block_map`` + ``quant_qk`` + ``quant_v`` on the same tensors; the k column mean and the block
+    means are shared between the mask and the quantisers instead of being formed twice.
+    """
+    _lib.require_gpu(q, k, v)
+    assert q.is_contiguous() and k.is_contiguous() and v.is_contiguous()
+    assert q.shape == k.shape == v.shape and q.dtype == k.dtype == v.dtype
+    B, H, L, D = q.shape
+    dt = _lib.dtype_code(q.dtype)
+    M, N = (L + SAGE_BLKQ - 1) // SAGE_BLKQ, (L + SAGE_BLKK - 1) // SAGE_BLKK
+    T = topk_count(N, topk_ratio)
+    dev = q.device
+    ws = _lib.workspace(_lib.WS_SAGE_PREPARE, dt, B, H, L, D, SAGE_BLKQ, SAGE_BLKK, T, dev)
+    sparse_map = torch.empty((B, H, M, N), dtype=torch.int8, device=dev)
+    lut = torch.empty((B, H, M, T), dtype=torch.int64, device=dev)
+    q8 = torch.empty((B, H, L, D), dtype=torch.int8, device=dev)
+    k8 = torch.empty((B, H, L, D), dtype=torch.int8, device=dev)
+    qs = torch.empty((B, H, M), dtype=torch.float32, device=dev)
+    ks = torch.empty((B, H, N), dtype=torch.float32, device=dev)
+    v8 = torch.empty((B, H, L, D), dtype=torch.float8_e4m3fn, device=dev)
+    vs = torch.empty((B, H, D), dtype=torch.float32, device=dev)
+    rc = _lib.load().sage_prepare(q.data_ptr(), k.data_ptr(), v.data_ptr(), dt, B, H, L, D, SAGE_BLKQ, SAGE_BLKK, T,
+                                  sparse_map.data_ptr(), lut.data_ptr(), 8, q8.data_ptr(), qs.data_ptr(), k8.data_ptr(),
+                                  ks.data_ptr(), v8.data_ptr(), vs.data_ptr(), ws.data_ptr(), ws.numel(),
+                                  _lib.stream_ptr(dev))
+    _lib.check(rc)
+    return sparse_map, lut, T, q8, qs, k8, ks, v8, vs
 
 
 def sage_attn_fwd(q8, qs, k8, ks, v8, vs, lut, topk, out_dtype, qk_scale=None):
@@ -96,14 +128,19 @@ class SageSparseLinearAttention(nn.Module):
         q = q.contiguous()
         k = k.contiguous()
         v = v.contiguous()
-        sparse_map, lut, real_topk = get_block_map(q, k, topk_ratio=self.topk, BLKQ=SAGE_BLKQ, BLKK=SAGE_BLKK)
-        q = q.to(self.dtype)
-        k = k.to(self.dtype)
-        v = v.to(self.dtype)
         headdim = q.size(-1)
         assert headdim in [64, 128], "headdim should be in [64, 128]. For other headdim, you can use padding and specify the softmax scale."
-        q8, qs, k8, ks = quant_qk(q, k)
-        v8, vs = quant_v(v)
+        if q.dtype == k.dtype == v.dtype == self.dtype:
+            # the mask sees the same values as the quantisers: one pass structure for both
+            sparse_map, lut, real_topk, q8, qs, k8, ks, v8, vs = sage_prepare(q, k, v, self.topk)
+        else:
+            # the mask is built from the inputs as given, the quantisers work in the compute dtype (core.py:96-100)
+            sparse_map, lut, real_topk = get_block_map(q, k, topk_ratio=self.topk, BLKQ=SAGE_BLKQ, BLKK=SAGE_BLKK)
+            q = q.to(self.dtype)
+            k = k.to(self.dtype)
+            v = v.to(self.dtype)
+            q8, qs, k8, ks = quant_qk(q, k)
+            v8, vs = quant_v(v)
         o_s = sage_attn_fwd(q8, qs, k8, ks, v8, vs, lut, real_topk, self.dtype)
         o = linear_fwd(q, k, v, self.proj_l.weight, self.proj_l.bias, o_s, self.feature_map).to(dtype)
         if return_sparsity:

@@ -93,6 +93,14 @@ def test_other_entry_points_validate():
     assert "headdim" in _lib.last_error()
     assert lib.sage_sparse_attn_fwd(FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, 8, FAKE, 1, 1, 1, 128, 128, 128, 64, 9, 0.1,
                                     None) == _lib.ERR_BAD_ARG
+    # one-call SageSLA preparation: block sizes, topk range and workspace are checked before any launch
+    prep = lambda BLKQ, topk, ws: lib.sage_prepare(FAKE, FAKE, FAKE, 1, 1, 1, 256, 128, BLKQ, 64, topk, FAKE, FAKE, 8, FAKE,  # noqa: E731
+                                                   FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, ws, None)
+    assert prep(64, 1, 1 << 30) == _lib.ERR_UNSUPPORTED
+    assert prep(128, 5, 1 << 30) == _lib.ERR_BAD_ARG and "topk" in _lib.last_error()
+    assert prep(128, 2, 8) == _lib.ERR_WORKSPACE
+    need = lib.sla_workspace_bytes(_lib.WS_SAGE_PREPARE, 1, 1, 1, 256, 128, 128, 64, 2)
+    assert need > lib.sla_workspace_bytes(_lib.WS_SAGE_QUANT, 1, 1, 1, 256, 128, 128, 64, 2) > 0
 
 
 def test_host_api_mirrors_reference_names_and_errors():

@@ -8,7 +8,8 @@ from conftest import cos_sim
 from oracle import sla_oracle as O
 from sla_amd import SageSparseLinearAttention
 from sla_amd.inputs import CONFIGS, make_inputs, make_proj
-from sla_amd.sage import quant_qk, quant_v, sage_attn_fwd
+from sla_amd import get_block_map
+from sla_amd.sage import quant_qk, quant_v, sage_attn_fwd, sage_prepare
 
 pytestmark = pytest.mark.gpu
 
@@ -32,6 +33,24 @@ def test_quantisers_bit_exact(dev, L, D):
     assert torch.equal(qs.cpu(), qsr) and torch.equal(ks.cpu(), ksr) and torch.equal(vs.cpu(), vsr)
     assert torch.equal(q8.cpu(), q8r) and torch.equal(k8.cpu(), k8r)
     assert torch.equal(v8.cpu().view(torch.uint8), v8r.view(torch.uint8))
+
+
+@pytest.mark.parametrize("L,D,ratio,dtype", [(512, 128, 0.5, torch.bfloat16), (1000, 128, 0.3, torch.bfloat16),
+                                              (333, 64, 0.5, torch.float16), (2048, 128, 0.1, torch.float16),
+                                              (100, 64, 1.0, torch.bfloat16)])
+def test_one_call_preparation_equals_the_separate_calls(dev, L, D, ratio, dtype):
+    """Block map + both quantisers in one call: bit-identical to get_block_map, quant_qk, quant_v and to the oracle's map."""
+    q, k, v = (x.to(dtype) for x in _qkv(L, D, 7 * L + D))
+    m_ref, lut_ref, T_ref = O.get_block_map(q, k, ratio, 128, 64)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    m, lut, T, q8, qs, k8, ks, v8, vs = sage_prepare(qd, kd, vd, ratio)
+    assert T == T_ref and torch.equal(lut.cpu(), lut_ref) and torch.equal(m.cpu(), m_ref)
+    m2, lut2, T2 = get_block_map(qd, kd, ratio, 128, 64)
+    assert T2 == T and torch.equal(lut2, lut) and torch.equal(m2, m)
+    q8b, qsb, k8b, ksb = quant_qk(qd, kd)
+    v8b, vsb = quant_v(vd)
+    assert torch.equal(q8, q8b) and torch.equal(qs, qsb) and torch.equal(k8, k8b) and torch.equal(ks, ksb)
+    assert torch.equal(v8.view(torch.uint8), v8b.view(torch.uint8)) and torch.equal(vs, vsb)
 
 
 @pytest.mark.parametrize("L,D,ratio", [(512, 128, 0.5), (1000, 128, 0.3), (333, 64, 0.5), (2048, 128, 0.1)])
