@@ -51,6 +51,12 @@ extern "C" {
 #define SLA_WS_SAGE_QUANT 4
 #define SLA_WS_LINEAR_COMPLEMENT 5
 #define SLA_WS_SAGE_PREPARE 6
+#define SLA_WS_LINEAR_STATES 7 /* not an operation: the leading bytes of the SLA_WS_LINEAR_FWD workspace that hold the
+                                  finished per-head states (see sla_linear_bwd, SLA_BWD_STATES_READY) */
+
+/* flags of sla_linear_bwd */
+#define SLA_BWD_ACCUMULATE 1   /* dq, dk, dv already hold the sparse branch's gradients: add to them */
+#define SLA_BWD_STATES_READY 2 /* the workspace already starts with the states of the forward: do not rebuild them */
 
 int sla_version(void);
 const char* sla_last_error(void);
@@ -133,13 +139,17 @@ int sla_linear_complement_fwd(const void* q, const void* k, const void* v, const
 
 /* Linear branch backward.  d_out is the gradient of `out` above.  Writes dq, dk, dv in `dtype`
  * (gradients of the linear branch only; the residual's gradient is d_out itself) and the
- * fp32 gradients of weight (D,D) and bias (D).  With accumulate != 0, dq/dk/dv already hold
+ * fp32 gradients of weight (D,D) and bias (D).  flags: with SLA_BWD_ACCUMULATE, dq/dk/dv already hold
  * the gradients of the sparse branch and the linear ones, rounded to `dtype`, are added to them
  * as a tensor addition in `dtype` would (the sum is formed in fp32 and rounded once more).
+ * The backward needs the per-head states of the forward again; it rebuilds them from k and v unless
+ * SLA_BWD_STATES_READY says that the caller has copied the first sla_workspace_bytes(SLA_WS_LINEAR_STATES, ..)
+ * bytes of the forward's workspace (after sla_linear_state_fwd / sla_linear_fwd with the same k, v, weight)
+ * to the start of this workspace.
  * Replaces torch autograd through sparse_linear_attention/core.py:90-99. */
 int sla_linear_bwd(const void* q, const void* k, const void* v, const float* weight, const float* bias,
                    const void* d_out, void* dq, void* dk, void* dv, float* d_weight, float* d_bias,
-                   int dtype, int fmap, int B, int H, int L, int D, int accumulate, void* workspace,
+                   int dtype, int fmap, int B, int H, int L, int D, int flags, void* workspace,
                    int64_t workspace_bytes, void* stream);
 
 /* SageSLA: per-block INT8 quantisation of q (BLKQ rows) and of k - mean_L(k) (BLKK rows).

@@ -15,7 +15,8 @@ LIB_PATH = os.path.join(_HERE, "lib", "libsla_hip.so")
 
 SLA_F32, SLA_BF16, SLA_F16 = 0, 1, 2
 FMAP = {"elu": 0, "relu": 1, "softmax": 2}
-WS_BLOCK_MAP, WS_SPARSE_BWD, WS_LINEAR_FWD, WS_LINEAR_BWD, WS_SAGE_QUANT, WS_LINEAR_COMPLEMENT, WS_SAGE_PREPARE = range(7)
+WS_BLOCK_MAP, WS_SPARSE_BWD, WS_LINEAR_FWD, WS_LINEAR_BWD, WS_SAGE_QUANT, WS_LINEAR_COMPLEMENT, WS_SAGE_PREPARE, WS_LINEAR_STATES = range(8)
+BWD_ACCUMULATE, BWD_STATES_READY = 1, 2
 
 ERR_BAD_ARG, ERR_UNSUPPORTED, ERR_LAUNCH, ERR_WORKSPACE = -1, -2, -3, -4
 

@@ -27,6 +27,7 @@ int64_t linear_fwd_workspace_bytes(int BH, int L, int D);
 int64_t linear_bwd_workspace_bytes(int BH, int L, int D);
 int64_t sage_quant_workspace_bytes(int BH, int L, int D);
 int64_t sage_prepare_workspace_bytes(int BH, int L, int D);
+int64_t linear_states_bytes(int BH, int L, int D);
 int64_t linear_complement_workspace_bytes(int BH, int L, int D);
 
 }  // namespace sla
@@ -55,6 +56,8 @@ extern "C" int64_t sla_workspace_bytes(int op, int dtype, int B, int H, int L, i
       return linear_bwd_workspace_bytes(BH, L, D);
     case SLA_WS_SAGE_QUANT:
       return sage_quant_workspace_bytes(BH, L, D);
+    case SLA_WS_LINEAR_STATES:
+      return linear_states_bytes(BH, L, D);
     case SLA_WS_SAGE_PREPARE:
       return sage_prepare_workspace_bytes(BH, L, D);
     case SLA_WS_LINEAR_COMPLEMENT:

@@ -137,6 +137,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
 // ---- host side ----------------------------------------------------------------------------
 int64_t linear_fwd_workspace_bytes(int BH, int L, int D) { return (int64_t)lin_ws(BH, L, D).total; }
+int64_t linear_states_bytes(int BH, int L, int D) { return (int64_t)lin_ws(BH, L, D).states_end; }
 
 template <typename Tag, int D>
 static int linear_state_impl(const void* k, const void* v, const float* weight, int fmap, int BH, int L, char* ws,

@@ -204,7 +204,7 @@ __global__ __launch_bounds__(64 * NW) void linear_bwd_rows_kernel(
 // ---- states -------------------------------------------------------------------------------
 // grid (nsplit, BH).  dS^T partial [d2][d1] per (bh, split); dW^T partial [d][e] per (bh, split).
 template <typename Tag, int D>
-__global__ __launch_bounds__(256) void linear_bwd_states_kernel(
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void linear_bwd_states_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ dn, const uint16_t* __restrict__ gout,
     const uint16_t* __restrict__ y, const float* __restrict__ dden, float* __restrict__ ds_part, float* __restrict__ dw_part,
     float* __restrict__ dz_part, float* __restrict__ db_part, int L, int rows_per_split, int fmap) {
@@ -221,7 +221,10 @@ __global__ __launch_bounds__(256) void linear_bwd_states_kernel(
   __shared__ __attribute__((aligned(16))) uint16_t sDN[TR * STR];
   __shared__ __attribute__((aligned(16))) uint16_t sG[TR * STR];
   __shared__ __attribute__((aligned(16))) uint16_t sY[TR * STR];
-  __shared__ float sRed[2][RPP][D];
+  // the cross-thread sums of dz / db at the very end reuse the first two tiles (two workgroups per
+  // compute unit need the LDS footprint below 80 KB)
+  static_assert(2 * TR * STR * 2 >= 2 * RPP * D * 4, "reduction scratch does not fit the tiles it reuses");
+  float (*sRed)[RPP][D] = reinterpret_cast<float (*)[RPP][D]>(sA);
 
   const int split = blockIdx.x, bh = blockIdx.y, nsplit = gridDim.x;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -248,7 +251,8 @@ __global__ __launch_bounds__(256) void linear_bwd_states_kernel(
   const int tr_row = (lane & 15) >> 2;
   const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
 
-  // rows of the next tile are fetched into registers while the current tile is multiplied
+  // (no register prefetch of the next tile: the second workgroup on the compute unit covers the latency,
+  //  and the registers it would take are what lets that second workgroup fit)
   i16x8_t rq[NP], rdn[NP], rg[NP], ry[NP];
   float rdd[NP];
   auto fetch = [&](int r0) {
@@ -270,8 +274,8 @@ __global__ __launch_bounds__(256) void linear_bwd_states_kernel(
       }
     }
   };
-  if (row_begin < row_end) fetch(row_begin);
   for (int r0 = row_begin; r0 < row_end; r0 += TR) {
+    fetch(r0);
     __syncthreads();
 #pragma unroll
     for (int p = 0; p < NP; ++p) {
@@ -318,7 +322,6 @@ __global__ __launch_bounds__(256) void linear_bwd_states_kernel(
       *reinterpret_cast<i16x8_t*>(&sY[row * STR + lcol]) = xy;
     }
     __syncthreads();
-    if (r0 + TR < row_end) fetch(r0 + TR);     // after the barrier: its fence would wait for these loads
 #pragma unroll
     for (int c = 0; c < TR / 16; ++c) {
       const int l0 = 16 * c + 8 * g + tr_row;
@@ -568,12 +571,14 @@ __global__ __launch_bounds__(64 * NW) void linear_bwd_kv_kernel(const uint16_t* 
 // ---- host ---------------------------------------------------------------------------------
 struct LinBwdWs {
   LinWs fwd;
+  LinSplit st;   // slices of the states kernel (two workgroups per compute unit)
   size_t dn, y, dden, ds_part, dw_part, dz_part, db_part, ds, dst, dz, dw_head, db_head, total;
 };
 static LinBwdWs lin_bwd_ws(int BH, int L, int D) {
   LinBwdWs w;
   w.fwd = lin_ws(BH, L, D);
-  const int64_t np = (int64_t)BH * w.fwd.nsplit;
+  w.st = lin_split(BH, L, 512);
+  const int64_t np = (int64_t)BH * w.st.nsplit;
   size_t off = w.fwd.total;
   w.dn = off;      off += align_up((int64_t)BH * L * D * 2, 256);
   w.y = off;       off += align_up((int64_t)BH * L * D * 2, 256);
@@ -594,10 +599,11 @@ int64_t linear_bwd_workspace_bytes(int BH, int L, int D) { return (int64_t)lin_b
 
 template <typename Tag, int D>
 static int linear_bwd_impl(const void* q, const void* k, const void* v, const float* weight, const void* d_out, void* dq,
-                           void* dk, void* dv, float* d_weight, float* d_bias, int fmap, int BH, int L, int accumulate,
+                           void* dk, void* dv, float* d_weight, float* d_bias, int fmap, int BH, int L, int flags,
                            char* ws, hipStream_t st) {
   const LinBwdWs w = lin_bwd_ws(BH, L, D);
-  launch_state_build<Tag, D>(k, v, weight, fmap, BH, L, ws, w.fwd, st);
+  const int accumulate = flags & SLA_BWD_ACCUMULATE;
+  if (!(flags & SLA_BWD_STATES_READY)) launch_state_build<Tag, D>(k, v, weight, fmap, BH, L, ws, w.fwd, st);
   uint16_t* kvt = (uint16_t*)(ws + w.fwd.kvt);
   uint16_t* z = (uint16_t*)(ws + w.fwd.z);
   uint16_t* dn = (uint16_t*)(ws + w.dn);
@@ -609,13 +615,13 @@ static int linear_bwd_impl(const void* q, const void* k, const void* v, const fl
   hipLaunchKernelGGL((linear_bwd_rows_kernel<Tag, D, NW_ROWS>), dim3(cdiv(L, 32 * NW_ROWS * tiles_rows), BH), dim3(64 * NW_ROWS), 0, st, (const uint16_t*)q,
                      (const uint16_t*)d_out, kvt, (const uint16_t*)(ws + w.fwd.kvp), z, (const uint16_t*)(ws + w.fwd.wt), (uint16_t*)dq, dn, y,
                      dden, L, fmap, tiles_rows, accumulate);
-  hipLaunchKernelGGL((linear_bwd_states_kernel<Tag, D>), dim3(w.fwd.nsplit, BH), dim3(256), 0, st, (const uint16_t*)q, dn,
+  hipLaunchKernelGGL((linear_bwd_states_kernel<Tag, D>), dim3(w.st.nsplit, BH), dim3(256), 0, st, (const uint16_t*)q, dn,
                      (const uint16_t*)d_out, y, dden, (float*)(ws + w.ds_part), (float*)(ws + w.dw_part),
-                     (float*)(ws + w.dz_part), (float*)(ws + w.db_part), L, w.fwd.rows_per_split, fmap);
+                     (float*)(ws + w.dz_part), (float*)(ws + w.db_part), L, w.st.rows_per_split, fmap);
   hipLaunchKernelGGL((linear_bwd_reduce_kernel<Tag>), dim3(cdiv(D * D, 256), BH), dim3(256), 0, st,
                      (const float*)(ws + w.ds_part), (const float*)(ws + w.dw_part), (const float*)(ws + w.dz_part),
                      (const float*)(ws + w.db_part), (uint16_t*)(ws + w.ds), (uint16_t*)(ws + w.dst), (float*)(ws + w.dz),
-                     (float*)(ws + w.dw_head), (float*)(ws + w.db_head), w.fwd.nsplit, D);
+                     (float*)(ws + w.dw_head), (float*)(ws + w.db_head), w.st.nsplit, D);
   hipLaunchKernelGGL(linear_bwd_reduce_heads_kernel, dim3(cdiv(D * D, 256)), dim3(256), 0, st,
                      (const float*)(ws + w.dw_head), (const float*)(ws + w.db_head), d_weight, d_bias, BH, D);
   hipLaunchKernelGGL((linear_bwd_kv_kernel<Tag, D, NW_KV>), dim3(cdiv(L, 32 * NW_KV * tiles_kv), BH), dim3(64 * NW_KV), 0, st, (const uint16_t*)k, (const uint16_t*)v,
@@ -630,10 +636,11 @@ using namespace sla;
 
 extern "C" int sla_linear_bwd(const void* q, const void* k, const void* v, const float* weight, const float* bias,
                               const void* d_out, void* dq, void* dk, void* dv, float* d_weight, float* d_bias, int dtype,
-                              int fmap, int B, int H, int L, int D, int accumulate, void* workspace,
+                              int fmap, int B, int H, int L, int D, int flags, void* workspace,
                               int64_t workspace_bytes, void* stream) {
   int rc = validate_linear(dtype, fmap, B, H, L, D);
   if (rc) return rc;
+  SLA_REQUIRE((flags & ~(SLA_BWD_ACCUMULATE | SLA_BWD_STATES_READY)) == 0, SLA_ERR_BAD_ARG, "unknown flag bits in %d", flags);
   (void)bias;  // the bias does not enter any gradient
   SLA_REQUIRE(q && k && v && weight && d_out && dq && dk && dv && d_weight && d_bias && workspace, SLA_ERR_BAD_ARG,
               "null pointer");
@@ -647,7 +654,7 @@ extern "C" int sla_linear_bwd(const void* q, const void* k, const void* v, const
   hipStream_t st = (hipStream_t)stream;
   char* ws = (char*)workspace;
 #define SLA_LINB_CASE(TAG, DD) \
-  return linear_bwd_impl<TAG, DD>(q, k, v, weight, d_out, dq, dk, dv, d_weight, d_bias, fmap, BH, L, accumulate, ws, st)
+  return linear_bwd_impl<TAG, DD>(q, k, v, weight, d_out, dq, dk, dv, d_weight, d_bias, fmap, BH, L, flags, ws, st)
   if (dtype == SLA_BF16) {
     if (D == 128) SLA_LINB_CASE(bf16_tag, 128);
     SLA_LINB_CASE(bf16_tag, 64);

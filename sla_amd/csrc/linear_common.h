@@ -90,8 +90,10 @@ static __device__ __forceinline__ void phi_backward(int fmap, const float (&x)[D
 struct LinSplit {
   int nsplit, rows_per_split;
 };
-static inline LinSplit lin_split(int BH, int L) {
-  int nsplit = cdiv(768, BH);
+// Slices of the sequence for the kernels that reduce over L: as many (head, slice) workgroups as fit the chip at
+// once (`slots` = 256 compute units x workgroups per unit), never more, so there is no second, part-filled round.
+static inline LinSplit lin_split(int BH, int L, int slots = 768) {
+  int nsplit = slots / BH;
   const int max_split = cdiv(L, 64);
   if (nsplit > max_split) nsplit = max_split;
   if (nsplit < 1) nsplit = 1;

@@ -208,9 +208,11 @@ __global__ void linear_prep_weight_kernel(const float* __restrict__ weight, uint
 }
 
 // ---- workspace layout of the state build -----------------------------------------------------
+// The finished states (kvt .. wt) come first: `states_end` bytes that a caller may copy aside after the
+// forward and put back at the start of the backward's workspace instead of having them rebuilt.
 struct LinWs {
   int nsplit, rows_per_split;
-  size_t kv_part, z_part, kvt, kvp, kvwt, z, wt, total;
+  size_t kvt, kvp, kvwt, z, wt, states_end, kv_part, z_part, total;
 };
 
 static inline LinWs lin_ws(int BH, int L, int D) {
@@ -219,13 +221,14 @@ static inline LinWs lin_ws(int BH, int L, int D) {
   w.nsplit = sp.nsplit;
   w.rows_per_split = sp.rows_per_split;
   size_t off = 0;
-  w.kv_part = off; off += align_up((int64_t)BH * w.nsplit * D * D * 4, 256);
-  w.z_part = off;  off += align_up((int64_t)BH * w.nsplit * D * 4, 256);
   w.kvt = off;     off += align_up((int64_t)BH * D * D * 2, 256);
   w.kvp = off;     off += align_up((int64_t)BH * D * D * 2, 256);
   w.kvwt = off;    off += align_up((int64_t)BH * D * D * 2, 256);
   w.z = off;       off += align_up((int64_t)BH * D * 2, 256);
   w.wt = off;      off += align_up((int64_t)D * D * 2, 256);
+  w.states_end = off;
+  w.kv_part = off; off += align_up((int64_t)BH * w.nsplit * D * D * 4, 256);
+  w.z_part = off;  off += align_up((int64_t)BH * w.nsplit * D * 4, 256);
   w.total = off;
   return w;
 }

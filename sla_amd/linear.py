@@ -71,12 +71,27 @@ def linear_complement_fwd(q, k, v, lut, topk, weight, bias, residual, fmap: str,
     return out
 
 
-def linear_bwd(q, k, v, weight, bias, d_out, fmap: str, accumulate_into=None):
+def saved_states(state_ws, q):
+    """Copy of the finished per-head states at the head of a :func:`linear_state_fwd` workspace (about
+    ``3 B H D^2`` 16-bit values): what :func:`linear_bwd` needs of the forward, without the partial sums."""
+    B, H, L, D = q.shape
+    n = _lib.load().sla_workspace_bytes(_lib.WS_LINEAR_STATES, _lib.dtype_code(q.dtype), B, H, L, D, 64, 64, 0)
+    if n < 0:
+        _lib.check(int(n))
+    return state_ws[:int(n)].clone()
+
+
+def linear_bwd(q, k, v, weight, bias, d_out, fmap: str, accumulate_into=None, states=None):
     """Gradients of the linear branch.  ``accumulate_into=(dq, dk, dv)`` adds them to existing
-    gradient tensors (those of the sparse branch) instead of allocating new ones."""
+    gradient tensors (those of the sparse branch) instead of allocating new ones.  ``states``
+    (from :func:`saved_states`, same k, v, weight) spares the backward rebuilding the forward's states."""
     B, H, L, D = q.shape
     dt = _lib.dtype_code(q.dtype)
     ws = _lib.workspace(_lib.WS_LINEAR_BWD, dt, B, H, L, D, 64, 64, 0, q.device)
+    flags = 0 if accumulate_into is None else _lib.BWD_ACCUMULATE
+    if states is not None:
+        ws[:states.numel()].copy_(states)
+        flags |= _lib.BWD_STATES_READY
     if accumulate_into is None:
         dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     else:
@@ -85,8 +100,7 @@ def linear_bwd(q, k, v, weight, bias, d_out, fmap: str, accumulate_into=None):
     db = torch.empty((D,), dtype=torch.float32, device=q.device)
     rc = _lib.load().sla_linear_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), weight.data_ptr(), bias.data_ptr(),
                                     d_out.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), dw.data_ptr(),
-                                    db.data_ptr(), dt, _lib.FMAP[fmap], B, H, L, D,
-                                    0 if accumulate_into is None else 1, ws.data_ptr(), ws.numel(),
+                                    db.data_ptr(), dt, _lib.FMAP[fmap], B, H, L, D, flags, ws.data_ptr(), ws.numel(),
                                     _lib.stream_ptr(q.device))
     _lib.check(rc)
     return dq, dk, dv, dw, db

@@ -6,7 +6,7 @@ import torch
 import torch.nn as nn
 
 from .block_map import get_block_map
-from .linear import linear_bwd, linear_complement_fwd, linear_state_fwd
+from .linear import linear_bwd, linear_complement_fwd, linear_state_fwd, saved_states
 from .sparse_attn import sparse_attn_bwd, sparse_attn_fwd, sparse_attn_linear_fwd
 
 FEATURE_MAPS = ("elu", "relu", "softmax")
@@ -29,21 +29,23 @@ class _sla_core(torch.autograd.Function):
         bias = bias.contiguous()
         # one kernel: attention over the selected blocks, then the linear branch of the same rows from the
         # per-head state, projection and sum in its epilogue; o_s is only written when a backward will need it
-        out, o_s, lse = sparse_attn_linear_fwd(q, k, v, lut, topk, BLKQ, BLKK, qk_scale, state.join(), bias, fmap,
+        state_ws = state.join()
+        out, o_s, lse = sparse_attn_linear_fwd(q, k, v, lut, topk, BLKQ, BLKK, qk_scale, state_ws, bias, fmap,
                                                want_o_s=needs_grad)
         if not needs_grad:
             return out
-        ctx.save_for_backward(q, k, v, weight, bias, sparse_map, lut, lse, o_s)
+        # the finished states (a few D x D matrices per head) are kept for the backward, the partial sums are not
+        ctx.save_for_backward(q, k, v, weight, bias, sparse_map, lut, lse, o_s, saved_states(state_ws, q))
         ctx.cfg = (topk, BLKQ, BLKK, fmap, qk_scale)
         return out
 
     @staticmethod
     def backward(ctx, d_out):
-        q, k, v, weight, bias, sparse_map, lut, lse, o_s = ctx.saved_tensors
+        q, k, v, weight, bias, sparse_map, lut, lse, o_s, states = ctx.saved_tensors
         topk, BLKQ, BLKK, fmap, qk_scale = ctx.cfg
         d_out = d_out.contiguous()
         dq, dk, dv = sparse_attn_bwd(q, k, v, o_s, d_out, lse, sparse_map, lut, topk, BLKQ, BLKK, qk_scale)
-        _, _, _, dw, db = linear_bwd(q, k, v, weight, bias, d_out, fmap, accumulate_into=(dq, dk, dv))
+        _, _, _, dw, db = linear_bwd(q, k, v, weight, bias, d_out, fmap, accumulate_into=(dq, dk, dv), states=states)
         return dq, dk, dv, dw, db, None, None, None, None, None, None, None, None
 
 

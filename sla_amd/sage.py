@@ -11,8 +11,8 @@ import torch.nn as nn
 
 from . import _lib
 from .block_map import get_block_map, topk_count
-from .linear import linear_fwd
-from .module import FEATURE_MAPS
+from .linear import linear_out_fwd
+from .module import FEATURE_MAPS, _StateBuild
 
 SAGE_BLKQ, SAGE_BLKK = 128, 64
 
@@ -141,8 +141,11 @@ class SageSparseLinearAttention(nn.Module):
             v = v.to(self.dtype)
             q8, qs, k8, ks = quant_qk(q, k)
             v8, vs = quant_v(v)
+        # the k/v half of the linear branch is memory-bound and runs on a side stream beside the attention
+        # kernel, which is bound by the vector ALU and the matrix cores
+        state = _StateBuild(k, v, self.proj_l.weight, self.feature_map)
         o_s = sage_attn_fwd(q8, qs, k8, ks, v8, vs, lut, real_topk, self.dtype)
-        o = linear_fwd(q, k, v, self.proj_l.weight, self.proj_l.bias, o_s, self.feature_map).to(dtype)
+        o = linear_out_fwd(q, self.proj_l.bias, o_s, state.join(), self.feature_map).to(dtype)
         if return_sparsity:
             return o, real_topk / sparse_map.shape[-1]
         return o

@@ -85,6 +85,11 @@ def test_other_entry_points_validate():
     assert lib.sla_linear_out_fwd(FAKE, FAKE, None, FAKE, 1, 0, 1, 1, 64, 128, None, 1 << 30, None) == _lib.ERR_BAD_ARG
     assert lib.sla_linear_bwd(FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, 1, 0, 1, 1, 64, 128, 0, FAKE,
                               8, None) == _lib.ERR_WORKSPACE
+    assert lib.sla_linear_bwd(FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, 1, 0, 1, 1, 64, 128, 4, FAKE,
+                              1 << 30, None) == _lib.ERR_BAD_ARG and "flag" in _lib.last_error()
+    states = lib.sla_workspace_bytes(_lib.WS_LINEAR_STATES, 1, 1, 12, 32760, 128, 64, 64, 0)
+    assert 0 < states <= 12 * 3 * 128 * 128 * 2 + 12 * 128 * 2 + 128 * 128 * 2 + 5 * 256
+    assert states < lib.sla_workspace_bytes(_lib.WS_LINEAR_FWD, 1, 1, 12, 32760, 128, 64, 64, 0)
     assert lib.sla_sparse_attn_bwd(FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, 8, FAKE, FAKE, FAKE, 1, 1, 1, 128, 128, 64,
                                    64, 1, 0.1, FAKE, 8, None) == _lib.ERR_WORKSPACE
     assert lib.sage_quant_qk(FAKE, FAKE, 1, 1, 1, 128, 128, 64, 64, FAKE, FAKE, FAKE, FAKE, FAKE, 1 << 30, None) == _lib.ERR_UNSUPPORTED

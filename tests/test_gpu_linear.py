@@ -5,7 +5,7 @@ import torch
 from conftest import cos_sim, max_abs
 from oracle import sla_oracle as O
 from sla_amd.inputs import CONFIGS, make_inputs, make_proj
-from sla_amd.linear import linear_fwd, linear_out_fwd, linear_state_fwd
+from sla_amd.linear import linear_bwd, linear_fwd, linear_out_fwd, linear_state_fwd
 
 pytestmark = pytest.mark.gpu
 
@@ -97,3 +97,25 @@ def test_split_entry_points_equal_the_fused_one(dev):
     ws.record_stream(torch.cuda.current_stream(dev))
     out = linear_out_fwd(q, b, res, ws, "elu")
     assert torch.equal(out, ref)
+
+
+@pytest.mark.parametrize("fmap,D", [("elu", 128), ("softmax", 64)])
+def test_backward_with_the_forward_states_handed_over(dev, fmap, D):
+    """States copied from the forward's workspace instead of rebuilt in the backward: same gradients, bit for bit."""
+    from sla_amd.linear import saved_states
+
+    g = torch.Generator().manual_seed(11)
+    q, k, v, do = (torch.randn(2, 2, 450, D, generator=g).to(torch.bfloat16).to(dev) for _ in range(4))
+    w, b = (t.to(dev) for t in make_proj(D))
+    ref = linear_bwd(q, k, v, w, b, do, fmap)
+    states = saved_states(linear_state_fwd(k, v, w, fmap), q)
+    assert states.numel() < 4 * 4 * D * D * 2 + 4096          # a few D x D matrices per head, no partial sums
+    out = linear_bwd(q, k, v, w, b, do, fmap, states=states)
+    for a, r in zip(out, ref):
+        assert torch.equal(a, r)
+    # accumulating variant
+    base = [torch.randn_like(q) for _ in range(3)]
+    acc_ref = linear_bwd(q, k, v, w, b, do, fmap, accumulate_into=tuple(t.clone() for t in base))
+    acc = linear_bwd(q, k, v, w, b, do, fmap, accumulate_into=tuple(t.clone() for t in base), states=states)
+    for a, r in zip(acc, acc_ref):
+        assert torch.equal(a, r)
