@@ -56,8 +56,6 @@ similarity >= 0.995 against the fp32 SLA math.
 """
 from __future__ import annotations
 
-import math
-
 import torch
 import torch.nn.functional as F
 

@@ -1,6 +1,5 @@
 """CPU-only checks of the C ABI: the library loads, exports every symbol the header declares,
 and validates arguments before touching the device (so error paths need no GPU)."""
-import ctypes
 import os
 import re
 

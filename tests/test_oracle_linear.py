@@ -1,7 +1,6 @@
 """Pins the linear branch / projection / sum of the CPU oracle."""
 import pytest
 import torch
-import torch.nn.functional as F
 
 from oracle import sla_oracle as O
 from sla_amd.inputs import make_proj
