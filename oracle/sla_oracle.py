@@ -39,7 +39,9 @@ Two things are fixed here that the reference leaves open, because without them
       ``KMEAN_GROUP`` consecutive chunks; the group sums added one by one in
       ascending order; one IEEE division by L;
     - pooled score: ``acc = acc + (a_d * b_d)`` for d ascending, product and sum
-      rounded separately (no fused multiply-add).
+      rounded separately.  (For bf16 / f16 inputs the product is exact in fp32
+      above the subnormal range, so a fused multiply-add yields the same bits;
+      the kernel uses one there and the separate form for fp32 inputs.)
   All results are then rounded to the input dtype exactly where the reference
   materialises a tensor of that dtype.
 
