@@ -91,3 +91,41 @@ def test_cfg3_two_heads_forward(dev):
     o_ref, _ = O.sparse_attn_fwd_gather(d["q"], d["k"], d["v"], lut, 64, 64)
     o = _run(d["q"], d["k"], d["v"], lut, m, T, 64, dev)
     assert max_abs(o, o_ref) <= TOL_ABS and cos_sim(o, o_ref) >= TOL_COS
+
+
+@pytest.mark.parametrize("order", ["ascending", "descending", "random"])
+def test_wide_score_range_moves_the_reference_maximum(dev, order):
+    """Scores that span hundreds of log2 units, arranged so that the running maximum rises with every key
+    block (ascending), never rises after the first (descending), or jumps at random: the lazily updated
+    reference maximum of the kernels has to rescale on the first pattern and must not lose the small terms
+    on the second.  The sage kernel runs the same inputs against the fp32 math."""
+    from sla_amd.sage import quant_qk, quant_v, sage_attn_fwd
+
+    g = torch.Generator().manual_seed(3)
+    L, D, H = 640, 128, 2
+    N = L // 64
+    q = torch.randn(1, H, L, D, generator=g)
+    k = torch.randn(1, H, L, D, generator=g)
+    v = torch.randn(1, H, L, D, generator=g)
+    # block j of k gets a component along the mean query direction whose size depends on j
+    qdir = q.mean(dim=-2, keepdim=True) + 0.5
+    qdir = qdir / qdir.norm(dim=-1, keepdim=True)
+    q = q + 6.0 * qdir
+    steps = {"ascending": torch.arange(N), "descending": torch.arange(N).flip(0),
+             "random": torch.randperm(N, generator=g)}[order].float()
+    k = k + (4.0 * steps.repeat_interleave(64).view(1, 1, L, 1)) * qdir
+    q, k, v = (t.to(torch.bfloat16) for t in (q, k, v))
+    lut = torch.arange(N).expand(1, H, N, N).contiguous()
+    m = torch.ones(1, H, N, N, dtype=torch.int8)
+    ref, lse_ref = O.sparse_attn_fwd_dense(q, k, v, m, 64, 64)
+    assert float(lse_ref.max() - lse_ref.min()) > 20          # the case is what it claims to be
+    o = _run(q, k, v, lut, m, N, 64, dev)
+    assert max_abs(o, ref) <= TOL_ABS and cos_sim(o, ref) >= TOL_COS
+    # SageSLA kernel (BLKQ 128): same selection
+    M2 = L // 128
+    lut2 = torch.arange(N).expand(1, H, M2, N).contiguous()
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    q8, qs, k8, ks = quant_qk(qd, kd)
+    v8, vs = quant_v(vd)
+    o8 = sage_attn_fwd(q8, qs, k8, ks, v8, vs, lut2.to(dev), N, torch.bfloat16).cpu()
+    assert cos_sim(o8, ref) >= 0.995
