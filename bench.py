@@ -83,8 +83,8 @@ def cpu_baseline(cfg, heads, torch):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="cfg3")
     ap.add_argument("--cpu-heads", type=int, default=12, help="heads of the workload timed on the CPU oracle (0 = skip)")
     ap.add_argument("--no-extras", action="store_true", help="skip the per-kernel, backward and SageSLA timings")
