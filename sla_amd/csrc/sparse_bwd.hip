@@ -46,55 +46,67 @@ __global__ __launch_bounds__(256) void bwd_delta_kernel(const uint16_t* __restri
 }
 
 // ---- per-key-block lists ------------------------------------------------------------------
-// One wavefront per strip of 64 key blocks.  The map is read 64 rows at a time with coalesced
-// 16-byte loads (the next tile's loads are in flight while this one is scanned) and transposed
-// through LDS; lane c then walks the 64 bytes of its column in order, so list[bh][n][0..count)
-// holds the selecting query blocks in ascending order.  Capacity Mblk per list (only `count`
-// entries are ever touched).
-__global__ __launch_bounds__(64) void bwd_col_lists_kernel(const int8_t* __restrict__ sparse_map, int* __restrict__ list,
-                                                           int* __restrict__ count, int Mblk, int Nblk, int vec_ok) {
-  __shared__ __attribute__((aligned(16))) int8_t tile[64][80];
+// One workgroup of COL_NW wavefronts per strip of 64 key blocks.  Every wavefront takes its own chunk of
+// 64 map rows (query blocks): it reads them with coalesced 16-byte loads and transposes them through its
+// private LDS tile; lane c counts the ones of column c in that chunk.  After a barrier every wave knows
+// how many entries the chunks before its own contribute to each column and writes its matches at that
+// offset, walking the chunk in row order, so list[bh][n][0..count) holds the selecting query blocks in
+// ascending order.  Capacity Mblk per list (only `count` entries are ever touched).
+constexpr int COL_NW = 8;
+__global__ __launch_bounds__(64 * COL_NW) void bwd_col_lists_kernel(const int8_t* __restrict__ sparse_map,
+                                                                    int* __restrict__ list, int* __restrict__ count,
+                                                                    int Mblk, int Nblk, int vec_ok) {
+  __shared__ __attribute__((aligned(16))) int8_t tile[COL_NW][64][80];
+  __shared__ int cnt[COL_NW][64];
   const int bh = blockIdx.y;
   const int n0 = blockIdx.x * 64;
-  const int lane = threadIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int n = n0 + lane;
   const int8_t* base = sparse_map + (size_t)bh * Mblk * Nblk;
   int* out = list + ((size_t)bh * Nblk + (n < Nblk ? n : 0)) * Mblk;
   // lane -> (row lr + 16j, 16-byte chunk lc) of the tile
   const int lr = lane >> 2, lc = (lane & 3) * 16;
-  i32x4_t pre[4];
-  auto fetch = [&](int m0) {
+  int done = 0;              // entries of column `lane` written by earlier rounds
+  for (int r0 = 0; r0 < Mblk; r0 += 64 * COL_NW) {
+    const int m0 = r0 + 64 * wave;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int m = m0 + lr + 16 * j;
-      pre[j] = i32x4_t{0, 0, 0, 0};
+      i32x4_t x = {0, 0, 0, 0};
       if (m < Mblk) {
         if (vec_ok && n0 + lc + 16 <= Nblk) {
-          pre[j] = *reinterpret_cast<const i32x4_t*>(base + (size_t)m * Nblk + n0 + lc);
+          x = *reinterpret_cast<const i32x4_t*>(base + (size_t)m * Nblk + n0 + lc);
         } else {
-          int8_t* b = reinterpret_cast<int8_t*>(&pre[j]);
+          int8_t* b = reinterpret_cast<int8_t*>(&x);
           for (int e = 0; e < 16; ++e)
             if (n0 + lc + e < Nblk) b[e] = base[(size_t)m * Nblk + n0 + lc + e];
         }
       }
+      *reinterpret_cast<i32x4_t*>(&tile[wave][lr + 16 * j][lc]) = x;
     }
-  };
-  int c = 0;
-  fetch(0);
-  for (int m0 = 0; m0 < Mblk; m0 += 64) {
-    __syncthreads();
-#pragma unroll
-    for (int j = 0; j < 4; ++j) *reinterpret_cast<i32x4_t*>(&tile[lr + 16 * j][lc]) = pre[j];
-    __syncthreads();
-    if (m0 + 64 < Mblk) fetch(m0 + 64);
-    if (n < Nblk) {
+    wave_lds_fence();
+    int mine = 0;
 #pragma unroll 16
-      for (int r = 0; r < 64; ++r) {
-        if (tile[r][lane] == 1) out[c++] = m0 + r;
-      }
+    for (int r = 0; r < 64; ++r) mine += tile[wave][r][lane] == 1;
+    cnt[wave][lane] = mine;
+    __syncthreads();
+    int before = 0, all = 0;
+#pragma unroll
+    for (int w = 0; w < COL_NW; ++w) {
+      const int cw = cnt[w][lane];
+      before += w < wave ? cw : 0;
+      all += cw;
     }
+    if (n < Nblk) {
+      int c = done + before;
+#pragma unroll 16
+      for (int r = 0; r < 64; ++r)
+        if (tile[wave][r][lane] == 1) out[c++] = m0 + r;
+    }
+    done += all;
+    __syncthreads();         // cnt and the tiles are rewritten by the next round
   }
-  if (n < Nblk) count[(size_t)bh * Nblk + n] = c;
+  if (wave == 0 && n < Nblk) count[(size_t)bh * Nblk + n] = done;
 }
 
 // ---- dQ ---------------------------------------------------------------------------------
@@ -526,7 +538,7 @@ static int bwd_impl(const void* q, const void* k, const void* v, const void* o, 
                      (const uint16_t*)o, (const uint16_t*)d_o, delta, rows);
   // 16-byte loads of map rows need 16-byte aligned rows
   const int vec_ok = (Nblk % 16 == 0) && ((uintptr_t)sparse_map % 16 == 0);
-  hipLaunchKernelGGL(bwd_col_lists_kernel, dim3(cdiv(Nblk, 64), BH), dim3(64), 0, st, sparse_map, list, count, Mblk, Nblk,
+  hipLaunchKernelGGL(bwd_col_lists_kernel, dim3(cdiv(Nblk, 64), BH), dim3(64 * COL_NW), 0, st, sparse_map, list, count, Mblk, Nblk,
                      vec_ok);
   const int total_q = BH * Mblk;
   hipLaunchKernelGGL((bwd_dq_kernel<Tag, D, BLKQ>), dim3(xcd_grid(total_q)), dim3(BLKQ * 2), 0, st, (const uint16_t*)q,

@@ -79,3 +79,19 @@ def test_cfg3_shape_invariants_and_two_heads(dev):
     # (signed sums of bf16-rounded terms: the tolerance scales with the sum of magnitudes)
     ta, tb = d["q"].double() * dq.double(), d["k"].double() * dk.double()
     assert abs(ta.sum() - tb.sum()) <= 1e-3 * float(ta.abs().sum() + tb.abs().sum())
+
+
+def test_more_query_blocks_than_one_round_of_the_list_builder(dev):
+    """L = 40000 at BLKQ 64 is 625 query blocks: the per-key-block lists are built in two rounds of row chunks and
+    the last round is ragged.  dK / dV (the consumers of the lists) against the gather oracle."""
+    g = torch.Generator().manual_seed(41)
+    L, D = 40000, 64
+    q, k, v, do = (torch.randn(1, 1, L, D, generator=g).to(torch.bfloat16) for _ in range(4))
+    m, lut, T = O.get_block_map(q, k, 0.01, 64, 64)
+    assert m.shape[-2] == 625 and T == 6
+    o_ref, lse_ref = O.sparse_attn_fwd_gather(q, k, v, lut, 64, 64)
+    refs = O.sparse_attn_bwd_gather(q, k, v, o_ref, do, lse_ref, lut, 64, 64)
+    o, dq, dk, dv = _grads(q, k, v, do, m, lut, T, 64, dev)
+    for name, a, b in zip(("dq", "dk", "dv"), (dq, dk, dv), refs):
+        assert max_abs(a, b) <= TOL_ABS, name
+        assert cos_sim(a, b) >= TOL_COS, name
