@@ -127,6 +127,27 @@ int sla_linear_state_fwd(const void* k, const void* v, const float* weight, int 
 int sla_linear_out_fwd(const void* q, const float* bias, const void* residual, void* out, int dtype, int fmap, int B,
                        int H, int L, int D, void* workspace, int64_t workspace_bytes, void* stream);
 
+/* The module's inference forward for callers whose activations are not laid out as contiguous (B, H, L, D):
+ * strided variants of the three calls that touch q, k, v and out.  `*_strides` = {batch, head, row} strides in
+ * elements of a tensor indexed (b, h, l, d) whose last dimension is contiguous: {H*L*D, L*D, D} for the
+ * contiguous layout, {L*H*D, D, H*D} for a (B, L, H, D) activation, {L*3*H*D, D, 3*H*D} for the q / k / v
+ * slices of a packed (B, L, 3, H, D) projection.  All strides must be multiples of 8 elements (4 for fp32
+ * inputs of the mask builder) and one head must span less than 4 GiB.  Everything else as in the calls without
+ * the suffix (workspaces, lut, lse and o_s keep their contiguous shapes).
+ * They replace the layout copies either side of the operator in a transformer block
+ * (evaluate/bench_kernel.py:68-71 of the reference: transpose(1, 2).contiguous() of q, k, v and of the output). */
+int sla_block_map_fwd_strided(const void* q, const void* k, const int64_t* qk_strides, int dtype, int B, int H, int L,
+                              int D, int BLKQ, int BLKK, int topk, void* workspace, int64_t workspace_bytes,
+                              int8_t* sparse_map, void* lut, int lut_elem_bytes, void* stream);
+int sla_linear_state_fwd_strided(const void* k, const void* v, const int64_t* kv_strides, const float* weight, int dtype,
+                                 int fmap, int B, int H, int L, int D, void* workspace, int64_t workspace_bytes,
+                                 void* stream);
+int sla_sparse_attn_linear_fwd_strided(const void* q, const void* k, const void* v, const int64_t* qkv_strides,
+                                       const void* lut, int lut_elem_bytes, const void* linear_workspace,
+                                       int64_t linear_workspace_bytes, const float* bias, void* o_s, void* out,
+                                       const int64_t* out_strides, float* lse, int dtype, int fmap, int B, int H, int L,
+                                       int D, int BLKQ, int BLKK, int topk, float qk_scale, void* stream);
+
 /* Linear branch in "complement" mode (opt-in; forward only): query block i attends linearly only to the key
  * blocks (of 64 rows) that its look-up row did NOT select; projection, bias and residual as in
  * sla_linear_fwd.  out = residual + proj(o_l).  lut as produced by sla_block_map_fwd; BLKK must be 64.

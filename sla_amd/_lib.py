@@ -30,6 +30,10 @@ SIGNATURES = {
     "sla_workspace_bytes": (_I64, [_I] * 9),
     "sla_mean_pool": (_I, [_P, _P, _I, _I, _I, _I, _I, _P]),
     "sla_block_map_fwd": (_I, [_P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _I64, _P, _P, _I, _P]),
+    "sla_block_map_fwd_strided": (_I, [_P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _I64, _P, _P, _I, _P]),
+    "sla_linear_state_fwd_strided": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I64, _P]),
+    "sla_sparse_attn_linear_fwd_strided": (_I, [_P, _P, _P, _P, _P, _I, _P, _I64, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I,
+                                                _I, _I, _I, _I, _F, _P]),
     "sla_sparse_attn_fwd": (_I, [_P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _P]),
     "sla_sparse_attn_linear_fwd": (_I, [_P, _P, _P, _P, _I, _P, _I64, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I,
                                         _F, _P]),
@@ -105,6 +109,49 @@ def require_gpu(*tensors) -> None:
     for t in tensors:
         if not t.is_cuda:
             raise RuntimeError("sla_amd runs on the GPU only: got a tensor on " + str(t.device))
+
+
+def _significant_strides(t):
+    """Strides of the batch, head and row dimensions; None where the dimension has one entry (its stride is never used)."""
+    return tuple(st if n > 1 else None for n, st in zip(t.shape[:3], t.stride()[:3]))
+
+
+def row_strided(*tensors) -> bool:
+    """True when the (B, H, L, D) tensors can be handed to the ``*_strided`` entry points as they are: same
+    strides, contiguous last dimension, every row 16-byte aligned, rows not overlapping."""
+    t0 = tensors[0]
+    if t0.dim() != 4 or t0.stride(-1) != 1:
+        return False
+    vec = 16 // t0.element_size()
+    for t in tensors:
+        if (t.shape != t0.shape or t.dtype != t0.dtype or t.stride(-1) != 1 or t.data_ptr() % 16
+                or _significant_strides(t) != _significant_strides(t0)):
+            return False
+    sb, sh, sl = _significant_strides(t0)
+    if any(st is not None and (st <= 0 or st % vec) for st in (sb, sh, sl)):
+        return False
+    return sl is None or sl >= t0.shape[-1]
+
+
+def strides_arg(t):
+    """{batch, head, row} strides of a (B, H, L, D) tensor as the int64[3] the ``*_strided`` entry points take
+    (dimensions with one entry get a harmless aligned value)."""
+    B, H, L, D = t.shape
+    sb, sh, sl = _significant_strides(t)
+    sl = D if sl is None else sl
+    sh = L * sl if sh is None else sh
+    sb = H * L * sl if sb is None else sb
+    return (ctypes.c_int64 * 3)(sb, sh, sl)
+
+
+def empty_like_rows(t):
+    """Uninitialised tensor of t's shape and dtype whose dimensions are ordered in memory like t's (so a
+    (B, L, H, D) activation viewed as (B, H, L, D) gets an output it can view back for free), densely packed."""
+    order = sorted(range(t.dim() - 1), key=lambda i: (-t.stride(i), i)) + [t.dim() - 1]
+    shape = [t.shape[i] for i in order]
+    out = torch.empty(shape, dtype=t.dtype, device=t.device)
+    inv = [order.index(i) for i in range(t.dim())]
+    return out.permute(inv)
 
 
 def workspace(op: int, dtype: int, B, H, L, D, BLKQ, BLKK, topk, device) -> torch.Tensor:

@@ -36,8 +36,9 @@ def get_block_map(q: torch.Tensor, k: torch.Tensor, topk_ratio: float, BLKQ: int
     ascending order (the reference leaves the order unspecified); equal scores
     are resolved towards the lowest block index.
     """
-    assert q.is_contiguous() and k.is_contiguous()
     assert q.shape == k.shape and q.dtype == k.dtype
+    strided = not (q.is_contiguous() and k.is_contiguous())
+    assert not strided or _lib.row_strided(q, k), "q and k must be contiguous or share row-contiguous strides"
     _lib.require_gpu(q, k)
     B, H, L, D = q.shape
     M = (L + BLKQ - 1) // BLKQ
@@ -47,8 +48,13 @@ def get_block_map(q: torch.Tensor, k: torch.Tensor, topk_ratio: float, BLKQ: int
     ws = _lib.workspace(_lib.WS_BLOCK_MAP, dt, B, H, L, D, BLKQ, BLKK, T, q.device)
     sparse_map = torch.empty((B, H, M, N), dtype=torch.int8, device=q.device)
     lut = torch.empty((B, H, M, T), dtype=torch.int64, device=q.device)
-    rc = _lib.load().sla_block_map_fwd(q.data_ptr(), k.data_ptr(), dt, B, H, L, D, BLKQ, BLKK, T, ws.data_ptr(),
-                                       ws.numel(), sparse_map.data_ptr(), lut.data_ptr(), 8,
-                                       _lib.stream_ptr(q.device))
+    if strided:
+        rc = _lib.load().sla_block_map_fwd_strided(q.data_ptr(), k.data_ptr(), _lib.strides_arg(q), dt, B, H, L, D, BLKQ,
+                                                   BLKK, T, ws.data_ptr(), ws.numel(), sparse_map.data_ptr(),
+                                                   lut.data_ptr(), 8, _lib.stream_ptr(q.device))
+    else:
+        rc = _lib.load().sla_block_map_fwd(q.data_ptr(), k.data_ptr(), dt, B, H, L, D, BLKQ, BLKK, T, ws.data_ptr(),
+                                           ws.numel(), sparse_map.data_ptr(), lut.data_ptr(), 8,
+                                           _lib.stream_ptr(q.device))
     _lib.check(rc)
     return sparse_map, lut, T

@@ -53,7 +53,7 @@ struct alignas(16) Vec16 {
 // MODE 2: block mean of round(x - colmean)     -> out     (BH, nblk, D)
 // One thread owns VEC adjacent columns of one block and walks its rows in order.
 template <typename IO, int MODE>
-static __device__ __forceinline__ void pool_body(const typename IO::raw* __restrict__ x,
+static __device__ __forceinline__ void pool_body(const typename IO::raw* __restrict__ x, const RowLayout lay,
                                                  const typename IO::raw* __restrict__ colmean, void* __restrict__ out, int L,
                                                  int D, int BLK, int nblk, int bx, int bh) {
   constexpr int VEC = IO::VEC;
@@ -74,14 +74,15 @@ static __device__ __forceinline__ void pool_body(const typename IO::raw* __restr
 #pragma unroll
     for (int e = 0; e < VEC; ++e) cm[e] = IO::ld(m.e[e]);
   }
-  const typename IO::raw* p = x + ((size_t)bh * L + row0) * D + c;
+  const size_t pitch = (size_t)lay.sl;
+  const typename IO::raw* p = x + lay.head(bh) + (size_t)row0 * pitch + c;
   // rows are fetched sixteen at a time (all loads of a batch in flight together), then added in row order
   constexpr int BATCH = 16;
   int r = 0;
   for (; r + BATCH <= nrows; r += BATCH) {
     Vec16<IO> v[BATCH];
 #pragma unroll
-    for (int i = 0; i < BATCH; ++i) v[i] = *reinterpret_cast<const Vec16<IO>*>(p + (size_t)(r + i) * D);
+    for (int i = 0; i < BATCH; ++i) v[i] = *reinterpret_cast<const Vec16<IO>*>(p + (size_t)(r + i) * pitch);
 #pragma unroll
     for (int i = 0; i < BATCH; ++i)
 #pragma unroll
@@ -92,7 +93,7 @@ static __device__ __forceinline__ void pool_body(const typename IO::raw* __restr
       }
   }
   for (; r < nrows; ++r) {
-    Vec16<IO> v = *reinterpret_cast<const Vec16<IO>*>(p + (size_t)r * D);
+    Vec16<IO> v = *reinterpret_cast<const Vec16<IO>*>(p + (size_t)r * pitch);
 #pragma unroll
     for (int e = 0; e < VEC; ++e) {
       float f = IO::ld(v.e[e]);
@@ -115,10 +116,10 @@ static __device__ __forceinline__ void pool_body(const typename IO::raw* __restr
 }
 
 template <typename IO, int MODE>
-__global__ __launch_bounds__(256) void pool_kernel(const typename IO::raw* __restrict__ x,
+__global__ __launch_bounds__(256) void pool_kernel(const typename IO::raw* __restrict__ x, const RowLayout lay,
                                                    const typename IO::raw* __restrict__ colmean,
                                                    void* __restrict__ out, int L, int D, int BLK, int nblk) {
-  pool_body<IO, MODE>(x, colmean, out, L, D, BLK, nblk, blockIdx.x, blockIdx.y);
+  pool_body<IO, MODE>(x, lay, colmean, out, L, D, BLK, nblk, blockIdx.x, blockIdx.y);
 }
 
 // The two independent first passes of the mask builder in one launch (neither fills the memory system alone):
@@ -126,11 +127,12 @@ __global__ __launch_bounds__(256) void pool_kernel(const typename IO::raw* __res
 template <typename IO>
 __global__ __launch_bounds__(256) void pool_pair_kernel(const typename IO::raw* __restrict__ k, float* __restrict__ chunk_sums,
                                                         int nchunk, const typename IO::raw* __restrict__ q,
-                                                        typename IO::raw* __restrict__ pq, int BLKQ, int nblkq, int L, int D) {
+                                                        const RowLayout lay, typename IO::raw* __restrict__ pq, int BLKQ,
+                                                        int nblkq, int L, int D) {
   if (blockIdx.z == 0)
-    pool_body<IO, 0>(k, nullptr, chunk_sums, L, D, KMEAN_CHUNK, nchunk, blockIdx.x, blockIdx.y);
+    pool_body<IO, 0>(k, lay, nullptr, chunk_sums, L, D, KMEAN_CHUNK, nchunk, blockIdx.x, blockIdx.y);
   else
-    pool_body<IO, 1>(q, nullptr, pq, L, D, BLKQ, nblkq, blockIdx.x, blockIdx.y);
+    pool_body<IO, 1>(q, lay, nullptr, pq, L, D, BLKQ, nblkq, blockIdx.x, blockIdx.y);
 }
 
 // Column mean of K, levels 2 and 3 of the fixed summation order:
@@ -398,11 +400,12 @@ static int validate_pool(int dtype, int BH, int L, int D, int BLK) {
 }
 
 template <typename IO, int MODE>
-static void launch_pool(const void* x, const void* colmean, void* out, int BH, int L, int D, int BLK, hipStream_t st) {
+static void launch_pool(const void* x, const RowLayout& lay, const void* colmean, void* out, int BH, int L, int D, int BLK,
+                        hipStream_t st) {
   const int nblk = cdiv(L, BLK);
   const int bpw = 256 / (D / IO::VEC);
   dim3 grid(cdiv(nblk, bpw), BH);
-  hipLaunchKernelGGL((pool_kernel<IO, MODE>), grid, dim3(256), 0, st, (const typename IO::raw*)x,
+  hipLaunchKernelGGL((pool_kernel<IO, MODE>), grid, dim3(256), 0, st, (const typename IO::raw*)x, lay,
                      (const typename IO::raw*)colmean, out, L, D, BLK, nblk);
 }
 
@@ -422,13 +425,13 @@ static void launch_colmean_reduce(float* chunk_sums, float* group_sums, typename
 template <typename IO>
 static void launch_k_colmean_t(const void* k, int BH, int L, int D, float* chunk_sums, float* group_sums,
                                typename IO::raw* colmean, hipStream_t st) {
-  launch_pool<IO, 0>(k, nullptr, chunk_sums, BH, L, D, KMEAN_CHUNK, st);
+  launch_pool<IO, 0>(k, contiguous_layout(BH, L, D), nullptr, chunk_sums, BH, L, D, KMEAN_CHUNK, st);
   launch_colmean_reduce<IO>(chunk_sums, group_sums, colmean, BH, L, D, st);
 }
 
 template <typename IO>
-static int block_map_impl(const void* q, const void* k, int dtype, int BH, int L, int D, int BLKQ, int BLKK, int topk,
-                          char* ws, int8_t* sparse_map, void* lut, int lut64, hipStream_t st) {
+static int block_map_impl(const void* q, const void* k, const RowLayout& lay, int dtype, int BH, int L, int D, int BLKQ,
+                          int BLKK, int topk, char* ws, int8_t* sparse_map, void* lut, int lut64, hipStream_t st) {
   const MapWs w = map_ws(dtype, BH, L, D, BLKQ, BLKK);
   const int M = cdiv(L, BLKQ), N = cdiv(L, BLKK);
   float* chunk_sums = (float*)(ws + w.chunk_sums);
@@ -442,10 +445,10 @@ static int block_map_impl(const void* q, const void* k, int dtype, int BH, int L
     const int bpw = 256 / (D / IO::VEC);
     dim3 grid(cdiv(max(nchunk, M), bpw), BH, 2);
     hipLaunchKernelGGL((pool_pair_kernel<IO>), grid, dim3(256), 0, st, (const typename IO::raw*)k, chunk_sums, nchunk,
-                       (const typename IO::raw*)q, pq, BLKQ, M, L, D);
+                       (const typename IO::raw*)q, lay, pq, BLKQ, M, L, D);
   }
   launch_colmean_reduce<IO>(chunk_sums, (float*)(ws + w.group_sums), colmean, BH, L, D, st);
-  launch_pool<IO, 2>(k, colmean, pk, BH, L, D, BLKK, st);
+  launch_pool<IO, 2>(k, lay, colmean, pk, BH, L, D, BLKK, st);
   hipLaunchKernelGGL((score_kernel<IO>), dim3(cdiv(N, 64), cdiv(M, 64), BH), dim3(256), 0, st, pq, pk, score, M, N, D);
   // topk == 0 selects nothing: the kernel then only clears the map row.
   launch_topk<IO>(score, sparse_map, lut, lut64, N, topk, (size_t)BH * M, st);
@@ -496,15 +499,16 @@ extern "C" int sla_mean_pool(const void* x, void* out, int dtype, int BH, int L,
   SLA_REQUIRE(x && out, SLA_ERR_BAD_ARG, "null pointer");
   SLA_REQUIRE(((uintptr_t)x | (uintptr_t)out) % 16 == 0, SLA_ERR_BAD_ARG, "pointers must be 16-byte aligned");
   hipStream_t st = (hipStream_t)stream;
-  if (dtype == SLA_F32) launch_pool<IoF32, 1>(x, nullptr, out, BH, L, D, BLK, st);
-  else if (dtype == SLA_BF16) launch_pool<IoBf16, 1>(x, nullptr, out, BH, L, D, BLK, st);
-  else launch_pool<IoF16, 1>(x, nullptr, out, BH, L, D, BLK, st);
+  const RowLayout lay = contiguous_layout(BH, L, D);
+  if (dtype == SLA_F32) launch_pool<IoF32, 1>(x, lay, nullptr, out, BH, L, D, BLK, st);
+  else if (dtype == SLA_BF16) launch_pool<IoBf16, 1>(x, lay, nullptr, out, BH, L, D, BLK, st);
+  else launch_pool<IoF16, 1>(x, lay, nullptr, out, BH, L, D, BLK, st);
   return check_launch("mean_pool");
 }
 
-extern "C" int sla_block_map_fwd(const void* q, const void* k, int dtype, int B, int H, int L, int D, int BLKQ, int BLKK,
-                                 int topk, void* workspace, int64_t workspace_bytes, int8_t* sparse_map, void* lut,
-                                 int lut_elem_bytes, void* stream) {
+static int block_map_entry(const void* q, const void* k, const int64_t* strides, int dtype, int B, int H, int L, int D,
+                           int BLKQ, int BLKK, int topk, void* workspace, int64_t workspace_bytes, int8_t* sparse_map,
+                           void* lut, int lut_elem_bytes, void* stream) {
   SLA_REQUIRE(B > 0 && H > 0, SLA_ERR_BAD_ARG, "non-positive batch/head count (B=%d H=%d)", B, H);
   const int64_t BH64 = (int64_t)B * H;
   SLA_REQUIRE(BH64 <= 65535, SLA_ERR_UNSUPPORTED, "B*H=%lld exceeds 65535", (long long)BH64);
@@ -525,10 +529,31 @@ extern "C" int sla_block_map_fwd(const void* q, const void* k, int dtype, int B,
   const int64_t need = block_map_workspace_bytes(dtype, BH, L, D, BLKQ, BLKK);
   SLA_REQUIRE(workspace_bytes >= need, SLA_ERR_WORKSPACE, "workspace of %lld bytes, need %lld", (long long)workspace_bytes,
               (long long)need);
+  RowLayout lay;
+  rc = make_layout(strides, B, H, L, D, dtype == SLA_F32 ? 4 : 2, &lay);
+  if (rc) return rc;
   hipStream_t st = (hipStream_t)stream;
   char* ws = (char*)workspace;
   const int lut64 = lut_elem_bytes == 8;
-  if (dtype == SLA_F32) return block_map_impl<IoF32>(q, k, dtype, BH, L, D, BLKQ, BLKK, topk, ws, sparse_map, lut, lut64, st);
-  if (dtype == SLA_BF16) return block_map_impl<IoBf16>(q, k, dtype, BH, L, D, BLKQ, BLKK, topk, ws, sparse_map, lut, lut64, st);
-  return block_map_impl<IoF16>(q, k, dtype, BH, L, D, BLKQ, BLKK, topk, ws, sparse_map, lut, lut64, st);
+  if (dtype == SLA_F32)
+    return block_map_impl<IoF32>(q, k, lay, dtype, BH, L, D, BLKQ, BLKK, topk, ws, sparse_map, lut, lut64, st);
+  if (dtype == SLA_BF16)
+    return block_map_impl<IoBf16>(q, k, lay, dtype, BH, L, D, BLKQ, BLKK, topk, ws, sparse_map, lut, lut64, st);
+  return block_map_impl<IoF16>(q, k, lay, dtype, BH, L, D, BLKQ, BLKK, topk, ws, sparse_map, lut, lut64, st);
+}
+
+extern "C" int sla_block_map_fwd(const void* q, const void* k, int dtype, int B, int H, int L, int D, int BLKQ, int BLKK,
+                                 int topk, void* workspace, int64_t workspace_bytes, int8_t* sparse_map, void* lut,
+                                 int lut_elem_bytes, void* stream) {
+  return block_map_entry(q, k, nullptr, dtype, B, H, L, D, BLKQ, BLKK, topk, workspace, workspace_bytes, sparse_map, lut,
+                         lut_elem_bytes, stream);
+}
+
+extern "C" int sla_block_map_fwd_strided(const void* q, const void* k, const int64_t* qk_strides, int dtype, int B, int H,
+                                         int L, int D, int BLKQ, int BLKK, int topk, void* workspace,
+                                         int64_t workspace_bytes, int8_t* sparse_map, void* lut, int lut_elem_bytes,
+                                         void* stream) {
+  SLA_REQUIRE(qk_strides, SLA_ERR_BAD_ARG, "null strides");
+  return block_map_entry(q, k, qk_strides, dtype, B, H, L, D, BLKQ, BLKK, topk, workspace, workspace_bytes, sparse_map, lut,
+                         lut_elem_bytes, stream);
 }

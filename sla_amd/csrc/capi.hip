@@ -21,6 +21,26 @@ int check_launch(const char* what) {
   return SLA_OK;
 }
 
+int make_layout(const int64_t* strides, int B, int H, int L, int D, int elem_bytes, RowLayout* out) {
+  if (!strides) {
+    *out = contiguous_layout(H, L, D);
+    return SLA_OK;
+  }
+  const int64_t sb = strides[0], sh = strides[1], sl = strides[2];
+  const int64_t vec = 16 / elem_bytes;     // elements per 16-byte access
+  SLA_REQUIRE(sl >= D && sh > 0 && sb > 0, SLA_ERR_BAD_ARG, "strides (%lld, %lld, %lld): the row stride must be at least D=%d and all must be positive",
+              (long long)sb, (long long)sh, (long long)sl, D);
+  SLA_REQUIRE(sb % vec == 0 && sh % vec == 0 && sl % vec == 0, SLA_ERR_BAD_ARG,
+              "strides (%lld, %lld, %lld) must be multiples of %lld elements (16-byte aligned rows)", (long long)sb,
+              (long long)sh, (long long)sl, (long long)vec);
+  // rows of one head must not run into each other or into another head's rows of the same token
+  SLA_REQUIRE(sh >= D || sh >= (int64_t)L * sl, SLA_ERR_BAD_ARG, "head stride %lld overlaps rows of width D=%d", (long long)sh, D);
+  SLA_REQUIRE(((int64_t)(L - 1) * sl + D) * elem_bytes < (1ll << 32) - 65536, SLA_ERR_UNSUPPORTED,
+              "one head spans 4 GiB or more with row stride %lld", (long long)sl);
+  *out = RowLayout{sb, sh, sl, H};
+  return SLA_OK;
+}
+
 int64_t block_map_workspace_bytes(int dtype, int BH, int L, int D, int BLKQ, int BLKK);
 int64_t sparse_bwd_workspace_bytes(int BH, int L, int D, int BLKQ, int BLKK, int topk);
 int64_t linear_fwd_workspace_bytes(int BH, int L, int D);

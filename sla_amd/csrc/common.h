@@ -136,13 +136,13 @@ struct TileRows {
   static constexpr int CPR = D / 8, N = 32 * CPR / 64, SSTR = D + 8;
   i16x8_t x[N];
 
-  // global -> registers; rows at or past rows_valid read as zero
-  __device__ __forceinline__ void fetch(const uint16_t* gtile, int rows_valid, int lane) {
+  // global -> registers; rows at or past rows_valid read as zero; `pitch` = elements between rows in memory
+  __device__ __forceinline__ void fetch(const uint16_t* gtile, int rows_valid, int lane, size_t pitch = D) {
 #pragma unroll
     for (int i = 0; i < N; ++i) {
       const int idx = lane + 64 * i, row = idx / CPR, col = (idx % CPR) * 8;
       x[i] = i16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
-      if (row < rows_valid) x[i] = *reinterpret_cast<const i16x8_t*>(gtile + (size_t)row * D + col);
+      if (row < rows_valid) x[i] = *reinterpret_cast<const i16x8_t*>(gtile + (size_t)row * pitch + col);
     }
   }
   // registers -> the wave's staging tile
@@ -163,11 +163,11 @@ struct TileRows {
     }
   }
   // registers -> global
-  __device__ __forceinline__ void store(uint16_t* gtile, int rows_valid, int lane) const {
+  __device__ __forceinline__ void store(uint16_t* gtile, int rows_valid, int lane, size_t pitch = D) const {
 #pragma unroll
     for (int i = 0; i < N; ++i) {
       const int idx = lane + 64 * i, row = idx / CPR, col = (idx % CPR) * 8;
-      if (row < rows_valid) *reinterpret_cast<i16x8_t*>(gtile + (size_t)row * D + col) = x[i];
+      if (row < rows_valid) *reinterpret_cast<i16x8_t*>(gtile + (size_t)row * pitch + col) = x[i];
     }
   }
   // this += other, element-wise in fp32 with one rounding
@@ -241,5 +241,24 @@ static __device__ __forceinline__ int xcd_remap(int wg, int grid, int total) {
 }
 
 static inline int xcd_grid(int64_t total) { return (int)((total + 7) / 8 * 8); }
+
+// Where the rows of a (B, H, L, D) tensor lie in memory: row l of head (b, h) starts `b*sb + h*sh + l*sl`
+// elements after the base pointer, its D elements are adjacent.  The contiguous (B, H, L, D) tensor of the
+// reference has (H*L*D, L*D, D); a (B, L, H, D) activation viewed as (B, H, L, D) has (L*H*D, D, H*D), and
+// the q / k / v slices of a packed (B, L, 3, H, D) projection have (L*3*H*D, D, 3*H*D).
+struct RowLayout {
+  int64_t sb, sh, sl;
+  int H;
+  __host__ __device__ size_t head(int bh) const { return (size_t)(bh / H) * (size_t)sb + (size_t)(bh % H) * (size_t)sh; }
+  // bytes from the first element of a head to the end of its last row (the range of a buffer descriptor:
+  // rows past L then lie outside it and read as zero)
+  __host__ __device__ uint32_t head_range_bytes(int L, int D) const { return (uint32_t)(((int64_t)(L - 1) * sl + D) * 2); }
+};
+static inline RowLayout contiguous_layout(int H, int L, int D) {
+  return RowLayout{(int64_t)H * L * D, (int64_t)L * D, (int64_t)D, H};
+}
+// strides = {batch, head, row} in elements, or null for the contiguous (B, H, L, D) tensor.  Checks what the
+// kernels rely on: rows do not overlap, every row starts 16-byte aligned, one head spans less than 4 GiB.
+int make_layout(const int64_t* strides, int B, int H, int L, int D, int elem_bytes, RowLayout* out);
 
 }  // namespace sla

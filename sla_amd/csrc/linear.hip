@@ -140,10 +140,10 @@ int64_t linear_fwd_workspace_bytes(int BH, int L, int D) { return (int64_t)lin_w
 int64_t linear_states_bytes(int BH, int L, int D) { return (int64_t)lin_ws(BH, L, D).states_end; }
 
 template <typename Tag, int D>
-static int linear_state_impl(const void* k, const void* v, const float* weight, int fmap, int BH, int L, char* ws,
-                             hipStream_t st) {
+static int linear_state_impl(const void* k, const void* v, const RowLayout& lay, const float* weight, int fmap, int BH, int L,
+                             char* ws, hipStream_t st) {
   const LinWs w = lin_ws(BH, L, D);
-  launch_state_build<Tag, D>(k, v, weight, fmap, BH, L, ws, w, st);
+  launch_state_build<Tag, D>(k, v, lay, weight, fmap, BH, L, ws, w, st);
   hipLaunchKernelGGL((linear_fold_kernel<Tag>), dim3(cdiv(D * D, 256), BH), dim3(256), 0, st,
                      (const uint16_t*)(ws + w.kvt), weight, (uint16_t*)(ws + w.kvwt), D);
   return check_launch("linear_state_fwd");
@@ -183,8 +183,8 @@ static int check_linear_ws(int BH, int L, int D, const void* workspace, int64_t 
   return SLA_OK;
 }
 
-extern "C" int sla_linear_state_fwd(const void* k, const void* v, const float* weight, int dtype, int fmap, int B, int H,
-                                    int L, int D, void* workspace, int64_t workspace_bytes, void* stream) {
+static int linear_state_entry(const void* k, const void* v, const int64_t* strides, const float* weight, int dtype, int fmap,
+                              int B, int H, int L, int D, void* workspace, int64_t workspace_bytes, void* stream) {
   int rc = validate_linear(dtype, fmap, B, H, L, D);
   if (rc) return rc;
   SLA_REQUIRE(k && v && weight, SLA_ERR_BAD_ARG, "null pointer");
@@ -193,9 +193,12 @@ extern "C" int sla_linear_state_fwd(const void* k, const void* v, const float* w
   const int BH = B * H;
   rc = check_linear_ws(BH, L, D, workspace, workspace_bytes);
   if (rc) return rc;
+  RowLayout lay;
+  rc = make_layout(strides, B, H, L, D, 2, &lay);
+  if (rc) return rc;
   hipStream_t st = (hipStream_t)stream;
   char* ws = (char*)workspace;
-#define SLA_LIN_CASE(TAG, DD) return linear_state_impl<TAG, DD>(k, v, weight, fmap, BH, L, ws, st)
+#define SLA_LIN_CASE(TAG, DD) return linear_state_impl<TAG, DD>(k, v, lay, weight, fmap, BH, L, ws, st)
   if (dtype == SLA_BF16) {
     if (D == 128) SLA_LIN_CASE(bf16_tag, 128);
     SLA_LIN_CASE(bf16_tag, 64);
@@ -203,6 +206,18 @@ extern "C" int sla_linear_state_fwd(const void* k, const void* v, const float* w
   if (D == 128) SLA_LIN_CASE(f16_tag, 128);
   SLA_LIN_CASE(f16_tag, 64);
 #undef SLA_LIN_CASE
+}
+
+extern "C" int sla_linear_state_fwd(const void* k, const void* v, const float* weight, int dtype, int fmap, int B, int H,
+                                    int L, int D, void* workspace, int64_t workspace_bytes, void* stream) {
+  return linear_state_entry(k, v, nullptr, weight, dtype, fmap, B, H, L, D, workspace, workspace_bytes, stream);
+}
+
+extern "C" int sla_linear_state_fwd_strided(const void* k, const void* v, const int64_t* kv_strides, const float* weight,
+                                            int dtype, int fmap, int B, int H, int L, int D, void* workspace,
+                                            int64_t workspace_bytes, void* stream) {
+  SLA_REQUIRE(kv_strides, SLA_ERR_BAD_ARG, "null strides");
+  return linear_state_entry(k, v, kv_strides, weight, dtype, fmap, B, H, L, D, workspace, workspace_bytes, stream);
 }
 
 extern "C" int sla_linear_out_fwd(const void* q, const float* bias, const void* residual, void* out, int dtype, int fmap,

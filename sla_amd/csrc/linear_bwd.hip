@@ -603,7 +603,7 @@ static int linear_bwd_impl(const void* q, const void* k, const void* v, const fl
                            char* ws, hipStream_t st) {
   const LinBwdWs w = lin_bwd_ws(BH, L, D);
   const int accumulate = flags & SLA_BWD_ACCUMULATE;
-  if (!(flags & SLA_BWD_STATES_READY)) launch_state_build<Tag, D>(k, v, weight, fmap, BH, L, ws, w.fwd, st);
+  if (!(flags & SLA_BWD_STATES_READY)) launch_state_build<Tag, D>(k, v, contiguous_layout(BH, L, D), weight, fmap, BH, L, ws, w.fwd, st);
   uint16_t* kvt = (uint16_t*)(ws + w.fwd.kvt);
   uint16_t* z = (uint16_t*)(ws + w.fwd.z);
   uint16_t* dn = (uint16_t*)(ws + w.dn);

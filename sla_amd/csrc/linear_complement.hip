@@ -309,7 +309,7 @@ static int complement_impl(const void* q, const void* k, const void* v, const vo
   float* hall = (float*)(ws + w.hall);
   float* zall = (float*)(ws + w.zall);
   hipLaunchKernelGGL((linear_state_partial_kernel<Tag, D, true>), dim3(N, BH), dim3(256), 0, st, (const uint16_t*)k,
-                     (const uint16_t*)v, (void*)hblk, zblk, L, 64, fmap);
+                     (const uint16_t*)v, contiguous_layout(BH, L, D), (void*)hblk, zblk, L, 64, fmap);
   float* hgrp = (float*)(ws + w.hgrp);
   float* zgrp = (float*)(ws + w.zgrp);
   hipLaunchKernelGGL((complement_group_kernel<Tag>), dim3(cdiv(D * D / 8, 256), w.ngroup, BH), dim3(256), 0, st, hblk, zblk,

@@ -9,9 +9,9 @@ namespace sla {
 // OUT16: the D x D partial is written rounded to 16 bit (per-key-block states of the complement mode).
 template <typename Tag, int D, bool OUT16 = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void linear_state_partial_kernel(const uint16_t* __restrict__ k,
-                                                                   const uint16_t* __restrict__ v, void* __restrict__ kv_part_,
-                                                                   float* __restrict__ z_part, int L, int rows_per_split,
-                                                                   int fmap) {
+                                                                   const uint16_t* __restrict__ v, const RowLayout lay,
+                                                                   void* __restrict__ kv_part_, float* __restrict__ z_part,
+                                                                   int L, int rows_per_split, int fmap) {
   using E = Elem<Tag>;
   constexpr int TR = 64;                 // rows per LDS tile
   constexpr int STR = D + 16;            // LDS row stride: transposed reads of 4 rows hit disjoint banks
@@ -31,8 +31,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
   const int g = lane >> 5;
   const int row_begin = split * rows_per_split;
   const int row_end = min(L, row_begin + rows_per_split);
-  const uint16_t* kh = k + (size_t)bh * L * D;
-  const uint16_t* vh = v + (size_t)bh * L * D;
+  const uint16_t* kh = k + lay.head(bh);
+  const uint16_t* vh = v + lay.head(bh);
+  const size_t pitch = (size_t)lay.sl;
 
   const int lrow = tid / CPR, lcol = (tid % CPR) * 8;
 
@@ -58,8 +59,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
       kreg[p] = i16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
       vreg[p] = i16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
       if (grow < row_end) {
-        kreg[p] = *reinterpret_cast<const i16x8_t*>(kh + (size_t)grow * D + lcol);
-        vreg[p] = *reinterpret_cast<const i16x8_t*>(vh + (size_t)grow * D + lcol);
+        kreg[p] = *reinterpret_cast<const i16x8_t*>(kh + (size_t)grow * pitch + lcol);
+        vreg[p] = *reinterpret_cast<const i16x8_t*>(vh + (size_t)grow * pitch + lcol);
       }
     }
   };
@@ -236,14 +237,14 @@ static inline LinWs lin_ws(int BH, int L, int D) {
 
 // Streams K and V once and leaves KVT, KVP, z (16 bit) and the 16-bit transposed weight in the workspace.
 template <typename Tag, int D>
-static inline void launch_state_build(const void* k, const void* v, const float* weight, int fmap, int BH, int L, char* ws,
-                                      const LinWs& w, hipStream_t st) {
+static inline void launch_state_build(const void* k, const void* v, const RowLayout& lay, const float* weight, int fmap,
+                                      int BH, int L, char* ws, const LinWs& w, hipStream_t st) {
   float* kv_part = (float*)(ws + w.kv_part);
   float* z_part = (float*)(ws + w.z_part);
   uint16_t* kvt = (uint16_t*)(ws + w.kvt);
   uint16_t* z = (uint16_t*)(ws + w.z);
   hipLaunchKernelGGL((linear_state_partial_kernel<Tag, D>), dim3(w.nsplit, BH), dim3(256), 0, st, (const uint16_t*)k,
-                     (const uint16_t*)v, kv_part, z_part, L, w.rows_per_split, fmap);
+                     (const uint16_t*)v, lay, kv_part, z_part, L, w.rows_per_split, fmap);
   hipLaunchKernelGGL((linear_state_reduce_kernel<Tag>), dim3(cdiv(D * D, 256), BH), dim3(256), 0, st, kv_part, z_part, kvt,
                      (uint16_t*)(ws + w.kvp), z, w.nsplit, D * D, D);
   hipLaunchKernelGGL((linear_prep_weight_kernel<Tag>), dim3(cdiv(D * D, 256)), dim3(256), 0, st, weight,

@@ -26,7 +26,8 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
                                                               const uint16_t* __restrict__ k,
                                                               const uint16_t* __restrict__ v,
                                                               const void* __restrict__ lut, int lut64,
-                                                              uint16_t* __restrict__ o, float* __restrict__ lse, int L,
+                                                              uint16_t* __restrict__ o, float* __restrict__ lse,
+                                                              const RowLayout lin, const RowLayout lout, int L,
                                                               int Mblk, int topk, float scale_log2e, int total,
                                                               const uint16_t* __restrict__ kvwt,
                                                               const uint16_t* __restrict__ zst,
@@ -58,8 +59,10 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
   const int g = lane >> 5;                  // which half of the MFMA contraction slots this lane feeds
   const int r = lane & 31;                  // query column (S^T, O^T) / key row (A operand)
 
-  const size_t head_off = (size_t)bh * L * D;
-  const uint32_t head_bytes = (uint32_t)L * D * 2;
+  // q, k, v rows of this head: lin.sl elements apart (D for the contiguous layout); out rows: lout.sl apart
+  const size_t head_off = lin.head(bh);
+  const uint32_t pitch = (uint32_t)lin.sl;
+  const uint32_t head_bytes = lin.head_range_bytes(L, D);
   const __amdgpu_buffer_rsrc_t kh = make_rsrc(k + head_off, head_bytes);
   const __amdgpu_buffer_rsrc_t vh = make_rsrc(v + head_off, head_bytes);
 
@@ -72,7 +75,7 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
   uint16_t* const stage = smem + wave * 32 * TileRows<D>::SSTR;
   static_assert(BLKQ / 32 * 32 * TileRows<D>::SSTR <= BLKK * KSTR + BLKK * VSTR, "staging tiles exceed the K/V buffers");
   TileRows<D> qt;
-  qt.fetch(q + head_off + (size_t)qrow0 * D, qrows_valid, lane);   // rows past L: 0
+  qt.fetch(q + head_off + (size_t)qrow0 * pitch, qrows_valid, lane, pitch);   // rows past L: 0
 
   const size_t lut_row = ((size_t)bh * Mblk + mb) * topk;
   auto lut_at = [&](int i) -> int {
@@ -89,7 +92,7 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
       const int idx = tid + i * NT;
       const int row = idx / CPR, col = (idx % CPR) * 8;
       // rows past L lie beyond the buffer range and read as zero (0 * garbage could be NaN)
-      dst[i] = buf_load_b128(base, ((uint32_t)(nb * BLKK + row) * D + col) * 2);
+      dst[i] = buf_load_b128(base, ((uint32_t)(nb * BLKK + row) * pitch + col) * 2);
     }
   };
   auto store_rows_from = [&](const i16x8_t (&src)[NLD], uint16_t* dst, int stride) {
@@ -311,7 +314,7 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
   const float inv = 1.0f / l_tot;
   // (the loop ended with a barrier: every wave is done with the K/V buffers, the staging tiles are free)
   constexpr int SSTR = TileRows<D>::SSTR;
-  const size_t tile_off = head_off + (size_t)qrow0_e * D;
+  const size_t out_off = lout.head(bh) + (size_t)qrow0_e * (size_t)lout.sl;
   if (qrow_e < L && g_e == 0) lse[(size_t)bh * L + qrow_e] = m_run + fast_log2(l_tot);
   // normalised attention output of this lane, packed, into its row of the staging tile
   auto park_attention = [&]() {
@@ -326,15 +329,15 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
       }
     wave_lds_fence();
   };
-  auto flush_rows = [&](uint16_t* dst) {   // staging tile -> global rows
+  auto flush_rows = [&](uint16_t* dst_tile, size_t dst_pitch) {   // staging tile -> global rows
     TileRows<D> t;
     t.unpark(stage_e, lane_e);
-    t.store(dst + tile_off, qrows_valid_e, lane_e);
+    t.store(dst_tile, qrows_valid_e, lane_e, dst_pitch);
     wave_lds_fence();
   };
   if (!FUSED) {
     park_attention();
-    flush_rows(o);
+    flush_rows(o + out_off, (size_t)lout.sl);
   } else {
     // ---- linear branch of the same rows ----
     // The per-head state (32 KB) is read straight from L2 in MFMA A-operand order (row 32et + r, 16-byte
@@ -393,10 +396,10 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
       }
     }
     wave_lds_fence();
-    flush_rows(o);
-    if (o_s) {
+    flush_rows(o + out_off, (size_t)lout.sl);
+    if (o_s) {                 // (kept for a backward: always the contiguous (B, H, L, D) tensor)
       park_attention();
-      flush_rows(o_s);
+      flush_rows(o_s + ((size_t)bh * L + qrow0_e) * D, D);
     }
   }
 }
@@ -410,8 +413,9 @@ struct FusedLinear {        // state of the linear branch for the fused epilogue
 };
 
 template <typename Tag>
-static int launch_fwd(const void* q, const void* k, const void* v, const void* lut, int lut64, void* o, float* lse, int BH,
-                      int L, int D, int BLKQ, int topk, float qk_scale, const FusedLinear* fl, hipStream_t st) {
+static int launch_fwd(const void* q, const void* k, const void* v, const void* lut, int lut64, void* o, float* lse,
+                      const RowLayout& lin, const RowLayout& lout, int BH, int L, int D, int BLKQ, int topk, float qk_scale,
+                      const FusedLinear* fl, hipStream_t st) {
   const int Mblk = cdiv(L, BLKQ);
   const int64_t total64 = (int64_t)BH * Mblk;
   const int total = (int)total64;
@@ -421,12 +425,12 @@ static int launch_fwd(const void* q, const void* k, const void* v, const void* l
   if (D == DD && BLKQ == BQ) {                                                                                        \
     if (fl)                                                                                                           \
       hipLaunchKernelGGL((sparse_fwd_kernel<Tag, DD, BQ, true>), dim3(grid), dim3(BQ * 2), 0, st, (const uint16_t*)q, \
-                         (const uint16_t*)k, (const uint16_t*)v, lut, lut64, (uint16_t*)o, lse, L, Mblk, topk, c,    \
-                         total, fl->kvwt, fl->zst, fl->bias, fl->fmap, fl->o_s);                                      \
+                         (const uint16_t*)k, (const uint16_t*)v, lut, lut64, (uint16_t*)o, lse, lin, lout, L, Mblk,   \
+                         topk, c, total, fl->kvwt, fl->zst, fl->bias, fl->fmap, fl->o_s);                             \
     else                                                                                                              \
       hipLaunchKernelGGL((sparse_fwd_kernel<Tag, DD, BQ, false>), dim3(grid), dim3(BQ * 2), 0, st,                   \
                          (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, lut, lut64, (uint16_t*)o, lse,  \
-                         L, Mblk, topk, c, total, (const uint16_t*)nullptr, (const uint16_t*)nullptr,                 \
+                         lin, lout, L, Mblk, topk, c, total, (const uint16_t*)nullptr, (const uint16_t*)nullptr,      \
                          (const float*)nullptr, 0, (uint16_t*)nullptr);                                               \
     return check_launch("sparse_attn_fwd");                                                                           \
   }
@@ -469,15 +473,18 @@ extern "C" int sla_sparse_attn_fwd(const void* q, const void* k, const void* v, 
               "q, k, v, o must be 16-byte aligned");
   hipStream_t st = (hipStream_t)stream;
   const int BH = B * H;
+  const RowLayout lay = contiguous_layout(H, L, D);
   if (dtype == SLA_BF16)
-    return launch_fwd<bf16_tag>(q, k, v, lut, lut_elem_bytes == 8, o, lse, BH, L, D, BLKQ, topk, qk_scale, nullptr, st);
-  return launch_fwd<f16_tag>(q, k, v, lut, lut_elem_bytes == 8, o, lse, BH, L, D, BLKQ, topk, qk_scale, nullptr, st);
+    return launch_fwd<bf16_tag>(q, k, v, lut, lut_elem_bytes == 8, o, lse, lay, lay, BH, L, D, BLKQ, topk, qk_scale, nullptr,
+                                st);
+  return launch_fwd<f16_tag>(q, k, v, lut, lut_elem_bytes == 8, o, lse, lay, lay, BH, L, D, BLKQ, topk, qk_scale, nullptr, st);
 }
 
-extern "C" int sla_sparse_attn_linear_fwd(const void* q, const void* k, const void* v, const void* lut, int lut_elem_bytes,
-                                          const void* linear_workspace, int64_t linear_workspace_bytes, const float* bias,
-                                          void* o_s, void* out, float* lse, int dtype, int fmap, int B, int H, int L, int D,
-                                          int BLKQ, int BLKK, int topk, float qk_scale, void* stream) {
+static int attn_linear_entry(const void* q, const void* k, const void* v, const int64_t* qkv_strides, const void* lut,
+                             int lut_elem_bytes, const void* linear_workspace, int64_t linear_workspace_bytes,
+                             const float* bias, void* o_s, void* out, const int64_t* out_strides, float* lse, int dtype,
+                             int fmap, int B, int H, int L, int D, int BLKQ, int BLKK, int topk, float qk_scale,
+                             void* stream) {
   int rc = validate_attn_shape(dtype, B, H, L, D, BLKQ, BLKK, topk, lut_elem_bytes);
   if (rc) return rc;
   rc = validate_linear(dtype, fmap, B, H, L, D);
@@ -492,8 +499,33 @@ extern "C" int sla_sparse_attn_linear_fwd(const void* q, const void* k, const vo
               (long long)linear_workspace_bytes, (long long)w.total);
   const char* ws = (const char*)linear_workspace;
   FusedLinear fl{(const uint16_t*)(ws + w.kvwt), (const uint16_t*)(ws + w.z), bias, fmap, (uint16_t*)o_s};
+  RowLayout lin, lout;
+  rc = make_layout(qkv_strides, B, H, L, D, 2, &lin);
+  if (rc) return rc;
+  rc = make_layout(out_strides, B, H, L, D, 2, &lout);
+  if (rc) return rc;
   hipStream_t st = (hipStream_t)stream;
   if (dtype == SLA_BF16)
-    return launch_fwd<bf16_tag>(q, k, v, lut, lut_elem_bytes == 8, out, lse, BH, L, D, BLKQ, topk, qk_scale, &fl, st);
-  return launch_fwd<f16_tag>(q, k, v, lut, lut_elem_bytes == 8, out, lse, BH, L, D, BLKQ, topk, qk_scale, &fl, st);
+    return launch_fwd<bf16_tag>(q, k, v, lut, lut_elem_bytes == 8, out, lse, lin, lout, BH, L, D, BLKQ, topk, qk_scale, &fl,
+                                st);
+  return launch_fwd<f16_tag>(q, k, v, lut, lut_elem_bytes == 8, out, lse, lin, lout, BH, L, D, BLKQ, topk, qk_scale, &fl, st);
+}
+
+extern "C" int sla_sparse_attn_linear_fwd(const void* q, const void* k, const void* v, const void* lut, int lut_elem_bytes,
+                                          const void* linear_workspace, int64_t linear_workspace_bytes, const float* bias,
+                                          void* o_s, void* out, float* lse, int dtype, int fmap, int B, int H, int L, int D,
+                                          int BLKQ, int BLKK, int topk, float qk_scale, void* stream) {
+  return attn_linear_entry(q, k, v, nullptr, lut, lut_elem_bytes, linear_workspace, linear_workspace_bytes, bias, o_s, out,
+                           nullptr, lse, dtype, fmap, B, H, L, D, BLKQ, BLKK, topk, qk_scale, stream);
+}
+
+extern "C" int sla_sparse_attn_linear_fwd_strided(const void* q, const void* k, const void* v, const int64_t* qkv_strides,
+                                                  const void* lut, int lut_elem_bytes, const void* linear_workspace,
+                                                  int64_t linear_workspace_bytes, const float* bias, void* o_s, void* out,
+                                                  const int64_t* out_strides, float* lse, int dtype, int fmap, int B, int H,
+                                                  int L, int D, int BLKQ, int BLKK, int topk, float qk_scale,
+                                                  void* stream) {
+  SLA_REQUIRE(qkv_strides && out_strides, SLA_ERR_BAD_ARG, "null strides");
+  return attn_linear_entry(q, k, v, qkv_strides, lut, lut_elem_bytes, linear_workspace, linear_workspace_bytes, bias, o_s,
+                           out, out_strides, lse, dtype, fmap, B, H, L, D, BLKQ, BLKK, topk, qk_scale, stream);
 }

@@ -31,8 +31,14 @@ def linear_state_fwd(k, v, weight, fmap: str):
     B, H, L, D = k.shape
     dt = _lib.dtype_code(k.dtype)
     ws = _lib.workspace(_lib.WS_LINEAR_FWD, dt, B, H, L, D, 64, 64, 0, k.device)
-    rc = _lib.load().sla_linear_state_fwd(k.data_ptr(), v.data_ptr(), weight.data_ptr(), dt, _lib.FMAP[fmap], B, H, L, D,
-                                          ws.data_ptr(), ws.numel(), _lib.stream_ptr(k.device))
+    if k.is_contiguous() and v.is_contiguous():
+        rc = _lib.load().sla_linear_state_fwd(k.data_ptr(), v.data_ptr(), weight.data_ptr(), dt, _lib.FMAP[fmap], B, H, L,
+                                              D, ws.data_ptr(), ws.numel(), _lib.stream_ptr(k.device))
+    else:
+        assert _lib.row_strided(k, v), "k and v must be contiguous or share row-contiguous strides"
+        rc = _lib.load().sla_linear_state_fwd_strided(k.data_ptr(), v.data_ptr(), _lib.strides_arg(k), weight.data_ptr(), dt,
+                                                      _lib.FMAP[fmap], B, H, L, D, ws.data_ptr(), ws.numel(),
+                                                      _lib.stream_ptr(k.device))
     _lib.check(rc)
     return ws
 

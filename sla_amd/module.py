@@ -5,6 +5,7 @@ from __future__ import annotations
 import torch
 import torch.nn as nn
 
+from . import _lib
 from .block_map import get_block_map
 from .linear import linear_bwd, linear_complement_fwd, linear_state_fwd, saved_states
 from .sparse_attn import sparse_attn_bwd, sparse_attn_fwd, sparse_attn_linear_fwd
@@ -21,7 +22,8 @@ class _sla_core(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, q, k, v, weight, bias, sparse_map, lut, topk, BLKQ, BLKK, fmap, state, needs_grad=True):
-        assert q.is_contiguous() and k.is_contiguous() and v.is_contiguous()
+        # (row-contiguous views are accepted on the inference path only: the backward kernels take (B, H, L, D))
+        assert (q.is_contiguous() and k.is_contiguous() and v.is_contiguous()) or not needs_grad
         assert sparse_map.is_contiguous() and lut.is_contiguous()
         assert BLKQ == 64 or BLKQ == 128
         assert BLKK == 64
@@ -125,9 +127,19 @@ class SparseLinearAttention(nn.Module):
             return_sparsity: also return real_topk / n_key_blocks (reference core.py:102-103).
         """
         dtype = q.dtype
-        q = q.contiguous()
-        k = k.contiguous()
-        v = v.contiguous()
+        needs_grad = torch.is_grad_enabled() and any(
+            t.requires_grad for t in (q, k, v, self.proj_l.weight, self.proj_l.bias))
+        # Inference on activations that are not laid out as (B, H, L, D) -- a (B, L, H, D) tensor or the slices
+        # of a packed QKV projection, viewed as (B, H, L, D) -- reads them where they are and writes the output
+        # in the same dimension order, instead of copying three tensors in and one out (the reference makes
+        # the copies: core.py:77-79).  Training and the other cases take the contiguous route.
+        in_place = (not needs_grad and self.linear_mode == "global" and dtype == self.dtype
+                    and not (q.is_contiguous() and k.is_contiguous() and v.is_contiguous())
+                    and _lib.row_strided(q, k, v))
+        if not in_place:
+            q = q.contiguous()
+            k = k.contiguous()
+            v = v.contiguous()
 
         qc = q.to(self.dtype)
         kc = k.to(self.dtype)
@@ -141,8 +153,6 @@ class SparseLinearAttention(nn.Module):
         # the mask is built from the inputs in their own dtype (reference core.py:83)
         sparse_map, lut, real_topk = get_block_map(q, k, topk_ratio=self.topk, BLKQ=self.BLKQ, BLKK=self.BLKK)
 
-        needs_grad = torch.is_grad_enabled() and any(
-            t.requires_grad for t in (qc, kc, vc, weight, self.proj_l.bias))
         o = _sla_core.apply(qc, kc, vc, weight, self.proj_l.bias, sparse_map, lut, real_topk, self.BLKQ,
                             self.BLKK, self.feature_map, state, needs_grad)
         o = o.to(dtype)

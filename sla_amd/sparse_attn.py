@@ -36,17 +36,29 @@ def sparse_attn_linear_fwd(q, k, v, lut, topk, BLOCK_M, BLOCK_N, qk_scale, state
     """Attention forward with the linear branch, projection and sum fused into its epilogue.
 
     ``state_ws`` is the workspace :func:`sla_amd.linear.linear_state_fwd` filled.  Returns ``(out, o_s, lse)``;
-    ``o_s`` (the attention output alone, needed by the backward) is ``None`` unless ``want_o_s``."""
+    ``o_s`` (the attention output alone, needed by the backward) is ``None`` unless ``want_o_s``.
+
+    q, k, v may be row-contiguous views that share their strides (a ``(B, L, H, D)`` activation seen as
+    ``(B, H, L, D)``, slices of a packed projection): ``out`` then has its dimensions ordered in memory like q."""
     _lib.require_gpu(q, k, v, lut, state_ws, bias)
     B, H, L, D = q.shape
-    out = torch.empty_like(v)
-    o_s = torch.empty_like(v) if want_o_s else None
     lse = torch.empty(q.shape[:-1], device=q.device, dtype=torch.float32)
-    rc = _lib.load().sla_sparse_attn_linear_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), lut.data_ptr(), _lut_bytes(lut),
-                                                state_ws.data_ptr(), state_ws.numel(), bias.data_ptr(),
-                                                0 if o_s is None else o_s.data_ptr(), out.data_ptr(), lse.data_ptr(),
-                                                _lib.dtype_code(q.dtype), _lib.FMAP[fmap], B, H, L, D, BLOCK_M, BLOCK_N,
-                                                topk, float(qk_scale), _lib.stream_ptr(q.device))
+    o_s = torch.empty(q.shape, dtype=q.dtype, device=q.device) if want_o_s else None
+    if q.is_contiguous() and k.is_contiguous() and v.is_contiguous():
+        out = torch.empty_like(v)
+        rc = _lib.load().sla_sparse_attn_linear_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), lut.data_ptr(),
+                                                    _lut_bytes(lut), state_ws.data_ptr(), state_ws.numel(), bias.data_ptr(),
+                                                    0 if o_s is None else o_s.data_ptr(), out.data_ptr(), lse.data_ptr(),
+                                                    _lib.dtype_code(q.dtype), _lib.FMAP[fmap], B, H, L, D, BLOCK_M,
+                                                    BLOCK_N, topk, float(qk_scale), _lib.stream_ptr(q.device))
+    else:
+        assert _lib.row_strided(q, k, v), "q, k, v must be contiguous or share row-contiguous strides"
+        out = _lib.empty_like_rows(q)
+        rc = _lib.load().sla_sparse_attn_linear_fwd_strided(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), _lib.strides_arg(q), lut.data_ptr(), _lut_bytes(lut),
+            state_ws.data_ptr(), state_ws.numel(), bias.data_ptr(), 0 if o_s is None else o_s.data_ptr(), out.data_ptr(),
+            _lib.strides_arg(out), lse.data_ptr(), _lib.dtype_code(q.dtype), _lib.FMAP[fmap], B, H, L, D, BLOCK_M, BLOCK_N,
+            topk, float(qk_scale), _lib.stream_ptr(q.device))
     _lib.check(rc)
     return out, o_s, lse
 

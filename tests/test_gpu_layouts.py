@@ -1,0 +1,76 @@
+"""Row-contiguous views as inputs: a (B, L, H, D) activation or the slices of a packed (B, L, 3, H, D) projection,
+seen as (B, H, L, D), must give bit for bit what the contiguous copies give, without being copied."""
+import pytest
+import torch
+
+from sla_amd import SLASelfAttention, SparseLinearAttention, get_block_map
+from sla_amd.inputs import make_proj
+from sla_amd.linear import linear_out_fwd, linear_state_fwd
+
+pytestmark = pytest.mark.gpu
+
+
+def _views(kind, B, H, L, D, dtype, dev, seed):
+    g = torch.Generator().manual_seed(seed)
+    if kind == "blhd":
+        return tuple(torch.randn(B, L, H, D, generator=g).to(dtype).to(dev).permute(0, 2, 1, 3) for _ in range(3))
+    packed = torch.randn(B, L, 3, H, D, generator=g).to(dtype).to(dev)
+    return tuple(packed[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+
+
+@pytest.mark.parametrize("kind", ["blhd", "packed"])
+@pytest.mark.parametrize("B,H,L,D,BLKQ,fmap,dtype,ratio", [(2, 3, 700, 128, 64, "elu", torch.bfloat16, 0.3),
+                                                           (1, 2, 333, 64, 128, "softmax", torch.float16, 0.3),
+                                                           (1, 1, 50, 128, 64, "relu", torch.bfloat16, 1.0)])
+def test_module_reads_views_in_place(dev, kind, B, H, L, D, BLKQ, fmap, dtype, ratio):
+    q, k, v = _views(kind, B, H, L, D, dtype, dev, L)
+    assert not q.is_contiguous() or B * H == 1
+    mod = SparseLinearAttention(D, ratio, fmap, BLKQ, 64, use_bf16=dtype == torch.bfloat16).to(dev)
+    w, b = make_proj(D)
+    with torch.no_grad():
+        mod.proj_l.weight.copy_(w)
+        mod.proj_l.bias.copy_(b)
+        ref = mod(q.contiguous(), k.contiguous(), v.contiguous())
+        m_ref, lut_ref, T = get_block_map(q.contiguous(), k.contiguous(), ratio, BLKQ, 64)
+        m, lut, T2 = get_block_map(q, k, ratio, BLKQ, 64)
+        assert T == T2 and torch.equal(lut, lut_ref) and torch.equal(m, m_ref)
+        out = mod(q, k, v)
+    assert out.shape == ref.shape and torch.equal(out, ref)
+    if not q.is_contiguous():
+        # the output is laid out like the inputs' dimension order: (B, L, H, D) in memory
+        assert out.transpose(1, 2).is_contiguous()
+    # the two-kernel linear branch on views
+    ws = linear_state_fwd(k, v, mod.proj_l.weight.detach(), fmap)
+    ws_ref = linear_state_fwd(k.contiguous(), v.contiguous(), mod.proj_l.weight.detach(), fmap)
+    a = linear_out_fwd(q.contiguous(), mod.proj_l.bias.detach(), None, ws, fmap)
+    b2 = linear_out_fwd(q.contiguous(), mod.proj_l.bias.detach(), None, ws_ref, fmap)
+    assert torch.equal(a, b2)
+
+
+def test_training_on_views_takes_the_contiguous_route(dev):
+    q, k, v = _views("packed", 1, 2, 512, 128, torch.bfloat16, dev, 5)
+    mod = SparseLinearAttention(128, 0.25, "elu").to(dev)
+    w, b = make_proj(128)
+    with torch.no_grad():
+        mod.proj_l.weight.copy_(w)
+        mod.proj_l.bias.copy_(b)
+    qg, kg, vg = (t.detach().requires_grad_(True) for t in (q, k, v))
+    out = mod(qg, kg, vg)
+    out.float().square().mean().backward()
+    with torch.no_grad():
+        ref = mod(q.contiguous(), k.contiguous(), v.contiguous())
+    assert torch.equal(out.detach(), ref) and qg.grad is not None and torch.isfinite(qg.grad.float()).all()
+
+
+def test_block_inference_equals_block_with_copies(dev):
+    torch.manual_seed(0)
+    blk = SLASelfAttention(dim=256, num_heads=2, topk=0.25, feature_map="elu").to(dev).to(torch.bfloat16)
+    blk.attn.proj_l.float()
+    with torch.no_grad():
+        blk.attn.proj_l.weight.normal_(0, 128 ** -0.5)
+        x = torch.randn(2, 640, 256, device=dev, dtype=torch.bfloat16)
+        y = blk(x)
+        qkv = blk.qkv(x).view(2, 640, 3, 2, 128).permute(2, 0, 3, 1, 4).contiguous()
+        o = blk.attn(qkv[0], qkv[1], qkv[2])
+        y_ref = blk.proj(o.transpose(1, 2).reshape(2, 640, 256))
+    assert torch.equal(y, y_ref)
