@@ -97,6 +97,20 @@ def test_other_entry_points_validate():
     assert "headdim" in _lib.last_error()
     assert lib.sage_sparse_attn_fwd(FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, 8, FAKE, 1, 1, 1, 128, 128, 128, 64, 9, 0.1,
                                     None) == _lib.ERR_BAD_ARG
+    # strided variants: strides are {batch, head, row} in elements, checked before anything is launched
+    import ctypes
+    st = lambda *v: (ctypes.c_int64 * 3)(*v)  # noqa: E731
+    bm = lambda strides: lib.sla_block_map_fwd_strided(FAKE, FAKE, strides, 1, 1, 2, 256, 128, 64, 64, 1, FAKE, 1 << 30,  # noqa: E731
+                                                       FAKE, FAKE, 8, None)
+    assert bm(None) == _lib.ERR_BAD_ARG and "strides" in _lib.last_error()
+    assert bm(st(65536, 128, 100)) == _lib.ERR_BAD_ARG          # row stride below D
+    assert bm(st(65536, 128, 260)) == _lib.ERR_BAD_ARG and "16-byte" in _lib.last_error()
+    assert bm(st(1 << 40, 128, 1 << 30)) == _lib.ERR_UNSUPPORTED and "4 GiB" in _lib.last_error()
+    assert lib.sla_linear_state_fwd_strided(FAKE, FAKE, st(65536, 128, 257), FAKE, 1, 0, 1, 2, 256, 128, FAKE, 1 << 30,
+                                            None) == _lib.ERR_BAD_ARG
+    assert lib.sla_sparse_attn_linear_fwd_strided(FAKE, FAKE, FAKE, st(65536, 128, 256), FAKE, 8, FAKE, 1 << 30, FAKE, None,
+                                                  FAKE, st(65536, 128, 4), FAKE, 1, 0, 1, 2, 256, 128, 64, 64, 1, 0.1,
+                                                  None) == _lib.ERR_BAD_ARG
     # one-call SageSLA preparation: block sizes, topk range and workspace are checked before any launch
     prep = lambda BLKQ, topk, ws: lib.sage_prepare(FAKE, FAKE, FAKE, 1, 1, 1, 256, 128, BLKQ, 64, topk, FAKE, FAKE, 8, FAKE,  # noqa: E731
                                                    FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, ws, None)
