@@ -127,8 +127,8 @@ int sla_linear_state_fwd(const void* k, const void* v, const float* weight, int 
 int sla_linear_out_fwd(const void* q, const float* bias, const void* residual, void* out, int dtype, int fmap, int B,
                        int H, int L, int D, void* workspace, int64_t workspace_bytes, void* stream);
 
-/* The module's inference forward for callers whose activations are not laid out as contiguous (B, H, L, D):
- * strided variants of the three calls that touch q, k, v and out.  `*_strides` = {batch, head, row} strides in
+/* For callers whose activations are not laid out as contiguous (B, H, L, D): strided variants of the calls that
+ * touch q, k, v, out and their gradients.  `*_strides` = {batch, head, row} strides in
  * elements of a tensor indexed (b, h, l, d) whose last dimension is contiguous: {H*L*D, L*D, D} for the
  * contiguous layout, {L*H*D, D, H*D} for a (B, L, H, D) activation, {L*3*H*D, D, 3*H*D} for the q / k / v
  * slices of a packed (B, L, 3, H, D) projection.  All strides must be multiples of 8 elements (4 for fp32
@@ -142,6 +142,18 @@ int sla_block_map_fwd_strided(const void* q, const void* k, const int64_t* qk_st
 int sla_linear_state_fwd_strided(const void* k, const void* v, const int64_t* kv_strides, const float* weight, int dtype,
                                  int fmap, int B, int H, int L, int D, void* workspace, int64_t workspace_bytes,
                                  void* stream);
+/* The two backward calls with strides: q, k, v, dq, dk, dv share `qkv_strides` (e.g. slices of one packed
+ * (B, L, 3, H, D) buffer and of its gradient), d_o / d_out has `do_strides`; o (the saved o_s), lse and the
+ * workspaces are contiguous as in the calls without the suffix. */
+int sla_sparse_attn_bwd_strided(const void* q, const void* k, const void* v, const int64_t* qkv_strides, const void* o,
+                                const void* d_o, const int64_t* do_strides, const float* lse, const int8_t* sparse_map,
+                                const void* lut, int lut_elem_bytes, void* dq, void* dk, void* dv, int dtype, int B, int H,
+                                int L, int D, int BLKQ, int BLKK, int topk, float qk_scale, void* workspace,
+                                int64_t workspace_bytes, void* stream);
+int sla_linear_bwd_strided(const void* q, const void* k, const void* v, const int64_t* qkv_strides, const float* weight,
+                           const float* bias, const void* d_out, const int64_t* do_strides, void* dq, void* dk, void* dv,
+                           float* d_weight, float* d_bias, int dtype, int fmap, int B, int H, int L, int D, int flags,
+                           void* workspace, int64_t workspace_bytes, void* stream);
 int sla_sparse_attn_linear_fwd_strided(const void* q, const void* k, const void* v, const int64_t* qkv_strides,
                                        const void* lut, int lut_elem_bytes, const void* linear_workspace,
                                        int64_t linear_workspace_bytes, const float* bias, void* o_s, void* out,

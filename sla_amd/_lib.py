@@ -34,6 +34,10 @@ SIGNATURES = {
     "sla_linear_state_fwd_strided": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I64, _P]),
     "sla_sparse_attn_linear_fwd_strided": (_I, [_P, _P, _P, _P, _P, _I, _P, _I64, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I,
                                                 _I, _I, _I, _I, _F, _P]),
+    "sla_sparse_attn_bwd_strided": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I,
+                                         _I, _F, _P, _I64, _P]),
+    "sla_linear_bwd_strided": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P, _I64,
+                                    _P]),
     "sla_sparse_attn_fwd": (_I, [_P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _P]),
     "sla_sparse_attn_linear_fwd": (_I, [_P, _P, _P, _P, _I, _P, _I64, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I,
                                         _F, _P]),

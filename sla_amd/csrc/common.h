@@ -111,6 +111,8 @@ static __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p
 static __device__ __forceinline__ i16x8_t buf_load_b128(__amdgpu_buffer_rsrc_t r, uint32_t byte_off) {
   return __builtin_bit_cast(i16x8_t, __builtin_amdgcn_raw_buffer_load_b128(r, (int)byte_off, 0, 0));
 }
+// (The whole offset goes into the vector operand on purpose: the scalar offset operand of a buffer load takes no
+//  part in the range check, and the kernels rely on out-of-range rows reading as zero.)
 
 // Orders this wave's LDS writes before its later LDS reads when lanes exchange data through a
 // wave-private region: the hardware keeps one wave's LDS operations in order, this keeps the compiler
@@ -207,15 +209,16 @@ static __device__ __forceinline__ void park_acc_tile(uint16_t* stage, const floa
 // ADD_DEST the addend is what the destination rows hold (read here, while the tile sits in LDS).
 template <typename E, int D, bool ADD_DEST = false>
 static __device__ __forceinline__ void store_acc_tile(uint16_t* stage, const float (&val)[D / 32][16], uint16_t* gtile,
-                                                       const TileRows<D>* addend, int rows_valid, int lane) {
+                                                       const TileRows<D>* addend, int rows_valid, int lane,
+                                                       size_t pitch = D) {
   TileRows<D> old;
-  if (ADD_DEST) old.fetch(gtile, rows_valid, lane);
+  if (ADD_DEST) old.fetch(gtile, rows_valid, lane, pitch);
   park_acc_tile<E, D>(stage, val, lane);
   TileRows<D> t;
   t.unpark(stage, lane);
   if (ADD_DEST) t.template add<E>(old);
   else if (addend) t.template add<E>(*addend);
-  t.store(gtile, rows_valid, lane);
+  t.store(gtile, rows_valid, lane, pitch);
   wave_lds_fence();   // the staging area may be rewritten right after
 }
 

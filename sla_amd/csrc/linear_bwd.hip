@@ -28,7 +28,7 @@ template <typename Tag, int D, int NW>
 __global__ __launch_bounds__(64 * NW) void linear_bwd_rows_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ gout, const uint16_t* __restrict__ kvt,
     const uint16_t* __restrict__ kvp, const uint16_t* __restrict__ z, const uint16_t* __restrict__ wt,
-    uint16_t* __restrict__ dq, uint16_t* __restrict__ dn_out,
+    uint16_t* __restrict__ dq, const RowLayout lin, const RowLayout ldo, uint16_t* __restrict__ dn_out,
     uint16_t* __restrict__ y_out, float* __restrict__ dden_out, int L, int fmap, int tiles_per_wg, int accumulate) {
   using E = Elem<Tag>;
   constexpr int DC = D / 16;
@@ -58,14 +58,17 @@ __global__ __launch_bounds__(64 * NW) void linear_bwd_rows_kernel(
   }
   __syncthreads();
 
+  // q and dq rows lie lin.sl elements apart, the rows of G ldo.sl; the temporaries dn, y are contiguous
   const size_t head_off = (size_t)bh * L * D;
+  const size_t head_in = lin.head(bh), head_g = ldo.head(bh);
+  const size_t pitch = (size_t)lin.sl, pitch_g = (size_t)ldo.sl;
   uint16_t* stage = sStage[wave];
   constexpr int STEP = 32 * NW;
   const int first_row = blockIdx.x * tiles_per_wg * STEP + wave * 32;
   TileRows<D> qt, gt;                  // q and G rows of the tile about to be processed
   if (first_row < L) {
-    qt.fetch(q + head_off + (size_t)first_row * D, min(32, L - first_row), lane);
-    gt.fetch(gout + head_off + (size_t)first_row * D, min(32, L - first_row), lane);
+    qt.fetch(q + head_in + (size_t)first_row * pitch, min(32, L - first_row), lane, pitch);
+    gt.fetch(gout + head_g + (size_t)first_row * pitch_g, min(32, L - first_row), lane, pitch_g);
   }
   for (int tt = 0; tt < tiles_per_wg; ++tt) {
     const int row0 = first_row + tt * STEP;
@@ -74,6 +77,7 @@ __global__ __launch_bounds__(64 * NW) void linear_bwd_rows_kernel(
     const int qrow = row0 + r;
     const bool ok = qrow < L;
     const size_t toff = head_off + (size_t)row0 * D;
+    const size_t toff_in = head_in + (size_t)row0 * pitch;
 
     // q in B-operand order (d = 16c + 8g + j) and in accumulator order (d = 32t + 8i4 + 4g + j)
     qt.park(stage, lane);
@@ -97,10 +101,10 @@ __global__ __launch_bounds__(64 * NW) void linear_bwd_rows_kernel(
     for (int c = 0; c < DC; ++c) gf[c] = *reinterpret_cast<const i16x8_t*>(&stage[r * STR + 16 * c + 8 * g]);
     wave_lds_fence();
     TileRows<D> dq_old;
-    if (accumulate) dq_old.fetch(dq + toff, rows_valid, lane);
+    if (accumulate) dq_old.fetch(dq + toff_in, rows_valid, lane, pitch);
     if (tt + 1 < tiles_per_wg && row0 + STEP < L) {
-      qt.fetch(q + toff + (size_t)STEP * D, min(32, L - row0 - STEP), lane);
-      gt.fetch(gout + toff + (size_t)STEP * D, min(32, L - row0 - STEP), lane);
+      qt.fetch(q + toff_in + (size_t)STEP * pitch, min(32, L - row0 - STEP), lane, pitch);
+      gt.fetch(gout + head_g + (size_t)(row0 + STEP) * pitch_g, min(32, L - row0 - STEP), lane, pitch_g);
     }
 
     float row_mx, row_inv;
@@ -197,7 +201,7 @@ __global__ __launch_bounds__(64 * NW) void linear_bwd_rows_kernel(
       }
     }
     phi_backward<DT>(fmap, xq, da, row_mx, row_inv);
-    store_acc_tile<E, D>(stage, da, dq + toff, accumulate ? &dq_old : nullptr, rows_valid, lane);
+    store_acc_tile<E, D>(stage, da, dq + toff_in, accumulate ? &dq_old : nullptr, rows_valid, lane, pitch);
   }
 }
 
@@ -206,8 +210,9 @@ __global__ __launch_bounds__(64 * NW) void linear_bwd_rows_kernel(
 template <typename Tag, int D>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void linear_bwd_states_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ dn, const uint16_t* __restrict__ gout,
-    const uint16_t* __restrict__ y, const float* __restrict__ dden, float* __restrict__ ds_part, float* __restrict__ dw_part,
-    float* __restrict__ dz_part, float* __restrict__ db_part, int L, int rows_per_split, int fmap) {
+    const uint16_t* __restrict__ y, const float* __restrict__ dden, const RowLayout lin, const RowLayout ldo,
+    float* __restrict__ ds_part, float* __restrict__ dw_part, float* __restrict__ dz_part, float* __restrict__ db_part, int L,
+    int rows_per_split, int fmap) {
   using E = Elem<Tag>;
   constexpr int TR = 64;
   constexpr int STR = D + 16;
@@ -265,10 +270,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       ry[p] = rq[p];
       rdd[p] = 0.f;
       if (grow < row_end) {
-        const size_t off = head_off + (size_t)grow * D + lcol;
-        rq[p] = *reinterpret_cast<const i16x8_t*>(q + off);
+        const size_t off = head_off + (size_t)grow * D + lcol;          // dn, y: contiguous temporaries
+        rq[p] = *reinterpret_cast<const i16x8_t*>(q + lin.head(bh) + (size_t)grow * (size_t)lin.sl + lcol);
         rdn[p] = *reinterpret_cast<const i16x8_t*>(dn + off);
-        rg[p] = *reinterpret_cast<const i16x8_t*>(gout + off);
+        rg[p] = *reinterpret_cast<const i16x8_t*>(gout + ldo.head(bh) + (size_t)grow * (size_t)ldo.sl + lcol);
         ry[p] = *reinterpret_cast<const i16x8_t*>(y + off);
         rdd[p] = dden[(size_t)bh * L + grow];
       }
@@ -444,12 +449,14 @@ __global__ __launch_bounds__(256) void linear_bwd_reduce_heads_kernel(const floa
 // ---- kv -----------------------------------------------------------------------------------
 // Same tile traffic as the rows kernel: NW waves of 32 keys, whole-row global accesses through a
 // wave-private staging tile.
-template <typename Tag, int D, int NW>
+// CONTIG: k, v, dk, dv are contiguous (B, H, L, D): the row pitch is the compile-time D.
+template <typename Tag, int D, int NW, bool CONTIG>
 __global__ __launch_bounds__(64 * NW) void linear_bwd_kv_kernel(const uint16_t* __restrict__ k, const uint16_t* __restrict__ v,
                                                                 const uint16_t* __restrict__ ds,
                                                                 const uint16_t* __restrict__ dst, const float* __restrict__ dz,
-                                                                uint16_t* __restrict__ dk, uint16_t* __restrict__ dv, int L,
-                                                                int fmap, int tiles_per_wg, int accumulate) {
+                                                                uint16_t* __restrict__ dk, uint16_t* __restrict__ dv,
+                                                                const RowLayout lin, int L, int fmap, int tiles_per_wg,
+                                                                int accumulate) {
   using E = Elem<Tag>;
   constexpr int DC = D / 16;
   constexpr int DT = D / 32;
@@ -472,7 +479,8 @@ __global__ __launch_bounds__(64 * NW) void linear_bwd_kv_kernel(const uint16_t* 
   if (tid < D) sDZ[tid] = dz[(size_t)bh * D + tid];
   __syncthreads();
 
-  const size_t head_off = (size_t)bh * L * D;
+  const size_t head_off = lin.head(bh);   // k, v, dk, dv rows: lin.sl elements apart
+  const size_t pitch = CONTIG ? (size_t)D : (size_t)lin.sl;
   uint16_t* stage = sStage[wave];
   constexpr int STEP = 32 * NW;
   const int first_row = blockIdx.x * tiles_per_wg * STEP + wave * 32;
@@ -480,12 +488,12 @@ __global__ __launch_bounds__(64 * NW) void linear_bwd_kv_kernel(const uint16_t* 
     const int row0 = first_row + tt * STEP;
     if (row0 >= L) break;
     const int rows_valid = min(32, L - row0);
-    const size_t toff = head_off + (size_t)row0 * D;
+    const size_t toff = head_off + (size_t)row0 * pitch;
 
     // two waves share a SIMD and cover each other's load latency; registers are too scarce to fetch ahead
     TileRows<D> kt, vt;
-    kt.fetch(k + toff, rows_valid, lane);
-    vt.fetch(v + toff, rows_valid, lane);
+    kt.fetch(k + toff, rows_valid, lane, pitch);
+    vt.fetch(v + toff, rows_valid, lane, pitch);
     kt.park(stage, lane);
     float f[DC][8];
 #pragma unroll
@@ -533,9 +541,9 @@ __global__ __launch_bounds__(64 * NW) void linear_bwd_kv_kernel(const uint16_t* 
         for (int i = 0; i < 16; ++i) dvv[t][i] = vacc[i];
       }
       if (accumulate)
-        store_acc_tile<E, D, true>(stage, dvv, dv + toff, nullptr, rows_valid, lane);
+        store_acc_tile<E, D, true>(stage, dvv, dv + toff, nullptr, rows_valid, lane, pitch);
       else
-        store_acc_tile<E, D, false>(stage, dvv, dv + toff, nullptr, rows_valid, lane);
+        store_acc_tile<E, D, false>(stage, dvv, dv + toff, nullptr, rows_valid, lane, pitch);
     }
     // dc^T = dS v^T + dz ; dk = phi'(k) dc
     float dc[DT][16], xk[DT][16];
@@ -562,9 +570,9 @@ __global__ __launch_bounds__(64 * NW) void linear_bwd_kv_kernel(const uint16_t* 
     }
     phi_backward<DT>(fmap, xk, dc, row_mx, row_inv);
     if (accumulate)
-      store_acc_tile<E, D, true>(stage, dc, dk + toff, nullptr, rows_valid, lane);
+      store_acc_tile<E, D, true>(stage, dc, dk + toff, nullptr, rows_valid, lane, pitch);
     else
-      store_acc_tile<E, D, false>(stage, dc, dk + toff, nullptr, rows_valid, lane);
+      store_acc_tile<E, D, false>(stage, dc, dk + toff, nullptr, rows_valid, lane, pitch);
   }
 }
 
@@ -599,11 +607,11 @@ int64_t linear_bwd_workspace_bytes(int BH, int L, int D) { return (int64_t)lin_b
 
 template <typename Tag, int D>
 static int linear_bwd_impl(const void* q, const void* k, const void* v, const float* weight, const void* d_out, void* dq,
-                           void* dk, void* dv, float* d_weight, float* d_bias, int fmap, int BH, int L, int flags,
-                           char* ws, hipStream_t st) {
+                           void* dk, void* dv, const RowLayout& lin, const RowLayout& ldo, float* d_weight, float* d_bias,
+                           int fmap, int BH, int L, int flags, char* ws, hipStream_t st) {
   const LinBwdWs w = lin_bwd_ws(BH, L, D);
   const int accumulate = flags & SLA_BWD_ACCUMULATE;
-  if (!(flags & SLA_BWD_STATES_READY)) launch_state_build<Tag, D>(k, v, contiguous_layout(BH, L, D), weight, fmap, BH, L, ws, w.fwd, st);
+  if (!(flags & SLA_BWD_STATES_READY)) launch_state_build<Tag, D>(k, v, lin, weight, fmap, BH, L, ws, w.fwd, st);
   uint16_t* kvt = (uint16_t*)(ws + w.fwd.kvt);
   uint16_t* z = (uint16_t*)(ws + w.fwd.z);
   uint16_t* dn = (uint16_t*)(ws + w.dn);
@@ -613,10 +621,10 @@ static int linear_bwd_impl(const void* q, const void* k, const void* v, const fl
   const int tiles_rows = balanced_tiles(cdiv(L, 32 * NW_ROWS), BH, 1);
   const int tiles_kv = balanced_tiles(cdiv(L, 32 * NW_KV), BH, 1);
   hipLaunchKernelGGL((linear_bwd_rows_kernel<Tag, D, NW_ROWS>), dim3(cdiv(L, 32 * NW_ROWS * tiles_rows), BH), dim3(64 * NW_ROWS), 0, st, (const uint16_t*)q,
-                     (const uint16_t*)d_out, kvt, (const uint16_t*)(ws + w.fwd.kvp), z, (const uint16_t*)(ws + w.fwd.wt), (uint16_t*)dq, dn, y,
+                     (const uint16_t*)d_out, kvt, (const uint16_t*)(ws + w.fwd.kvp), z, (const uint16_t*)(ws + w.fwd.wt), (uint16_t*)dq, lin, ldo, dn, y,
                      dden, L, fmap, tiles_rows, accumulate);
   hipLaunchKernelGGL((linear_bwd_states_kernel<Tag, D>), dim3(w.st.nsplit, BH), dim3(256), 0, st, (const uint16_t*)q, dn,
-                     (const uint16_t*)d_out, y, dden, (float*)(ws + w.ds_part), (float*)(ws + w.dw_part),
+                     (const uint16_t*)d_out, y, dden, lin, ldo, (float*)(ws + w.ds_part), (float*)(ws + w.dw_part),
                      (float*)(ws + w.dz_part), (float*)(ws + w.db_part), L, w.st.rows_per_split, fmap);
   hipLaunchKernelGGL((linear_bwd_reduce_kernel<Tag>), dim3(cdiv(D * D, 256), BH), dim3(256), 0, st,
                      (const float*)(ws + w.ds_part), (const float*)(ws + w.dw_part), (const float*)(ws + w.dz_part),
@@ -624,9 +632,16 @@ static int linear_bwd_impl(const void* q, const void* k, const void* v, const fl
                      (float*)(ws + w.dw_head), (float*)(ws + w.db_head), w.st.nsplit, D);
   hipLaunchKernelGGL(linear_bwd_reduce_heads_kernel, dim3(cdiv(D * D, 256)), dim3(256), 0, st,
                      (const float*)(ws + w.dw_head), (const float*)(ws + w.db_head), d_weight, d_bias, BH, D);
-  hipLaunchKernelGGL((linear_bwd_kv_kernel<Tag, D, NW_KV>), dim3(cdiv(L, 32 * NW_KV * tiles_kv), BH), dim3(64 * NW_KV), 0, st, (const uint16_t*)k, (const uint16_t*)v,
-                     (const uint16_t*)(ws + w.ds), (const uint16_t*)(ws + w.dst), (const float*)(ws + w.dz), (uint16_t*)dk,
-                     (uint16_t*)dv, L, fmap, tiles_kv, accumulate);
+  if (lin.sl == D)
+    hipLaunchKernelGGL((linear_bwd_kv_kernel<Tag, D, NW_KV, true>), dim3(cdiv(L, 32 * NW_KV * tiles_kv), BH), dim3(64 * NW_KV),
+                       0, st, (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)(ws + w.ds),
+                       (const uint16_t*)(ws + w.dst), (const float*)(ws + w.dz), (uint16_t*)dk, (uint16_t*)dv, lin, L, fmap,
+                       tiles_kv, accumulate);
+  else
+    hipLaunchKernelGGL((linear_bwd_kv_kernel<Tag, D, NW_KV, false>), dim3(cdiv(L, 32 * NW_KV * tiles_kv), BH), dim3(64 * NW_KV),
+                       0, st, (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)(ws + w.ds),
+                       (const uint16_t*)(ws + w.dst), (const float*)(ws + w.dz), (uint16_t*)dk, (uint16_t*)dv, lin, L, fmap,
+                       tiles_kv, accumulate);
   return check_launch("linear_bwd");
 }
 
@@ -634,10 +649,10 @@ static int linear_bwd_impl(const void* q, const void* k, const void* v, const fl
 
 using namespace sla;
 
-extern "C" int sla_linear_bwd(const void* q, const void* k, const void* v, const float* weight, const float* bias,
-                              const void* d_out, void* dq, void* dk, void* dv, float* d_weight, float* d_bias, int dtype,
-                              int fmap, int B, int H, int L, int D, int flags, void* workspace,
-                              int64_t workspace_bytes, void* stream) {
+static int linear_bwd_entry(const void* q, const void* k, const void* v, const int64_t* qkv_strides, const float* weight,
+                            const float* bias, const void* d_out, const int64_t* do_strides, void* dq, void* dk, void* dv,
+                            float* d_weight, float* d_bias, int dtype, int fmap, int B, int H, int L, int D, int flags,
+                            void* workspace, int64_t workspace_bytes, void* stream) {
   int rc = validate_linear(dtype, fmap, B, H, L, D);
   if (rc) return rc;
   SLA_REQUIRE((flags & ~(SLA_BWD_ACCUMULATE | SLA_BWD_STATES_READY)) == 0, SLA_ERR_BAD_ARG, "unknown flag bits in %d", flags);
@@ -651,10 +666,15 @@ extern "C" int sla_linear_bwd(const void* q, const void* k, const void* v, const
   const int64_t need = linear_bwd_workspace_bytes(BH, L, D);
   SLA_REQUIRE(workspace_bytes >= need, SLA_ERR_WORKSPACE, "workspace of %lld bytes, need %lld", (long long)workspace_bytes,
               (long long)need);
+  RowLayout lin, ldo;
+  rc = make_layout(qkv_strides, B, H, L, D, 2, &lin);
+  if (rc) return rc;
+  rc = make_layout(do_strides, B, H, L, D, 2, &ldo);
+  if (rc) return rc;
   hipStream_t st = (hipStream_t)stream;
   char* ws = (char*)workspace;
 #define SLA_LINB_CASE(TAG, DD) \
-  return linear_bwd_impl<TAG, DD>(q, k, v, weight, d_out, dq, dk, dv, d_weight, d_bias, fmap, BH, L, flags, ws, st)
+  return linear_bwd_impl<TAG, DD>(q, k, v, weight, d_out, dq, dk, dv, lin, ldo, d_weight, d_bias, fmap, BH, L, flags, ws, st)
   if (dtype == SLA_BF16) {
     if (D == 128) SLA_LINB_CASE(bf16_tag, 128);
     SLA_LINB_CASE(bf16_tag, 64);
@@ -662,4 +682,22 @@ extern "C" int sla_linear_bwd(const void* q, const void* k, const void* v, const
   if (D == 128) SLA_LINB_CASE(f16_tag, 128);
   SLA_LINB_CASE(f16_tag, 64);
 #undef SLA_LINB_CASE
+}
+
+extern "C" int sla_linear_bwd(const void* q, const void* k, const void* v, const float* weight, const float* bias,
+                              const void* d_out, void* dq, void* dk, void* dv, float* d_weight, float* d_bias, int dtype,
+                              int fmap, int B, int H, int L, int D, int flags, void* workspace,
+                              int64_t workspace_bytes, void* stream) {
+  return linear_bwd_entry(q, k, v, nullptr, weight, bias, d_out, nullptr, dq, dk, dv, d_weight, d_bias, dtype, fmap, B, H, L,
+                          D, flags, workspace, workspace_bytes, stream);
+}
+
+extern "C" int sla_linear_bwd_strided(const void* q, const void* k, const void* v, const int64_t* qkv_strides,
+                                      const float* weight, const float* bias, const void* d_out, const int64_t* do_strides,
+                                      void* dq, void* dk, void* dv, float* d_weight, float* d_bias, int dtype, int fmap,
+                                      int B, int H, int L, int D, int flags, void* workspace, int64_t workspace_bytes,
+                                      void* stream) {
+  SLA_REQUIRE(qkv_strides && do_strides, SLA_ERR_BAD_ARG, "null strides");
+  return linear_bwd_entry(q, k, v, qkv_strides, weight, bias, d_out, do_strides, dq, dk, dv, d_weight, d_bias, dtype, fmap, B,
+                          H, L, D, flags, workspace, workspace_bytes, stream);
 }

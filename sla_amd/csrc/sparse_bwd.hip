@@ -28,15 +28,17 @@ int validate_attn_shape(int dtype, int B, int H, int L, int D, int BLKQ, int BLK
 // ---- delta ------------------------------------------------------------------------------
 template <typename Tag, int D>
 __global__ __launch_bounds__(256) void bwd_delta_kernel(const uint16_t* __restrict__ o, const uint16_t* __restrict__ d_o,
-                                                        float* __restrict__ delta, size_t rows) {
+                                                        const RowLayout ldo, float* __restrict__ delta, size_t rows, int L) {
   using E = Elem<Tag>;
   constexpr int CPR = D / 8;
-  const size_t row = (size_t)blockIdx.x * (256 / CPR) + threadIdx.x / CPR;
+  const size_t row = (size_t)blockIdx.x * (256 / CPR) + threadIdx.x / CPR;   // = bh * L + l
   const int col = (threadIdx.x % CPR) * 8;
   float s = 0.f;
   if (row < rows) {
+    const int bh = (int)(row / (size_t)L);
+    const size_t l = row - (size_t)bh * L;
     const i16x8_t a = *reinterpret_cast<const i16x8_t*>(o + row * D + col);
-    const i16x8_t b = *reinterpret_cast<const i16x8_t*>(d_o + row * D + col);
+    const i16x8_t b = *reinterpret_cast<const i16x8_t*>(d_o + ldo.head(bh) + l * (size_t)ldo.sl + col);
 #pragma unroll
     for (int e = 0; e < 8; ++e) s += E::to_float((uint16_t)a[e]) * E::to_float((uint16_t)b[e]);
   }
@@ -113,11 +115,14 @@ __global__ __launch_bounds__(64 * COL_NW) void bwd_col_lists_kernel(const int8_t
 // One workgroup per query block, one wave per 32 queries.  Register use is held to 256 so that two waves
 // share a SIMD.  K and V tiles go global -> registers -> LDS; both tiles of the next step are in flight
 // during the whole current step.
-template <typename Tag, int D, int BLKQ>
+// CONTIG: all tensors are contiguous (B, H, L, D); the row pitch is then the compile-time D and every in-tile
+// offset folds into an instruction immediate (the strided variant pays a few registers for the run-time pitch).
+template <typename Tag, int D, int BLKQ, bool CONTIG>
 __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))) void bwd_dq_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ k, const uint16_t* __restrict__ v,
     const uint16_t* __restrict__ d_o, const float* __restrict__ lse, const float* __restrict__ delta,
-    const void* __restrict__ lut, int lut64, uint16_t* __restrict__ dq, int L, int Mblk, int topk, float qk_scale, int total) {
+    const void* __restrict__ lut, int lut64, uint16_t* __restrict__ dq, const RowLayout lin, const RowLayout ldo, int L,
+    int Mblk, int topk, float qk_scale, int total) {
   using E = Elem<Tag>;
   constexpr int BLKK = 64;
   constexpr int NT = BLKQ * 2;
@@ -139,10 +144,13 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
   const int g = lane >> 5, r = lane & 31;
   const float c_log2e = qk_scale * 1.4426950408889634f;
 
-  const size_t head_off = (size_t)bh * L * D;
-  const uint32_t head_bytes = (uint32_t)L * D * 2;
+  // q, k, v (and dq) rows of this head lie lin.sl elements apart, dO rows ldo.sl (D for contiguous tensors)
+  const size_t head_off = CONTIG ? (size_t)bh * L * D : lin.head(bh);
+  const uint32_t pitch = CONTIG ? D : (uint32_t)lin.sl, pitch_do = CONTIG ? D : (uint32_t)ldo.sl;
+  const uint32_t head_bytes = CONTIG ? (uint32_t)L * D * 2 : lin.head_range_bytes(L, D);
   const __amdgpu_buffer_rsrc_t qh = make_rsrc(q + head_off, head_bytes);
-  const __amdgpu_buffer_rsrc_t doh = make_rsrc(d_o + head_off, head_bytes);
+  const __amdgpu_buffer_rsrc_t doh =
+      make_rsrc(d_o + (CONTIG ? head_off : ldo.head(bh)), CONTIG ? head_bytes : ldo.head_range_bytes(L, D));
   const __amdgpu_buffer_rsrc_t kh = make_rsrc(k + head_off, head_bytes);
   const __amdgpu_buffer_rsrc_t vh = make_rsrc(v + head_off, head_bytes);
   const int qrow = mb * BLKQ + wave * 32 + r;
@@ -151,8 +159,8 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
   i16x8_t qf[DC], dof[DC];
 #pragma unroll
   for (int c = 0; c < DC; ++c) {
-    qf[c] = buf_load_b128(qh, ((uint32_t)qrow * D + 16 * c + 8 * g) * 2);      // rows past L read as zero
-    dof[c] = buf_load_b128(doh, ((uint32_t)qrow * D + 16 * c + 8 * g) * 2);
+    qf[c] = buf_load_b128(qh, ((uint32_t)qrow * pitch + 16 * c + 8 * g) * 2);      // rows past L read as zero
+    dof[c] = buf_load_b128(doh, ((uint32_t)qrow * pitch_do + 16 * c + 8 * g) * 2);
   }
   // rows past L: lse = +inf makes every probability exactly 0 (the reference loads `other=inf`)
   const float lse_q = qok ? lse[(size_t)bh * L + qrow] : INFINITY;
@@ -164,12 +172,17 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
                  : reinterpret_cast<const int*>(lut)[lut_row + i];
   };
   i16x8_t kreg[NLD], vreg[NLD];
+  // chunk i of a thread is row tid / CPR + i * (NT / CPR) of the tile.  With a run-time pitch the per-chunk
+  // offsets are not instruction immediates; they are formed from one per-lane offset at every use (the opaque
+  // copy keeps the compiler from hoisting eight of them out of the loop into registers it does not have).
+  static_assert(NT % CPR == 0, "threads must cover whole rows");
+  const uint32_t lane_off = ((uint32_t)(tid / CPR) * pitch + (tid % CPR) * 8) * 2;
   auto load_tile = [&](int nb) {
+    uint32_t lo = lane_off + (uint32_t)(nb * BLKK) * pitch * 2;
+    if (!CONTIG) asm volatile("" : "+v"(lo));
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
-      const int idx = tid + i * NT;
-      const int row = idx / CPR, col = (idx % CPR) * 8;
-      const uint32_t off = ((uint32_t)(nb * BLKK + row) * D + col) * 2;      // rows past L read as zero
+      const uint32_t off = lo + (uint32_t)(i * (NT / CPR)) * pitch * 2;      // rows past L read as zero
       kreg[i] = buf_load_b128(kh, off);
       vreg[i] = buf_load_b128(vh, off);
     }
@@ -271,7 +284,7 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
     __syncthreads();                       // next tiles visible
   }
   if (qok) {
-    uint16_t* orow = dq + head_off + (size_t)qrow * D;
+    uint16_t* orow = dq + head_off + (size_t)qrow * pitch;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -292,12 +305,12 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
 // products) and hands a copy to its partner through LDS; then each adds all 64 rows into its own half of
 // dV^T += dO^T P and dK^T += Q^T dS.  Splitting the accumulators this way keeps a wave at 256 registers,
 // so two waves share a SIMD.
-template <typename Tag, int D, int BLKQ>
+template <typename Tag, int D, int BLKQ, bool CONTIG>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void bwd_dkdv_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ k, const uint16_t* __restrict__ v,
     const uint16_t* __restrict__ d_o, const float* __restrict__ lse, const float* __restrict__ delta,
-    const int* __restrict__ list, const int* __restrict__ count, uint16_t* __restrict__ dk, uint16_t* __restrict__ dv, int L,
-    int Mblk, int Nblk, float qk_scale, int total) {
+    const int* __restrict__ list, const int* __restrict__ count, uint16_t* __restrict__ dk, uint16_t* __restrict__ dv,
+    const RowLayout lin, const RowLayout ldo, int L, int Mblk, int Nblk, float qk_scale, int total) {
   using E = Elem<Tag>;
   constexpr int TQ = 64;                  // query rows per LDS tile
   constexpr int SUB = BLKQ / TQ;          // tiles per listed query block
@@ -324,10 +337,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int g = lane >> 5, r = lane & 31;
   const float c_log2e = qk_scale * 1.4426950408889634f;
 
-  const size_t head_off = (size_t)bh * L * D;
-  const uint32_t head_bytes = (uint32_t)L * D * 2;
+  const size_t head_off = CONTIG ? (size_t)bh * L * D : lin.head(bh);
+  const uint32_t pitch = CONTIG ? D : (uint32_t)lin.sl, pitch_do = CONTIG ? D : (uint32_t)ldo.sl;
+  const uint32_t head_bytes = CONTIG ? (uint32_t)L * D * 2 : lin.head_range_bytes(L, D);
   const __amdgpu_buffer_rsrc_t qh = make_rsrc(q + head_off, head_bytes);
-  const __amdgpu_buffer_rsrc_t doh = make_rsrc(d_o + head_off, head_bytes);
+  const __amdgpu_buffer_rsrc_t doh =
+      make_rsrc(d_o + (CONTIG ? head_off : ldo.head(bh)), CONTIG ? head_bytes : ldo.head_range_bytes(L, D));
   const __amdgpu_buffer_rsrc_t kb = make_rsrc(k + head_off, head_bytes);
   const __amdgpu_buffer_rsrc_t vb = make_rsrc(v + head_off, head_bytes);
   const float* lseh = lse + (size_t)bh * L;
@@ -339,8 +354,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   i16x8_t kf[DC], vf[DC];
 #pragma unroll
   for (int c = 0; c < DC; ++c) {
-    kf[c] = buf_load_b128(kb, ((uint32_t)krow * D + 16 * c + 8 * g) * 2);     // rows past L read as zero
-    vf[c] = buf_load_b128(vb, ((uint32_t)krow * D + 16 * c + 8 * g) * 2);
+    kf[c] = buf_load_b128(kb, ((uint32_t)krow * pitch + 16 * c + 8 * g) * 2);     // rows past L read as zero
+    vf[c] = buf_load_b128(vb, ((uint32_t)krow * pitch + 16 * c + 8 * g) * 2);
   }
 
   f32x16_t dkacc[DH], dvacc[DH];
@@ -363,9 +378,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     for (int i = 0; i < NLD; ++i) {
       const int idx = tid + i * NT;
       const int row = idx / CPR, col = (idx % CPR) * 8;
-      const uint32_t off = ((uint32_t)(row0 + row) * D + col) * 2;            // rows past L read as zero
-      qreg[i] = buf_load_b128(qh, off);
-      doreg[i] = buf_load_b128(doh, off);
+      // rows past L read as zero
+      qreg[i] = buf_load_b128(qh, ((uint32_t)(row0 + row) * pitch + col) * 2);
+      doreg[i] = buf_load_b128(doh, ((uint32_t)(row0 + row) * pitch_do + col) * 2);
     }
     if (tid < TQ) {
       const int grow = row0 + tid;
@@ -485,8 +500,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     __syncthreads();                       // next tile visible
   }
   if (kok) {
-    uint16_t* dkrow = dk + head_off + (size_t)krow * D;
-    uint16_t* dvrow = dv + head_off + (size_t)krow * D;
+    uint16_t* dkrow = dk + head_off + (size_t)krow * pitch;
+    uint16_t* dvrow = dv + head_off + (size_t)krow * pitch;
 #pragma unroll
     for (int dt = 0; dt < DH; ++dt)
 #pragma unroll
@@ -525,8 +540,9 @@ int64_t sparse_bwd_workspace_bytes(int BH, int L, int D, int BLKQ, int BLKK, int
 
 template <typename Tag, int D, int BLKQ>
 static int bwd_impl(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
-                    const int8_t* sparse_map, const void* lut, int lut64, void* dq, void* dk, void* dv, int BH, int L,
-                    int topk, float qk_scale, char* ws, hipStream_t st) {
+                    const int8_t* sparse_map, const void* lut, int lut64, void* dq, void* dk, void* dv,
+                    const RowLayout& lin, const RowLayout& ldo, int BH, int L, int topk, float qk_scale, char* ws,
+                    hipStream_t st) {
   const BwdWs w = bwd_ws(BH, L, BLKQ, 64);
   const int Mblk = cdiv(L, BLKQ), Nblk = cdiv(L, 64);
   float* delta = (float*)(ws + w.delta);
@@ -535,19 +551,27 @@ static int bwd_impl(const void* q, const void* k, const void* v, const void* o, 
   const size_t rows = (size_t)BH * L;
   constexpr int RPB = 256 / (D / 8);
   hipLaunchKernelGGL((bwd_delta_kernel<Tag, D>), dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, st,
-                     (const uint16_t*)o, (const uint16_t*)d_o, delta, rows);
+                     (const uint16_t*)o, (const uint16_t*)d_o, ldo, delta, rows, L);
   // 16-byte loads of map rows need 16-byte aligned rows
   const int vec_ok = (Nblk % 16 == 0) && ((uintptr_t)sparse_map % 16 == 0);
   hipLaunchKernelGGL(bwd_col_lists_kernel, dim3(cdiv(Nblk, 64), BH), dim3(64 * COL_NW), 0, st, sparse_map, list, count, Mblk, Nblk,
                      vec_ok);
   const int total_q = BH * Mblk;
-  hipLaunchKernelGGL((bwd_dq_kernel<Tag, D, BLKQ>), dim3(xcd_grid(total_q)), dim3(BLKQ * 2), 0, st, (const uint16_t*)q,
-                     (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse, delta, lut, lut64, (uint16_t*)dq, L,
-                     Mblk, topk, qk_scale, total_q);
   const int total_k = BH * Nblk;
-  hipLaunchKernelGGL((bwd_dkdv_kernel<Tag, D, BLKQ>), dim3(xcd_grid(total_k)), dim3(256), 0, st, (const uint16_t*)q,
-                     (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse, delta, list, count, (uint16_t*)dk,
-                     (uint16_t*)dv, L, Mblk, Nblk, qk_scale, total_k);
+  const bool contig = lin.sl == D && ldo.sl == D;
+#define SLA_BWD_LAUNCH(CONTIG)                                                                                              \
+  hipLaunchKernelGGL((bwd_dq_kernel<Tag, D, BLKQ, CONTIG>), dim3(xcd_grid(total_q)), dim3(BLKQ * 2), 0, st,                 \
+                     (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse, delta, lut,     \
+                     lut64, (uint16_t*)dq, lin, ldo, L, Mblk, topk, qk_scale, total_q);                                    \
+  hipLaunchKernelGGL((bwd_dkdv_kernel<Tag, D, BLKQ, CONTIG>), dim3(xcd_grid(total_k)), dim3(256), 0, st, (const uint16_t*)q, \
+                     (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse, delta, list, count, (uint16_t*)dk,  \
+                     (uint16_t*)dv, lin, ldo, L, Mblk, Nblk, qk_scale, total_k);
+  if (contig) {
+    SLA_BWD_LAUNCH(true)
+  } else {
+    SLA_BWD_LAUNCH(false)
+  }
+#undef SLA_BWD_LAUNCH
   return check_launch("sparse_attn_bwd");
 }
 
@@ -555,10 +579,11 @@ static int bwd_impl(const void* q, const void* k, const void* v, const void* o, 
 
 using namespace sla;
 
-extern "C" int sla_sparse_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o,
-                                   const float* lse, const int8_t* sparse_map, const void* lut, int lut_elem_bytes,
-                                   void* dq, void* dk, void* dv, int dtype, int B, int H, int L, int D, int BLKQ, int BLKK,
-                                   int topk, float qk_scale, void* workspace, int64_t workspace_bytes, void* stream) {
+static int attn_bwd_entry(const void* q, const void* k, const void* v, const int64_t* qkv_strides, const void* o,
+                          const void* d_o, const int64_t* do_strides, const float* lse, const int8_t* sparse_map,
+                          const void* lut, int lut_elem_bytes, void* dq, void* dk, void* dv, int dtype, int B, int H, int L,
+                          int D, int BLKQ, int BLKK, int topk, float qk_scale, void* workspace, int64_t workspace_bytes,
+                          void* stream) {
   int rc = validate_attn_shape(dtype, B, H, L, D, BLKQ, BLKK, topk, lut_elem_bytes);
   if (rc) return rc;
   SLA_REQUIRE(q && k && v && o && d_o && lse && sparse_map && dq && dk && dv && workspace && (lut || topk == 0),
@@ -572,12 +597,18 @@ extern "C" int sla_sparse_attn_bwd(const void* q, const void* k, const void* v, 
   SLA_REQUIRE(workspace_bytes >= need, SLA_ERR_WORKSPACE, "workspace of %lld bytes, need %lld", (long long)workspace_bytes,
               (long long)need);
   SLA_REQUIRE((int64_t)BH * cdiv(L, 64) * cdiv(L, BLKQ) < (1ll << 40), SLA_ERR_UNSUPPORTED, "block map too large");
+  RowLayout lin, ldo;
+  rc = make_layout(qkv_strides, B, H, L, D, 2, &lin);
+  if (rc) return rc;
+  rc = make_layout(do_strides, B, H, L, D, 2, &ldo);
+  if (rc) return rc;
   hipStream_t st = (hipStream_t)stream;
   char* ws = (char*)workspace;
   const int lut64 = lut_elem_bytes == 8;
-#define SLA_BWD_CASE(TAG, DD, BQ) \
-  if (D == DD && BLKQ == BQ)      \
-  return bwd_impl<TAG, DD, BQ>(q, k, v, o, d_o, lse, sparse_map, lut, lut64, dq, dk, dv, BH, L, topk, qk_scale, ws, st)
+#define SLA_BWD_CASE(TAG, DD, BQ)                                                                                          \
+  if (D == DD && BLKQ == BQ)                                                                                               \
+  return bwd_impl<TAG, DD, BQ>(q, k, v, o, d_o, lse, sparse_map, lut, lut64, dq, dk, dv, lin, ldo, BH, L, topk, qk_scale, \
+                               ws, st)
   if (dtype == SLA_BF16) {
     SLA_BWD_CASE(bf16_tag, 128, 64);
     SLA_BWD_CASE(bf16_tag, 128, 128);
@@ -592,4 +623,22 @@ extern "C" int sla_sparse_attn_bwd(const void* q, const void* k, const void* v, 
 #undef SLA_BWD_CASE
   set_error("unsupported D=%d BLKQ=%d", D, BLKQ);
   return SLA_ERR_UNSUPPORTED;
+}
+
+extern "C" int sla_sparse_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o,
+                                   const float* lse, const int8_t* sparse_map, const void* lut, int lut_elem_bytes,
+                                   void* dq, void* dk, void* dv, int dtype, int B, int H, int L, int D, int BLKQ, int BLKK,
+                                   int topk, float qk_scale, void* workspace, int64_t workspace_bytes, void* stream) {
+  return attn_bwd_entry(q, k, v, nullptr, o, d_o, nullptr, lse, sparse_map, lut, lut_elem_bytes, dq, dk, dv, dtype, B, H, L,
+                        D, BLKQ, BLKK, topk, qk_scale, workspace, workspace_bytes, stream);
+}
+
+extern "C" int sla_sparse_attn_bwd_strided(const void* q, const void* k, const void* v, const int64_t* qkv_strides,
+                                           const void* o, const void* d_o, const int64_t* do_strides, const float* lse,
+                                           const int8_t* sparse_map, const void* lut, int lut_elem_bytes, void* dq, void* dk,
+                                           void* dv, int dtype, int B, int H, int L, int D, int BLKQ, int BLKK, int topk,
+                                           float qk_scale, void* workspace, int64_t workspace_bytes, void* stream) {
+  SLA_REQUIRE(qkv_strides && do_strides, SLA_ERR_BAD_ARG, "null strides");
+  return attn_bwd_entry(q, k, v, qkv_strides, o, d_o, do_strides, lse, sparse_map, lut, lut_elem_bytes, dq, dk, dv, dtype, B,
+                        H, L, D, BLKQ, BLKK, topk, qk_scale, workspace, workspace_bytes, stream);
 }

@@ -4,10 +4,10 @@ The reference README (``README.md:2``, usage at ``README.md:30-50``) motivates S
 attention call inside a video-diffusion transformer block that is then fine-tuned; its benchmark moves between
 the ``(B, L, H, D)`` layout of such blocks and the operator's ``(B, H, L, D)`` (``evaluate/bench_kernel.py:68-71``).
 This module is that caller: QKV projection -> head split -> SLA -> head merge -> output projection.  The two
-projections are plain library GEMMs.  The head split and merge cost nothing at inference: q, k, v are handed
-over as ``(B, H, L, D)`` views of the packed ``(B, L, 3, H, D)`` projection, the kernels read the rows where
-they lie and write the output in ``(B, L, H, D)`` order, which the output projection takes as it is.  For
-training the operator makes the contiguous ``(B, H, L, D)`` copies its backward kernels need.
+projections are plain library GEMMs.  The head split and merge cost nothing, in training as at inference: the
+packed ``(B, L, 3, H, D)`` projection goes to ``SparseLinearAttention.forward_packed``, whose kernels read the
+q, k, v rows where they lie, write the output in ``(B, L, H, D)`` order, which the output projection takes as
+it is, and whose backward kernels write dq, dk, dv straight into one packed gradient tensor.
 """
 from __future__ import annotations
 
@@ -33,7 +33,5 @@ class SLASelfAttention(nn.Module):
         """x: (B, L, dim) -> (B, L, dim)."""
         B, L, C = x.shape
         H, D = self.num_heads, self.head_dim
-        qkv = self.qkv(x).view(B, L, 3, H, D)
-        q, k, v = (qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))      # (B, H, L, D) views, rows 3*H*D apart
-        o = self.attn(q, k, v)                                  # (B, H, L, D); at inference a view of (B, L, H, D)
-        return self.proj(o.transpose(1, 2).reshape(B, L, C))
+        o = self.attn.forward_packed(self.qkv(x).view(B, L, 3, H, D))      # (B, L, H, D)
+        return self.proj(o.reshape(B, L, C))

@@ -104,10 +104,19 @@ def linear_bwd(q, k, v, weight, bias, d_out, fmap: str, accumulate_into=None, st
         dq, dk, dv = accumulate_into
     dw = torch.empty((D, D), dtype=torch.float32, device=q.device)
     db = torch.empty((D,), dtype=torch.float32, device=q.device)
-    rc = _lib.load().sla_linear_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), weight.data_ptr(), bias.data_ptr(),
-                                    d_out.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), dw.data_ptr(),
-                                    db.data_ptr(), dt, _lib.FMAP[fmap], B, H, L, D, flags, ws.data_ptr(), ws.numel(),
-                                    _lib.stream_ptr(q.device))
+    if all(t.is_contiguous() for t in (q, k, v, d_out, dq, dk, dv)):
+        rc = _lib.load().sla_linear_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), weight.data_ptr(), bias.data_ptr(),
+                                        d_out.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), dw.data_ptr(),
+                                        db.data_ptr(), dt, _lib.FMAP[fmap], B, H, L, D, flags, ws.data_ptr(), ws.numel(),
+                                        _lib.stream_ptr(q.device))
+    else:
+        # row-contiguous views: q, k, v and the gradient tensors share their strides, d_out has its own
+        assert _lib.row_strided(q, k, v, dq, dk, dv) and _lib.row_strided(d_out), "tensors must be row-contiguous views"
+        rc = _lib.load().sla_linear_bwd_strided(q.data_ptr(), k.data_ptr(), v.data_ptr(), _lib.strides_arg(q),
+                                                weight.data_ptr(), bias.data_ptr(), d_out.data_ptr(),
+                                                _lib.strides_arg(d_out), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
+                                                dw.data_ptr(), db.data_ptr(), dt, _lib.FMAP[fmap], B, H, L, D, flags,
+                                                ws.data_ptr(), ws.numel(), _lib.stream_ptr(q.device))
     _lib.check(rc)
     return dq, dk, dv, dw, db
 

@@ -51,6 +51,48 @@ class _sla_core(torch.autograd.Function):
         return dq, dk, dv, dw, db, None, None, None, None, None, None, None, None
 
 
+class _sla_packed(torch.autograd.Function):
+    """The same operator on a packed ``(B, L, 3, H, D)`` projection output, returning ``(B, L, H, D)``.
+
+    A transformer block produces q, k, v as one packed tensor in token-major order and consumes the attention
+    output in token-major order.  Fed to ``_sla_core`` through views, autograd would rebuild the packed gradient
+    with three zero-fill-and-copy passes; here the kernels read q, k, v where they lie (row stride ``3*H*D``) and
+    the backward kernels write dq, dk, dv straight into one packed gradient tensor, so neither direction copies.
+    """
+
+    @staticmethod
+    def forward(ctx, qkv, weight, bias, topk_ratio, BLKQ, BLKK, fmap):
+        assert qkv.dim() == 5 and qkv.shape[2] == 3 and qkv.is_contiguous()
+        q, k, v = (qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))          # (B, H, L, D) views
+        weight = weight.contiguous()
+        bias = bias.contiguous()
+        state_ws = _StateBuild(k, v, weight, fmap)
+        sparse_map, lut, topk = get_block_map(q, k, topk_ratio=topk_ratio, BLKQ=BLKQ, BLKK=BLKK)
+        needs_grad = any(ctx.needs_input_grad[:3])
+        qk_scale = q.shape[-1] ** -0.5
+        out, o_s, lse = sparse_attn_linear_fwd(q, k, v, lut, topk, BLKQ, BLKK, qk_scale, state_ws.join(), bias, fmap,
+                                               want_o_s=needs_grad)
+        if needs_grad:
+            ctx.save_for_backward(qkv, weight, bias, sparse_map, lut, lse, o_s, saved_states(state_ws.ws, q))
+            ctx.cfg = (topk, BLKQ, BLKK, fmap, qk_scale)
+        ctx.density = topk / sparse_map.shape[-1]
+        return out.permute(0, 2, 1, 3)                                            # (B, L, H, D), contiguous
+
+    @staticmethod
+    def backward(ctx, d_out):
+        qkv, weight, bias, sparse_map, lut, lse, o_s, states = ctx.saved_tensors
+        topk, BLKQ, BLKK, fmap, qk_scale = ctx.cfg
+        q, k, v = (qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+        d_out = d_out.permute(0, 2, 1, 3)                                         # (B, H, L, D) view
+        if not _lib.row_strided(d_out):
+            d_out = d_out.contiguous()
+        d_qkv = torch.empty_like(qkv)
+        grads = tuple(d_qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+        sparse_attn_bwd(q, k, v, o_s, d_out, lse, sparse_map, lut, topk, BLKQ, BLKK, qk_scale, grads=grads)
+        _, _, _, dw, db = linear_bwd(q, k, v, weight, bias, d_out, fmap, accumulate_into=grads, states=states)
+        return d_qkv, dw, db, None, None, None, None
+
+
 class _StateBuild:
     """The k/v-only half of the linear branch, started on a side stream so that it runs beside the mask
     builder (both are short memory-bound kernels; neither fills the device on its own).  ``join`` makes
@@ -159,6 +201,29 @@ class SparseLinearAttention(nn.Module):
 
         if return_sparsity:
             return o, real_topk / sparse_map.shape[-1]
+        return o
+
+    def forward_packed(self, qkv, return_sparsity=False):
+        r"""
+        The forward on a packed projection output, without layout copies in either direction (extension; the
+        reference takes separate ``(B, H, L, D)`` tensors).
+
+        Args:
+            qkv: (B, L, 3, H, D), as ``nn.Linear(dim, 3 * dim)(x).view(B, L, 3, H, D)`` gives it.
+        Returns:
+            (B, L, H, D), ready for ``reshape(B, L, H * D)``.
+        """
+        if qkv.dtype != self.dtype or self.linear_mode != "global" or not _lib.row_strided(qkv[:, :, 0].permute(0, 2, 1, 3)):
+            q, k, v = (qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+            res = self.forward(q, k, v, return_sparsity)
+            o = res[0] if return_sparsity else res
+            o = o.permute(0, 2, 1, 3)
+            return (o, res[1]) if return_sparsity else o
+        o = _sla_packed.apply(qkv.contiguous(), self.proj_l.weight, self.proj_l.bias, self.topk, self.BLKQ, self.BLKK,
+                              self.feature_map)
+        if return_sparsity:
+            N = (qkv.shape[1] + self.BLKK - 1) // self.BLKK
+            return o, min(N, int(self.topk * N)) / N
         return o
 
     def _forward_complement(self, q, k, qc, kc, vc, dtype, return_sparsity):

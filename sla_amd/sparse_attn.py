@@ -63,19 +63,30 @@ def sparse_attn_linear_fwd(q, k, v, lut, topk, BLOCK_M, BLOCK_N, qk_scale, state
     return out, o_s, lse
 
 
-def sparse_attn_bwd(q, k, v, o, do, lse, k_block_id, lut, topk, BLOCK_M, BLOCK_N, qk_scale):
-    """Launches delta + dQ + dK/dV; returns ``(dq, dk, dv)``."""
+def sparse_attn_bwd(q, k, v, o, do, lse, k_block_id, lut, topk, BLOCK_M, BLOCK_N, qk_scale, grads=None):
+    """Launches delta + dQ + dK/dV; returns ``(dq, dk, dv)``.
+
+    ``grads=(dq, dk, dv)``: write into these tensors instead of new ones.  q, k, v (and the gradient tensors)
+    may be row-contiguous views sharing their strides, ``do`` a row-contiguous view of its own; ``o`` (the saved
+    attention output) and ``lse`` are contiguous."""
     B, H, L, D = q.shape
-    dq = torch.empty_like(q)
-    dk = torch.empty_like(k)
-    dv = torch.empty_like(v)
+    dq, dk, dv = (torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)) if grads is None else grads
     dt = _lib.dtype_code(q.dtype)
     ws = _lib.workspace(_lib.WS_SPARSE_BWD, dt, B, H, L, D, BLOCK_M, BLOCK_N, topk, q.device)
-    rc = _lib.load().sla_sparse_attn_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), do.data_ptr(),
-                                         lse.data_ptr(), k_block_id.data_ptr(), lut.data_ptr(), _lut_bytes(lut),
-                                         dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), dt, B, H, L, D, BLOCK_M,
-                                         BLOCK_N, topk, float(qk_scale), ws.data_ptr(), ws.numel(),
-                                         _lib.stream_ptr(q.device))
+    assert o.is_contiguous() and lse.is_contiguous()
+    if all(t.is_contiguous() for t in (q, k, v, do, dq, dk, dv)):
+        rc = _lib.load().sla_sparse_attn_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), do.data_ptr(),
+                                             lse.data_ptr(), k_block_id.data_ptr(), lut.data_ptr(), _lut_bytes(lut),
+                                             dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), dt, B, H, L, D, BLOCK_M,
+                                             BLOCK_N, topk, float(qk_scale), ws.data_ptr(), ws.numel(),
+                                             _lib.stream_ptr(q.device))
+    else:
+        assert _lib.row_strided(q, k, v, dq, dk, dv) and _lib.row_strided(do), "tensors must be row-contiguous views"
+        rc = _lib.load().sla_sparse_attn_bwd_strided(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), _lib.strides_arg(q), o.data_ptr(), do.data_ptr(),
+            _lib.strides_arg(do), lse.data_ptr(), k_block_id.data_ptr(), lut.data_ptr(), _lut_bytes(lut), dq.data_ptr(),
+            dk.data_ptr(), dv.data_ptr(), dt, B, H, L, D, BLOCK_M, BLOCK_N, topk, float(qk_scale), ws.data_ptr(),
+            ws.numel(), _lib.stream_ptr(q.device))
     _lib.check(rc)
     return dq, dk, dv
 

@@ -74,3 +74,36 @@ def test_block_inference_equals_block_with_copies(dev):
         o = blk.attn(qkv[0], qkv[1], qkv[2])
         y_ref = blk.proj(o.transpose(1, 2).reshape(2, 640, 256))
     assert torch.equal(y, y_ref)
+
+
+@pytest.mark.parametrize("B,H,L,D,BLKQ,fmap,dtype", [(2, 2, 700, 128, 64, "elu", torch.bfloat16),
+                                                     (1, 3, 333, 64, 128, "softmax", torch.float16)])
+def test_packed_training_equals_the_contiguous_route(dev, B, H, L, D, BLKQ, fmap, dtype):
+    """forward_packed: output and all gradients (the packed one included) bit for bit what the module gives on
+    contiguous (B, H, L, D) copies."""
+    g = torch.Generator().manual_seed(L + 1)
+    qkv = torch.randn(B, L, 3, H, D, generator=g).to(dtype).to(dev)
+    do = torch.randn(B, L, H, D, generator=g).to(dtype).to(dev)
+    mod = SparseLinearAttention(D, 0.3, fmap, BLKQ, 64, use_bf16=dtype == torch.bfloat16).to(dev)
+    w, b = make_proj(D)
+    with torch.no_grad():
+        mod.proj_l.weight.copy_(w)
+        mod.proj_l.bias.copy_(b)
+    # contiguous route
+    q, k, v = (qkv[:, :, i].permute(0, 2, 1, 3).contiguous().requires_grad_(True) for i in range(3))
+    out_ref = mod(q, k, v)
+    out_ref.backward(do.permute(0, 2, 1, 3).contiguous())
+    gw, gb = mod.proj_l.weight.grad.clone(), mod.proj_l.bias.grad.clone()
+    mod.zero_grad()
+    # packed route
+    qkv_g = qkv.clone().requires_grad_(True)
+    out, dens = mod.forward_packed(qkv_g, return_sparsity=True)
+    assert out.shape == (B, L, H, D) and out.is_contiguous() and 0 < dens <= 1
+    assert torch.equal(out.detach().permute(0, 2, 1, 3), out_ref.detach())
+    out.backward(do)
+    for i, t in enumerate((q, k, v)):
+        assert torch.equal(qkv_g.grad[:, :, i].permute(0, 2, 1, 3), t.grad), "qkv"[i]
+    assert torch.equal(mod.proj_l.weight.grad, gw) and torch.equal(mod.proj_l.bias.grad, gb)
+    # inference through the same entry
+    with torch.no_grad():
+        assert torch.equal(mod.forward_packed(qkv), out.detach())
