@@ -373,14 +373,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   i16x8_t qreg[NLD], doreg[NLD];
   float lreg = 0.f, dreg = 0.f;
   auto tile_row0 = [&](int ti) -> int { return mylist[ti / SUB] * BLKQ + (ti % SUB) * TQ; };
+  // (per-chunk offsets formed at every use from one per-lane offset, as in the dQ kernel)
+  static_assert(NT % CPR == 0, "threads must cover whole rows");
+  const uint32_t lane_off = ((uint32_t)(tid / CPR) * pitch + (tid % CPR) * 8) * 2;
+  const uint32_t lane_off_do = ((uint32_t)(tid / CPR) * pitch_do + (tid % CPR) * 8) * 2;
   auto load_tile = [&](int row0) {
+    uint32_t lo = lane_off + (uint32_t)row0 * pitch * 2, lo_do = lane_off_do + (uint32_t)row0 * pitch_do * 2;
+    asm volatile("" : "+v"(lo), "+v"(lo_do));
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
-      const int idx = tid + i * NT;
-      const int row = idx / CPR, col = (idx % CPR) * 8;
       // rows past L read as zero
-      qreg[i] = buf_load_b128(qh, ((uint32_t)(row0 + row) * pitch + col) * 2);
-      doreg[i] = buf_load_b128(doh, ((uint32_t)(row0 + row) * pitch_do + col) * 2);
+      qreg[i] = buf_load_b128(qh, lo + (uint32_t)(i * (NT / CPR)) * pitch * 2);
+      doreg[i] = buf_load_b128(doh, lo_do + (uint32_t)(i * (NT / CPR)) * pitch_do * 2);
     }
     if (tid < TQ) {
       const int grow = row0 + tid;

@@ -86,13 +86,18 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
   // One set of staging registers carries K of the next tile during the QK^T phase and V of the
   // next tile during the PV phase (each LDS buffer is free while the other one is being read).
   i16x8_t stg[NLD];
+  // chunk i of a thread is row tid / CPR + i * (NT / CPR) of the tile; the per-chunk offsets are formed from one
+  // per-lane offset at every use (the opaque copy keeps the compiler from hoisting one register per chunk out
+  // of the loop)
+  static_assert(NT % CPR == 0, "threads must cover whole rows");
+  const uint32_t lane_off = ((uint32_t)(tid / CPR) * pitch + (tid % CPR) * 8) * 2;
   auto load_rows_to = [&](i16x8_t (&dst)[NLD], const __amdgpu_buffer_rsrc_t& base, int nb) {
+    uint32_t lo = lane_off + (uint32_t)(nb * BLKK) * pitch * 2;
+    asm volatile("" : "+v"(lo));
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
-      const int idx = tid + i * NT;
-      const int row = idx / CPR, col = (idx % CPR) * 8;
       // rows past L lie beyond the buffer range and read as zero (0 * garbage could be NaN)
-      dst[i] = buf_load_b128(base, ((uint32_t)(nb * BLKK + row) * pitch + col) * 2);
+      dst[i] = buf_load_b128(base, lo + (uint32_t)(i * (NT / CPR)) * pitch * 2);
     }
   };
   auto store_rows_from = [&](const i16x8_t (&src)[NLD], uint16_t* dst, int stride) {
