@@ -53,3 +53,138 @@ def test_rows_are_convex_combinations(dev, full):
     ones = torch.ones_like(v)
     o, _ = sparse_attn_fwd(q, k, ones, lut, T, cfg.BLKQ, cfg.BLKK, cfg.D ** -0.5)
     assert float((o.float() - 1).abs().max()) <= 2 ** -7
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# The largest configuration (cfg4: B1 H40 L75600 D128, relu, forward + backward).  The inputs are generated on
+# the device (the CPU generator needs minutes at this size); the oracle checks the LAST head, copied to the host,
+# whose offsets are the largest the kernels form.
+# ---------------------------------------------------------------------------------------------------------------
+def _device_inputs(cfg, dev, seed, with_do):
+    import math
+    g = torch.Generator(device=dev).manual_seed(seed)
+    Fg, Y, X = cfg.grid
+    f = torch.arange(Fg, device=dev, dtype=torch.float32).view(Fg, 1, 1) / Fg
+    y = torch.arange(Y, device=dev, dtype=torch.float32).view(1, Y, 1) / Y
+    x = torch.arange(X, device=dev, dtype=torch.float32).view(1, 1, X) / X
+    freqs = ((1, 0, 0), (0, 1, 0), (0, 0, 1), (1, 1, 0), (0, 1, 1), (2, 0, 1))
+    shape = (cfg.B, cfg.H, cfg.L, cfg.D)
+    q = torch.empty(shape, device=dev, dtype=cfg.dtype)
+    k = torch.empty(shape, device=dev, dtype=cfg.dtype)
+    for b in range(cfg.B):
+        for h in range(cfg.H):
+            fld = torch.zeros(cfg.L, cfg.D, device=dev)
+            for af, ay, ax in freqs:
+                arg = (2 * math.pi) * (af * f + ay * y + ax * x).reshape(cfg.L, 1)
+                fld += torch.sin(arg + torch.rand(1, cfg.D, device=dev, generator=g) * (2 * math.pi)) / math.sqrt(3.0)
+            q[b, h] = 0.5 * torch.randn(cfg.L, cfg.D, device=dev, generator=g) + fld
+            k[b, h] = 0.5 * torch.randn(cfg.L, cfg.D, device=dev, generator=g) + fld
+            if cfg.k_bias_std > 0:
+                k[b, h] += cfg.k_bias_std * torch.randn(1, cfg.D, device=dev, generator=g)
+    v = torch.randn(shape, device=dev, generator=g).to(cfg.dtype)
+    do = torch.randn(shape, device=dev, generator=g).to(cfg.dtype) if with_do else None
+    return q, k, v, do
+
+
+def _check_map(m, lut, T, N):
+    assert lut.shape[-1] == T and m.shape[-1] == N
+    assert int(m.sum(-1).min()) == T and int(m.sum(-1).max()) == T
+    assert bool((lut[..., 1:] > lut[..., :-1]).all())                      # ascending, hence unique
+    assert int(lut.min()) >= 0 and int(lut.max()) < N
+    assert bool(torch.gather(m, -1, lut.long()).all())
+
+
+def test_largest_configuration_forward_backward(dev):
+    from conftest import cos_sim, max_abs
+    from oracle import sla_oracle as O
+    from sla_amd import _attention
+
+    cfg = CONFIGS["cfg4"]
+    q, k, v, do = _device_inputs(cfg, dev, 4, True)
+    m, lut, T = get_block_map(q, k, cfg.topk, cfg.BLKQ, cfg.BLKK)
+    assert T == 59
+    _check_map(m, lut, T, 1182)
+
+    # block-sparse attention, all 40 heads
+    qd, kd, vd = (t.clone().requires_grad_(True) for t in (q, k, v))
+    o = _attention.apply(qd, kd, vd, m, lut, T, cfg.BLKQ, cfg.BLKK)
+    o.backward(do)
+    dq, dk, dv = qd.grad, kd.grad, vd.grad
+    for t in (o, dq, dk, dv):
+        assert bool(torch.isfinite(t.float()).all())
+    # rows of P sum to one: sum over keys of dV == sum over queries of dO, per head and channel
+    assert max_abs(dv.double().sum(-2), do.double().sum(-2)) <= 1.0
+    # q.k is invariant under (q a, k / a): sum q.dq == sum k.dk, per head
+    ta, tb = (q.double() * dq.double()).sum((-1, -2)), (k.double() * dk.double()).sum((-1, -2))
+    scale = (q.double() * dq.double()).abs().sum((-1, -2)) + (k.double() * dk.double()).abs().sum((-1, -2))
+    assert bool(((ta - tb).abs() <= 1e-3 * scale).all())
+
+    # the last head against the oracle (mask builder, forward, backward)
+    h = cfg.H - 1
+    qc, kc, vc, doc = (t[:, h:h + 1].cpu() for t in (q, k, v, do))
+    m_ref, lut_ref, T_ref = O.get_block_map(qc, kc, cfg.topk, cfg.BLKQ, cfg.BLKK)
+    assert T_ref == T and torch.equal(m_ref, m[:, h:h + 1].cpu())
+    assert torch.equal(lut_ref.long(), lut[:, h:h + 1].cpu().long())
+    o_ref, lse_ref = O.sparse_attn_fwd_gather(qc, kc, vc, lut_ref, cfg.BLKQ, cfg.BLKK)
+    refs = O.sparse_attn_bwd_gather(qc, kc, vc, o_ref, doc, lse_ref, lut_ref, cfg.BLKQ, cfg.BLKK)
+    got = (o.detach(), dq, dk, dv)
+    for name, a, r in zip(("o", "dq", "dk", "dv"), got, (o_ref,) + tuple(refs)):
+        a = a[:, h:h + 1].cpu()
+        assert max_abs(a, r) <= 2e-2, (name, max_abs(a, r))
+        assert cos_sim(a, r) >= 0.999, (name, cos_sim(a, r))
+    del qd, kd, vd, o, dq, dk, dv
+
+    # the whole module (relu feature map, seeded projection): forward + backward run at this size, the linear
+    # branch of the last head agrees with the oracle, and the module output is attention + linear branch
+    w, b = make_proj(cfg.D)
+    mod = SparseLinearAttention(cfg.D, cfg.topk, cfg.feature_map, cfg.BLKQ, cfg.BLKK).to(dev)
+    with torch.no_grad():
+        mod.proj_l.weight.copy_(w)
+        mod.proj_l.bias.copy_(b)
+    qd, kd, vd = (t.clone().requires_grad_(True) for t in (q, k, v))
+    out = mod(qd, kd, vd)
+    out.backward(do)
+    for t in (out, qd.grad, kd.grad, vd.grad, mod.proj_l.weight.grad, mod.proj_l.bias.grad):
+        assert bool(torch.isfinite(t.float()).all())
+    lin_ref = O.linear_branch(qc, kc, vc, w, b, cfg.feature_map, torch.float32)
+    a = out.detach()[:, h:h + 1].cpu()
+    assert max_abs(a, o_ref + lin_ref) <= 2e-2 and cos_sim(a, o_ref + lin_ref) >= 0.999
+    # module gradient = attention gradient (above) + gradient of the linear branch (fp64 autograd of the oracle)
+    qr, kr, vr = (t.double().requires_grad_(True) for t in (qc, kc, vc))
+    O.linear_branch(qr, kr, vr, w.double(), b.double(), cfg.feature_map, torch.float64).backward(doc.double())
+    for name, a, r_lin, r_sp in zip(("dq", "dk", "dv"), (qd.grad, kd.grad, vd.grad), (qr.grad, kr.grad, vr.grad), refs):
+        a = a[:, h:h + 1].cpu()
+        r = r_lin + r_sp.double()
+        assert max_abs(a, r) <= 2e-2, (name, max_abs(a, r))
+        assert cos_sim(a, r) >= 0.999, (name, cos_sim(a, r))
+
+
+def test_largest_quantised_configuration(dev):
+    """cfg5 in full (B1 H40 L32760 D128, 128/64 blocks, topk 0.1, biased k): finite everywhere, the map is
+    well-formed, v = 1 gives 1 (normalisation of the fp8 P V product with its per-channel scale), and the last
+    head agrees with the fp32 mathematics of the same mask to the cosine bound."""
+    from conftest import cos_sim
+    from oracle import sla_oracle as O
+    from sla_amd import SageSparseLinearAttention
+    from sla_amd.sage import sage_attn_fwd, sage_prepare
+
+    cfg = CONFIGS["cfg5"]
+    q, k, v, _ = _device_inputs(cfg, dev, 5, False)
+    m, lut, T = get_block_map(q, k, cfg.topk, cfg.BLKQ, cfg.BLKK)
+    assert T == 51
+    _check_map(m, lut, T, 512)
+    mod = SageSparseLinearAttention(cfg.D, cfg.topk, cfg.feature_map).to(dev)
+    w, b = make_proj(cfg.D)
+    with torch.no_grad():
+        mod.proj_l.weight.copy_(w)
+        mod.proj_l.bias.copy_(b)
+        out = mod(q, k, v)
+        m2, lut2, T2, q8, qs, k8, ks, v8, vs = sage_prepare(q, k, torch.ones_like(v), cfg.topk)
+        assert T2 == T and torch.equal(lut2, lut) and torch.equal(m2, m)
+        ones = sage_attn_fwd(q8, qs, k8, ks, v8, vs, lut, T, torch.bfloat16)
+    assert bool(torch.isfinite(out.float()).all())
+    assert float((ones.float() - 1).abs().max()) <= 2 ** -4
+    h = cfg.H - 1
+    qc, kc, vc = (t[:, h:h + 1].cpu() for t in (q, k, v))
+    ref = O.sla_forward(qc, kc, vc, w, b, cfg.topk, cfg.feature_map, cfg.BLKQ, cfg.BLKK, linear_dtype=torch.float32)[0]
+    assert cos_sim(out[:, h:h + 1].cpu(), ref) >= 0.995
