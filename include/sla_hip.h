@@ -53,6 +53,7 @@ extern "C" {
 #define SLA_WS_SAGE_PREPARE 6
 #define SLA_WS_LINEAR_STATES 7 /* not an operation: the leading bytes of the SLA_WS_LINEAR_FWD workspace that hold the
                                   finished per-head states (see sla_linear_bwd, SLA_BWD_STATES_READY) */
+#define SLA_WS_LINEAR_COMPLEMENT_BWD 8
 
 /* flags of sla_linear_bwd */
 #define SLA_BWD_ACCUMULATE 1   /* dq, dk, dv already hold the sparse branch's gradients: add to them */
@@ -160,7 +161,7 @@ int sla_sparse_attn_linear_fwd_strided(const void* q, const void* k, const void*
                                        const int64_t* out_strides, float* lse, int dtype, int fmap, int B, int H, int L,
                                        int D, int BLKQ, int BLKK, int topk, float qk_scale, void* stream);
 
-/* Linear branch in "complement" mode (opt-in; forward only): query block i attends linearly only to the key
+/* Linear branch in "complement" mode (opt-in): query block i attends linearly only to the key
  * blocks (of 64 rows) that its look-up row did NOT select; projection, bias and residual as in
  * sla_linear_fwd.  out = residual + proj(o_l).  lut as produced by sla_block_map_fwd; BLKK must be 64.
  * The mounted reference has no code for this variant (its README.md:8 names it; core.py:92-96 computes
@@ -168,6 +169,18 @@ int sla_sparse_attn_linear_fwd_strided(const void* q, const void* k, const void*
 int sla_linear_complement_fwd(const void* q, const void* k, const void* v, const void* lut, int lut_elem_bytes,
                               const float* weight, const float* bias, const void* residual, void* out, int dtype,
                               int fmap, int B, int H, int L, int D, int BLKQ, int BLKK, int topk, void* workspace,
+                              int64_t workspace_bytes, void* stream);
+
+/* Backward of sla_linear_complement_fwd: gradients of the complement-mode linear branch only (the residual's
+ * gradient is d_out itself).  sparse_map and lut as produced by sla_block_map_fwd for the same q, k (the map
+ * gives the per-key-block lists of selecting query blocks).  dq, dk, dv in `dtype`, d_weight (D,D) and d_bias (D)
+ * fp32; flags: SLA_BWD_ACCUMULATE as in sla_linear_bwd.  Workspace: SLA_WS_LINEAR_COMPLEMENT_BWD.
+ * No counterpart in the mounted reference (see sla_linear_complement_fwd); checked against autograd through
+ * the oracle's definition. */
+int sla_linear_complement_bwd(const void* q, const void* k, const void* v, const int8_t* sparse_map, const void* lut,
+                              int lut_elem_bytes, const float* weight, const float* bias, const void* d_out, void* dq,
+                              void* dk, void* dv, float* d_weight, float* d_bias, int dtype, int fmap, int B, int H,
+                              int L, int D, int BLKQ, int BLKK, int topk, int flags, void* workspace,
                               int64_t workspace_bytes, void* stream);
 
 /* Linear branch backward.  d_out is the gradient of `out` above.  Writes dq, dk, dv in `dtype`

@@ -15,7 +15,8 @@ LIB_PATH = os.path.join(_HERE, "lib", "libsla_hip.so")
 
 SLA_F32, SLA_BF16, SLA_F16 = 0, 1, 2
 FMAP = {"elu": 0, "relu": 1, "softmax": 2}
-WS_BLOCK_MAP, WS_SPARSE_BWD, WS_LINEAR_FWD, WS_LINEAR_BWD, WS_SAGE_QUANT, WS_LINEAR_COMPLEMENT, WS_SAGE_PREPARE, WS_LINEAR_STATES = range(8)
+(WS_BLOCK_MAP, WS_SPARSE_BWD, WS_LINEAR_FWD, WS_LINEAR_BWD, WS_SAGE_QUANT, WS_LINEAR_COMPLEMENT, WS_SAGE_PREPARE,
+ WS_LINEAR_STATES, WS_LINEAR_COMPLEMENT_BWD) = range(9)
 BWD_ACCUMULATE, BWD_STATES_READY = 1, 2
 
 ERR_BAD_ARG, ERR_UNSUPPORTED, ERR_LAUNCH, ERR_WORKSPACE = -1, -2, -3, -4
@@ -48,6 +49,8 @@ SIGNATURES = {
     "sla_linear_out_fwd": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I64, _P]),
     "sla_linear_complement_fwd": (_I, [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _I64,
                                        _P]),
+    "sla_linear_complement_bwd": (_I, [_P, _P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I,
+                                       _I, _I, _I, _P, _I64, _P]),
     "sla_linear_bwd": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P, _I64, _P]),
     "sage_quant_qk": (_I, [_P, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _I64, _P]),
     "sage_prepare": (_I, [_P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I64, _P]),

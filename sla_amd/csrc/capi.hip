@@ -49,6 +49,7 @@ int64_t sage_quant_workspace_bytes(int BH, int L, int D);
 int64_t sage_prepare_workspace_bytes(int BH, int L, int D);
 int64_t linear_states_bytes(int BH, int L, int D);
 int64_t linear_complement_workspace_bytes(int BH, int L, int D);
+int64_t linear_complement_bwd_workspace_bytes(int BH, int L, int D, int BLKQ);
 
 }  // namespace sla
 
@@ -82,6 +83,9 @@ extern "C" int64_t sla_workspace_bytes(int op, int dtype, int B, int H, int L, i
       return sage_prepare_workspace_bytes(BH, L, D);
     case SLA_WS_LINEAR_COMPLEMENT:
       return linear_complement_workspace_bytes(BH, L, D);
+    case SLA_WS_LINEAR_COMPLEMENT_BWD:
+      SLA_REQUIRE(BLKQ == 64 || BLKQ == 128, SLA_ERR_UNSUPPORTED, "BLKQ=%d (64 or 128)", BLKQ);
+      return linear_complement_bwd_workspace_bytes(BH, L, D, BLKQ);
     default:
       set_error("unknown workspace op %d", op);
       return SLA_ERR_BAD_ARG;

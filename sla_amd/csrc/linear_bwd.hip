@@ -645,6 +645,58 @@ static int linear_bwd_impl(const void* q, const void* k, const void* v, const fl
   return check_launch("linear_bwd");
 }
 
+// dW and db alone, from the row-wise temporaries a rows kernel has left (used by the backward of the complement-mode
+// linear branch, whose state gradients are per query block and formed elsewhere): the states kernel, its reduction and
+// the sum over the heads.  `ws` is a region of weight_grads_workspace_bytes() bytes.
+struct WeightGradWs {
+  LinSplit st;
+  size_t ds_part, dw_part, dz_part, db_part, ds, dst, dz, dw_head, db_head, total;
+};
+static WeightGradWs weight_grad_ws(int BH, int L, int D) {
+  WeightGradWs w;
+  w.st = lin_split(BH, L, 512);
+  const int64_t np = (int64_t)BH * w.st.nsplit;
+  size_t off = 0;
+  w.ds_part = off; off += align_up(np * D * D * 4, 256);
+  w.dw_part = off; off += align_up(np * D * D * 4, 256);
+  w.dz_part = off; off += align_up(np * D * 4, 256);
+  w.db_part = off; off += align_up(np * D * 4, 256);
+  w.ds = off;      off += align_up((int64_t)BH * D * D * 2, 256);
+  w.dst = off;     off += align_up((int64_t)BH * D * D * 2, 256);
+  w.dz = off;      off += align_up((int64_t)BH * D * 4, 256);
+  w.dw_head = off; off += align_up((int64_t)BH * D * D * 4, 256);
+  w.db_head = off; off += align_up((int64_t)BH * D * 4, 256);
+  w.total = off;
+  return w;
+}
+int64_t weight_grads_workspace_bytes(int BH, int L, int D) { return (int64_t)weight_grad_ws(BH, L, D).total; }
+
+template <typename Tag, int D>
+static void weight_grads_impl(const void* q, const void* dn, const void* gout, const void* y, const float* dden, int BH, int L,
+                              int fmap, char* ws, float* d_weight, float* d_bias, hipStream_t st) {
+  const WeightGradWs w = weight_grad_ws(BH, L, D);
+  const RowLayout lay = contiguous_layout(BH, L, D);
+  hipLaunchKernelGGL((linear_bwd_states_kernel<Tag, D>), dim3(w.st.nsplit, BH), dim3(256), 0, st, (const uint16_t*)q,
+                     (const uint16_t*)dn, (const uint16_t*)gout, (const uint16_t*)y, dden, lay, lay, (float*)(ws + w.ds_part),
+                     (float*)(ws + w.dw_part), (float*)(ws + w.dz_part), (float*)(ws + w.db_part), L, w.st.rows_per_split, fmap);
+  hipLaunchKernelGGL((linear_bwd_reduce_kernel<Tag>), dim3(cdiv(D * D, 256), BH), dim3(256), 0, st,
+                     (const float*)(ws + w.ds_part), (const float*)(ws + w.dw_part), (const float*)(ws + w.dz_part),
+                     (const float*)(ws + w.db_part), (uint16_t*)(ws + w.ds), (uint16_t*)(ws + w.dst), (float*)(ws + w.dz),
+                     (float*)(ws + w.dw_head), (float*)(ws + w.db_head), w.st.nsplit, D);
+  hipLaunchKernelGGL(linear_bwd_reduce_heads_kernel, dim3(cdiv(D * D, 256)), dim3(256), 0, st,
+                     (const float*)(ws + w.dw_head), (const float*)(ws + w.db_head), d_weight, d_bias, BH, D);
+}
+void launch_weight_grads(int dtype, int D, const void* q, const void* dn, const void* gout, const void* y, const float* dden,
+                         int BH, int L, int fmap, char* ws, float* d_weight, float* d_bias, hipStream_t st) {
+  if (dtype == SLA_BF16) {
+    if (D == 128) weight_grads_impl<bf16_tag, 128>(q, dn, gout, y, dden, BH, L, fmap, ws, d_weight, d_bias, st);
+    else weight_grads_impl<bf16_tag, 64>(q, dn, gout, y, dden, BH, L, fmap, ws, d_weight, d_bias, st);
+  } else {
+    if (D == 128) weight_grads_impl<f16_tag, 128>(q, dn, gout, y, dden, BH, L, fmap, ws, d_weight, d_bias, st);
+    else weight_grads_impl<f16_tag, 64>(q, dn, gout, y, dden, BH, L, fmap, ws, d_weight, d_bias, st);
+  }
+}
+
 }  // namespace sla
 
 using namespace sla;

@@ -7,11 +7,14 @@ namespace sla {
 // ---- kernel 1: partial states -----------------------------------------------------------
 // grid (nsplit, BH), 256 threads.  Thread t moves 16-byte chunk (t%CPR) of rows t/CPR + i*RPP.
 // OUT16: the D x D partial is written rounded to 16 bit (per-key-block states of the complement mode).
-template <typename Tag, int D, bool OUT16 = false>
+// ZW: zweight holds one fp32 per row of the head, (BH, L), and the z partial becomes sum_rows zweight * phi(k)
+// instead of sum_rows phi(k) (used by the complement backward, where "k" is q and "v" a row gradient).
+template <typename Tag, int D, bool OUT16 = false, bool ZW = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void linear_state_partial_kernel(const uint16_t* __restrict__ k,
                                                                    const uint16_t* __restrict__ v, const RowLayout lay,
                                                                    void* __restrict__ kv_part_, float* __restrict__ z_part,
-                                                                   int L, int rows_per_split, int fmap) {
+                                                                   int L, int rows_per_split, int fmap,
+                                                                   const float* __restrict__ zweight = nullptr) {
   using E = Elem<Tag>;
   constexpr int TR = 64;                 // rows per LDS tile
   constexpr int STR = D + 16;            // LDS row stride: transposed reads of 4 rows hit disjoint banks
@@ -52,15 +55,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
 
   // rows of the next tile are fetched into registers while the current tile is multiplied
   i16x8_t kreg[NP], vreg[NP];
+  float wreg[NP];
   auto fetch = [&](int r0) {
 #pragma unroll
     for (int p = 0; p < NP; ++p) {
       const int grow = r0 + lrow + p * RPP;
       kreg[p] = i16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
       vreg[p] = i16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+      wreg[p] = 1.0f;
       if (grow < row_end) {
         kreg[p] = *reinterpret_cast<const i16x8_t*>(kh + (size_t)grow * pitch + lcol);
         vreg[p] = *reinterpret_cast<const i16x8_t*>(vh + (size_t)grow * pitch + lcol);
+        if (ZW) wreg[p] = zweight[(size_t)bh * L + grow];
       }
     }
   };
@@ -102,7 +108,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         if (!ok) f[e] = 0.f;              // rows past the end take no part (phi(0) is not 0 for elu/softmax)
-        zacc[e] += f[e];
+        zacc[e] += ZW ? wreg[p] * f[e] : f[e];
         fk[e] = (short)E::from_float(f[e]);
       }
       *reinterpret_cast<i16x8_t*>(&sK[row * STR + lcol]) = fk;

@@ -523,6 +523,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 }
 
 // ---- host ---------------------------------------------------------------------------------
+// list[bh][n][0..count[bh][n]) = the query blocks that selected key block n, ascending; capacity Mblk per list
+// (also used by the backward of the complement-mode linear branch)
+void launch_col_lists(const int8_t* sparse_map, int* list, int* count, int BH, int Mblk, int Nblk, hipStream_t st) {
+  // 16-byte loads of map rows need 16-byte aligned rows
+  const int vec_ok = (Nblk % 16 == 0) && ((uintptr_t)sparse_map % 16 == 0);
+  hipLaunchKernelGGL(bwd_col_lists_kernel, dim3(cdiv(Nblk, 64), BH), dim3(64 * COL_NW), 0, st, sparse_map, list, count, Mblk, Nblk,
+                     vec_ok);
+}
+
 struct BwdWs {
   size_t delta, count, list, total;
 };
@@ -556,10 +565,7 @@ static int bwd_impl(const void* q, const void* k, const void* v, const void* o, 
   constexpr int RPB = 256 / (D / 8);
   hipLaunchKernelGGL((bwd_delta_kernel<Tag, D>), dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, st,
                      (const uint16_t*)o, (const uint16_t*)d_o, ldo, delta, rows, L);
-  // 16-byte loads of map rows need 16-byte aligned rows
-  const int vec_ok = (Nblk % 16 == 0) && ((uintptr_t)sparse_map % 16 == 0);
-  hipLaunchKernelGGL(bwd_col_lists_kernel, dim3(cdiv(Nblk, 64), BH), dim3(64 * COL_NW), 0, st, sparse_map, list, count, Mblk, Nblk,
-                     vec_ok);
+  launch_col_lists(sparse_map, list, count, BH, Mblk, Nblk, st);
   const int total_q = BH * Mblk;
   const int total_k = BH * Nblk;
   const bool contig = lin.sl == D && ldo.sl == D;

@@ -60,7 +60,7 @@ def linear_complement_fwd(q, k, v, lut, topk, weight, bias, residual, fmap: str,
     """Linear branch over the key blocks each query block did NOT select, + projection + ``residual``.
 
     Opt-in variant (the paper's formulation); the reference module computes the global branch
-    (``core.py:92-96``).  Forward only."""
+    (``core.py:92-96``).  :func:`linear_complement_bwd` is its backward."""
     _lib.require_gpu(q, k, v, lut, weight, bias)
     B, H, L, D = q.shape
     dt = _lib.dtype_code(q.dtype)
@@ -75,6 +75,37 @@ def linear_complement_fwd(q, k, v, lut, topk, weight, bias, residual, fmap: str,
                                                ws.numel(), _lib.stream_ptr(q.device))
     _lib.check(rc)
     return out
+
+
+def linear_complement_bwd(q, k, v, sparse_map, lut, topk, weight, bias, d_out, fmap: str, BLKQ: int = 64, BLKK: int = 64,
+                          accumulate_into=None):
+    """Gradients of :func:`linear_complement_fwd` (the linear branch only; the residual's gradient is ``d_out``).
+
+    ``sparse_map`` and ``lut`` are the pair ``get_block_map`` returned.  ``accumulate_into=(dq, dk, dv)`` adds to
+    existing gradient tensors instead of allocating new ones.  Returns ``(dq, dk, dv, d_weight, d_bias)``."""
+    _lib.require_gpu(q, k, v, sparse_map, lut, weight, bias, d_out)
+    B, H, L, D = q.shape
+    dt = _lib.dtype_code(q.dtype)
+    if lut.dtype not in (torch.int32, torch.int64):
+        raise TypeError(f"lut must be int32 or int64, got {lut.dtype}")
+    assert sparse_map.dtype == torch.int8 and sparse_map.is_contiguous() and lut.is_contiguous()
+    assert q.is_contiguous() and k.is_contiguous() and v.is_contiguous() and d_out.is_contiguous()
+    ws = _lib.workspace(_lib.WS_LINEAR_COMPLEMENT_BWD, dt, B, H, L, D, BLKQ, BLKK, topk, q.device)
+    if accumulate_into is None:
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        flags = 0
+    else:
+        dq, dk, dv = accumulate_into
+        flags = _lib.BWD_ACCUMULATE
+    dw = torch.empty((D, D), dtype=torch.float32, device=q.device)
+    db = torch.empty((D,), dtype=torch.float32, device=q.device)
+    rc = _lib.load().sla_linear_complement_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), sparse_map.data_ptr(),
+                                               lut.data_ptr(), lut.element_size(), weight.data_ptr(), bias.data_ptr(),
+                                               d_out.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
+                                               dw.data_ptr(), db.data_ptr(), dt, _lib.FMAP[fmap], B, H, L, D, BLKQ, BLKK,
+                                               topk, flags, ws.data_ptr(), ws.numel(), _lib.stream_ptr(q.device))
+    _lib.check(rc)
+    return dq, dk, dv, dw, db
 
 
 def saved_states(state_ws, q):

@@ -7,7 +7,7 @@ import torch.nn as nn
 
 from . import _lib
 from .block_map import get_block_map
-from .linear import linear_bwd, linear_complement_fwd, linear_state_fwd, saved_states
+from .linear import linear_bwd, linear_complement_bwd, linear_complement_fwd, linear_state_fwd, saved_states
 from .sparse_attn import sparse_attn_bwd, sparse_attn_fwd, sparse_attn_linear_fwd
 
 FEATURE_MAPS = ("elu", "relu", "softmax")
@@ -49,6 +49,35 @@ class _sla_core(torch.autograd.Function):
         dq, dk, dv = sparse_attn_bwd(q, k, v, o_s, d_out, lse, sparse_map, lut, topk, BLKQ, BLKK, qk_scale)
         _, _, _, dw, db = linear_bwd(q, k, v, weight, bias, d_out, fmap, accumulate_into=(dq, dk, dv), states=states)
         return dq, dk, dv, dw, db, None, None, None, None, None, None, None, None
+
+
+class _sla_complement(torch.autograd.Function):
+    """Sparse branch + complement-mode linear branch (over the key blocks a query block did not select) + projection
+    + sum.  The reference has no such variant; the definition is ``linear_complement_fwd``'s."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, weight, bias, sparse_map, lut, topk, BLKQ, BLKK, fmap):
+        assert q.is_contiguous() and k.is_contiguous() and v.is_contiguous()
+        assert sparse_map.is_contiguous() and lut.is_contiguous()
+        assert BLKQ in (64, 128) and BLKK == 64
+        qk_scale = q.shape[-1] ** -0.5
+        weight, bias = weight.contiguous(), bias.contiguous()
+        o_s, lse = sparse_attn_fwd(q, k, v, lut, topk, BLKQ, BLKK, qk_scale)
+        out = linear_complement_fwd(q, k, v, lut, topk, weight, bias, o_s, fmap, BLKQ, BLKK)
+        if any(ctx.needs_input_grad[:5]):
+            ctx.save_for_backward(q, k, v, weight, bias, sparse_map, lut, lse, o_s)
+            ctx.cfg = (topk, BLKQ, BLKK, fmap, qk_scale)
+        return out
+
+    @staticmethod
+    def backward(ctx, d_out):
+        q, k, v, weight, bias, sparse_map, lut, lse, o_s = ctx.saved_tensors
+        topk, BLKQ, BLKK, fmap, qk_scale = ctx.cfg
+        d_out = d_out.contiguous()
+        dq, dk, dv = sparse_attn_bwd(q, k, v, o_s, d_out, lse, sparse_map, lut, topk, BLKQ, BLKK, qk_scale)
+        _, _, _, dw, db = linear_complement_bwd(q, k, v, sparse_map, lut, topk, weight, bias, d_out, fmap, BLKQ, BLKK,
+                                                accumulate_into=(dq, dk, dv))
+        return dq, dk, dv, dw, db, None, None, None, None, None, None
 
 
 class _sla_packed(torch.autograd.Function):
@@ -139,8 +168,7 @@ class SparseLinearAttention(nn.Module):
             tie_feature_map_qk: kept for signature compatibility; q and k always use the same map
                 (as in the reference, core.py:43-60).
             linear_mode: "global" (default, what the reference computes: the linear branch sees every key)
-                or "complement" (extension: it sees only the key blocks the query block did not select;
-                forward only).
+                or "complement" (extension: it sees only the key blocks the query block did not select).
         """
         super().__init__()
         self.dtype = torch.bfloat16 if use_bf16 else torch.float16
@@ -227,13 +255,9 @@ class SparseLinearAttention(nn.Module):
         return o
 
     def _forward_complement(self, q, k, qc, kc, vc, dtype, return_sparsity):
-        if torch.is_grad_enabled() and any(t.requires_grad for t in (qc, kc, vc, self.proj_l.weight, self.proj_l.bias)):
-            raise NotImplementedError("linear_mode='complement' has no backward; call it under torch.no_grad()")
         sparse_map, lut, real_topk = get_block_map(q, k, topk_ratio=self.topk, BLKQ=self.BLKQ, BLKK=self.BLKK)
-        assert self.BLKQ in (64, 128) and self.BLKK == 64
-        o_s, _ = sparse_attn_fwd(qc, kc, vc, lut, real_topk, self.BLKQ, self.BLKK, qc.shape[-1] ** -0.5)
-        o = linear_complement_fwd(qc, kc, vc, lut, real_topk, self.proj_l.weight.contiguous(),
-                                  self.proj_l.bias.contiguous(), o_s, self.feature_map, self.BLKQ, self.BLKK).to(dtype)
+        o = _sla_complement.apply(qc, kc, vc, self.proj_l.weight, self.proj_l.bias, sparse_map, lut, real_topk, self.BLKQ,
+                                  self.BLKK, self.feature_map).to(dtype)
         if return_sparsity:
             return o, real_topk / sparse_map.shape[-1]
         return o

@@ -78,6 +78,15 @@ def test_other_entry_points_validate():
                                           128, 64, 64, 1, 0.1, None) == _lib.ERR_BAD_ARG
     assert lib.sla_linear_complement_fwd(FAKE, FAKE, FAKE, FAKE, 8, FAKE, FAKE, None, FAKE, 1, 0, 1, 1, 128, 128, 64, 32, 1,
                                          FAKE, 1 << 30, None) == _lib.ERR_UNSUPPORTED
+    cb = lambda **kw: lib.sla_linear_complement_bwd(  # noqa: E731
+        FAKE, FAKE, FAKE, kw.get("m", FAKE), FAKE, 8, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, 1, 0, 1, 1, 128, 128,
+        kw.get("BLKQ", 64), 64, 1, kw.get("flags", 0), FAKE, kw.get("ws", 1 << 30), None)
+    assert cb(ws=8) == _lib.ERR_WORKSPACE
+    assert cb(flags=2) == _lib.ERR_BAD_ARG and "flag" in _lib.last_error()
+    assert cb(m=None) == _lib.ERR_BAD_ARG
+    assert cb(BLKQ=32) == _lib.ERR_UNSUPPORTED
+    need = lib.sla_workspace_bytes(_lib.WS_LINEAR_COMPLEMENT_BWD, 1, 1, 2, 128, 128, 64, 64, 1)
+    assert need > lib.sla_workspace_bytes(_lib.WS_LINEAR_COMPLEMENT, 1, 1, 2, 128, 128, 64, 64, 1) > 0
     assert lib.sla_linear_state_fwd(FAKE, FAKE, FAKE, 1, 0, 1, 1, 64, 128, FAKE, 8, None) == _lib.ERR_WORKSPACE
     assert lib.sla_linear_state_fwd(FAKE, None, FAKE, 1, 0, 1, 1, 64, 128, FAKE, 1 << 30, None) == _lib.ERR_BAD_ARG
     assert lib.sla_linear_out_fwd(FAKE, FAKE, None, FAKE, 0, 0, 1, 1, 64, 128, FAKE, 1 << 30, None) == _lib.ERR_UNSUPPORTED

@@ -6,7 +6,7 @@ from conftest import cos_sim, max_abs
 from oracle import sla_oracle as O
 from sla_amd import SparseLinearAttention
 from sla_amd.inputs import CONFIGS, make_inputs, make_proj
-from sla_amd.linear import linear_complement_fwd, linear_fwd
+from sla_amd.linear import linear_bwd, linear_complement_bwd, linear_complement_fwd, linear_fwd
 
 pytestmark = pytest.mark.gpu
 
@@ -58,6 +58,69 @@ def test_int32_lut_and_module_option(dev):
     out64 = linear_complement_fwd(q.to(dev), k.to(dev), v.to(dev), lut.to(dev), T, w.to(dev), b.to(dev), None, "relu")
     assert torch.equal(out32, out64)
     with pytest.raises(NotImplementedError):
-        mod(q.to(dev), k.to(dev), v.to(dev))          # gradients enabled: no backward for this mode
-    with pytest.raises(NotImplementedError):
         SparseLinearAttention(cfg.D, cfg.topk, "relu", linear_mode="selected")
+
+
+def _oracle_grads(q, k, v, lut, w, b, g, fmap, BLKQ):
+    leaves = [t.float().clone().requires_grad_(True) for t in (q, k, v, w, b)]
+    O.linear_branch_complement(*leaves[:3], lut, *leaves[3:], fmap, BLKQ, 64, torch.float32).backward(g.float())
+    return [t.grad for t in leaves]
+
+
+def _check_grads(got, refs):
+    for name, a, r in zip(("dq", "dk", "dv", "dW", "db"), got, refs):
+        a = a.cpu()
+        scale = max(1.0, float(r.abs().max()))          # dW/db are sums over B*H*L rows
+        assert max_abs(a, r) <= TOL_ABS * scale, (name, max_abs(a, r), scale)
+        assert cos_sim(a, r) >= TOL_COS, (name, cos_sim(a, r))
+
+
+@pytest.mark.parametrize("fmap", ["elu", "relu", "softmax"])
+@pytest.mark.parametrize("L,D,BLKQ,ratio", [(512, 128, 64, 0.25), (1000, 128, 128, 0.3), (333, 64, 64, 0.5), (700, 64, 128, 0.2),
+                                            (150, 128, 64, 0.4)])
+def test_complement_backward_vs_autograd_oracle(dev, fmap, L, D, BLKQ, ratio):
+    gen = torch.Generator().manual_seed(L + D + 1)
+    q, k, v, g = (torch.randn(2, 2, L, D, generator=gen).to(torch.bfloat16) for _ in range(4))
+    w, b = make_proj(D)
+    m, lut, T = O.get_block_map(q, k, ratio, BLKQ, 64)
+    refs = _oracle_grads(q, k, v, lut, w, b, g, fmap, BLKQ)
+    args = [t.to(dev) for t in (q, k, v, m, lut)]
+    got = linear_complement_bwd(*args, T, w.to(dev), b.to(dev), g.to(dev), fmap, BLKQ, 64)
+    _check_grads(got, refs)
+    # adding into existing gradients: one more 16-bit rounding of the sum
+    base = [torch.randn(2, 2, L, D, generator=gen).to(torch.bfloat16).to(dev) for _ in range(3)]
+    acc = linear_complement_bwd(*args, T, w.to(dev), b.to(dev), g.to(dev), fmap, BLKQ, 64,
+                                accumulate_into=tuple(t.clone() for t in base))
+    for a, x, y in zip(acc[:3], base, got[:3]):
+        assert torch.equal(a, (x.float() + y.float()).to(torch.bfloat16))
+    assert torch.equal(acc[3], got[3]) and torch.equal(acc[4], got[4])
+
+
+def test_backward_with_nothing_selected_equals_the_global_backward(dev):
+    gen = torch.Generator().manual_seed(13)
+    q, k, v, g = (torch.randn(1, 2, 640, 128, generator=gen).to(torch.bfloat16).to(dev) for _ in range(4))
+    w, b = (t.to(dev) for t in make_proj(128))
+    lut = torch.zeros((1, 2, 10, 0), dtype=torch.int64, device=dev)
+    m = torch.zeros((1, 2, 10, 10), dtype=torch.int8, device=dev)
+    got = linear_complement_bwd(q, k, v, m, lut, 0, w, b, g, "elu")
+    ref = linear_bwd(q, k, v, w, b, g, "elu")
+    _check_grads(got, [t.cpu().float() for t in ref])
+
+
+def test_module_trains_in_complement_mode(dev):
+    cfg = CONFIGS["cfg2"]
+    d = make_inputs(cfg, H=2)
+    q, k, v, do = (d[x] for x in ("q", "k", "v", "do"))
+    w, b = make_proj(cfg.D)
+    mod = SparseLinearAttention(cfg.D, cfg.topk, "softmax", cfg.BLKQ, cfg.BLKK, linear_mode="complement").to(dev)
+    with torch.no_grad():
+        mod.proj_l.weight.copy_(w)
+        mod.proj_l.bias.copy_(b)
+    qd, kd, vd = (t.to(dev).requires_grad_(True) for t in (q, k, v))
+    mod(qd, kd, vd).backward(do.to(dev))
+    m, lut, T = O.get_block_map(q, k, cfg.topk, cfg.BLKQ, cfg.BLKK)
+    o_s, lse = O.sparse_attn_fwd_gather(q, k, v, lut, cfg.BLKQ, cfg.BLKK)
+    sp = O.sparse_attn_bwd_gather(q, k, v, o_s, do, lse, lut, cfg.BLKQ, cfg.BLKK)
+    lin = _oracle_grads(q, k, v, lut, w, b, do, "softmax", cfg.BLKQ)
+    refs = [a + c for a, c in zip(sp, lin[:3])] + lin[3:]
+    _check_grads((qd.grad, kd.grad, vd.grad, mod.proj_l.weight.grad, mod.proj_l.bias.grad), refs)

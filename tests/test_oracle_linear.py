@@ -121,3 +121,21 @@ def test_complement_with_everything_selected_is_the_bias():
     got = O.linear_branch_complement(q, k, v, lut, w, b, "relu", 64, 64, torch.float32)
     # numerator and divisor state are (numerically) zero: o_l = 0 / 1e-5, so only the bias is left
     assert float((got - b).abs().max()) < 1e-2
+
+
+@pytest.mark.parametrize("fmap", ["elu", "relu", "softmax"])
+def test_complement_gradients_equal_those_of_the_masked_dense_form(fmap):
+    """Autograd through the block-state formulation (what the GPU tests use as the gradient oracle) against
+    autograd through the dense masked kernelised attention in fp64."""
+    q, k, v, m, lut, T, w, b = _complement_case()
+    L = q.shape[2]
+    g = torch.randn(q.shape, generator=torch.Generator().manual_seed(9))
+    leaves = [t.clone().requires_grad_(True) for t in (q, k, v, w, b)]
+    O.linear_branch_complement(*leaves[:3], lut, *leaves[3:], fmap, 64, 64, torch.float32).backward(g)
+    ref = [t.double().requires_grad_(True) for t in (q, k, v, w, b)]
+    phi = O.feature_map(fmap)
+    a = (phi(ref[0]) @ phi(ref[1]).transpose(-1, -2)) * ~O.expand_block_map(m, L, 64, 64)
+    o = (a @ ref[2]) / (1e-5 + a.sum(dim=-1, keepdim=True))
+    torch.nn.functional.linear(o, ref[3], ref[4]).backward(g.double())
+    for x, r in zip(leaves, ref):
+        assert float((x.grad.double() - r.grad).abs().max()) <= 1e-3 * max(1.0, float(r.grad.abs().max()))
