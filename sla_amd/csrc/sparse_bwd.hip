@@ -111,6 +111,101 @@ __global__ __launch_bounds__(64 * COL_NW) void bwd_col_lists_kernel(const int8_t
   if (wave == 0 && n < Nblk) count[(size_t)bh * Nblk + n] = done;
 }
 
+// ---- work items of the dK/dV kernel --------------------------------------------------------
+// A key block that very many query blocks selected (an attention "sink") would make one workgroup walk a list
+// many times the average length.  Lists longer than `seg` entries are therefore cut into segments of `seg`; every
+// segment is one work item.  item = {bh, key block, segment, slot}: slot < 0 for a key block with a single segment
+// (the workgroup writes dK / dV itself), otherwise the index of the fp32 partial this segment writes; the partials
+// of a key block occupy consecutive slots and are added in segment order by bwd_dkdv_reduce_kernel.
+// One workgroup of 1024 threads walks all (head, key block) pairs in order with a running prefix sum.
+__global__ __launch_bounds__(1024) void bwd_segments_kernel(const int* __restrict__ count, int* __restrict__ nseg,
+                                                            int* __restrict__ slot0, i32x4_t* __restrict__ items,
+                                                            int* __restrict__ totals, int nblocks, int Nblk, int seg,
+                                                            int max_items, int max_slots) {
+  __shared__ int wsum[2][16];
+  __shared__ int base[2];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  if (tid == 0) base[0] = base[1] = 0;
+  __syncthreads();
+  for (int i0 = 0; i0 < nblocks; i0 += 1024) {
+    const int i = i0 + tid;
+    const int ns = i < nblocks ? max(1, (count[i] + seg - 1) / seg) : 0;
+    const int ms = ns > 1 ? ns : 0;
+    int a = ns, b = ms;                       // inclusive scans inside the wave
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int ta = __shfl_up(a, o), tb = __shfl_up(b, o);
+      if (lane >= o) {
+        a += ta;
+        b += tb;
+      }
+    }
+    if (lane == 63) {
+      wsum[0][wave] = a;
+      wsum[1][wave] = b;
+    }
+    __syncthreads();
+    int pa = 0, pb = 0, ta = 0, tb = 0;
+#pragma unroll
+    for (int w = 0; w < 16; ++w) {
+      pa += w < wave ? wsum[0][w] : 0;
+      pb += w < wave ? wsum[1][w] : 0;
+      ta += wsum[0][w];
+      tb += wsum[1][w];
+    }
+    if (i < nblocks) {
+      const int first_item = base[0] + pa + a - ns, first_slot = base[1] + pb + b - ms;
+      nseg[i] = ns;
+      slot0[i] = first_slot;
+      const int bh = i / Nblk, nb = i - bh * Nblk;
+      // (a map whose rows hold more ones than the topk the workspace was sized for cannot overrun the tables: its
+      //  surplus items are dropped)
+      for (int sg = 0; sg < ns; ++sg)
+        if (first_item + sg < max_items && first_slot + ms <= max_slots)
+          items[first_item + sg] = i32x4_t{bh, nb, sg, ns > 1 ? first_slot + sg : -1};
+        else if (first_item + sg < max_items)
+          items[first_item + sg] = i32x4_t{bh, nb, sg, -2};
+    }
+    __syncthreads();
+    if (tid == 0) {
+      base[0] += ta;
+      base[1] += tb;
+    }
+    __syncthreads();
+  }
+  if (tid == 0) {
+    totals[0] = min(base[0], max_items);
+    totals[1] = min(base[1], max_slots);
+  }
+}
+
+// grid (Nblk, BH), 256 threads: key blocks whose list was cut add their partials (fp32, [slot][dk | dv][64][D]) in
+// segment order and write dK, dV; all others leave at once.
+template <typename Tag, int D>
+__global__ __launch_bounds__(256) void bwd_dkdv_reduce_kernel(const int* __restrict__ nseg, const int* __restrict__ slot0,
+                                                              const float* __restrict__ part, uint16_t* __restrict__ dk,
+                                                              uint16_t* __restrict__ dv, const RowLayout lin, int L, int Nblk,
+                                                              int max_slots) {
+  using E = Elem<Tag>;
+  const int nb = blockIdx.x, bh = blockIdx.y;
+  const int ns = nseg[(size_t)bh * Nblk + nb];
+  if (ns <= 1 || slot0[(size_t)bh * Nblk + nb] + ns > max_slots) return;
+  const float* p0 = part + (size_t)slot0[(size_t)bh * Nblk + nb] * (2 * 64 * D);
+  for (int idx = threadIdx.x * 4; idx < 2 * 64 * D; idx += 256 * 4) {
+    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+    for (int sg = 0; sg < ns; ++sg) acc += *reinterpret_cast<const f32x4_t*>(p0 + (size_t)sg * (2 * 64 * D) + idx);
+    const int which = idx / (64 * D), rem = idx - which * (64 * D);
+    const int row = nb * 64 + rem / D, col = rem % D;
+    if (row < L) {
+      i32x2_t w;
+      w[0] = (int)E::pack2(acc[0], acc[1]);
+      w[1] = (int)E::pack2(acc[2], acc[3]);
+      uint16_t* dst = (which ? dv : dk) + lin.head(bh) + (size_t)row * (size_t)lin.sl + col;
+      *reinterpret_cast<i32x2_t*>(dst) = w;
+    }
+  }
+}
+
 // ---- dQ ---------------------------------------------------------------------------------
 // One workgroup per query block, one wave per 32 queries.  Register use is held to 256 so that two waves
 // share a SIMD.  K and V tiles go global -> registers -> LDS; both tiles of the next step are in flight
@@ -309,8 +404,9 @@ template <typename Tag, int D, int BLKQ, bool CONTIG>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void bwd_dkdv_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ k, const uint16_t* __restrict__ v,
     const uint16_t* __restrict__ d_o, const float* __restrict__ lse, const float* __restrict__ delta,
-    const int* __restrict__ list, const int* __restrict__ count, uint16_t* __restrict__ dk, uint16_t* __restrict__ dv,
-    const RowLayout lin, const RowLayout ldo, int L, int Mblk, int Nblk, float qk_scale, int total) {
+    const int* __restrict__ list, const int* __restrict__ count, const i32x4_t* __restrict__ items,
+    const int* __restrict__ totals, float* __restrict__ part, int seg, uint16_t* __restrict__ dk, uint16_t* __restrict__ dv,
+    const RowLayout lin, const RowLayout ldo, int L, int Mblk, int Nblk, float qk_scale) {
   using E = Elem<Tag>;
   constexpr int TQ = 64;                  // query rows per LDS tile
   constexpr int SUB = BLKQ / TQ;          // tiles per listed query block
@@ -328,10 +424,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   __shared__ __attribute__((aligned(16))) i16x8_t sXP[4][2][64];    // [wave][16-row group][lane] packed P
   __shared__ __attribute__((aligned(16))) i16x8_t sXS[4][2][64];    // same for dS
 
-  const int logical = xcd_remap(blockIdx.x, gridDim.x, total);
-  if (logical < 0) return;
-  const int bh = logical / Nblk;
-  const int nb = logical - bh * Nblk;
+  // The grid covers the largest possible number of work items; the actual number is known on the device only.
+  // Every XCD takes one contiguous range of the actual items (consecutive workgroup ids go round-robin to the XCDs).
+  const int total = totals[0];
+  const int per_xcd = (total + 7) >> 3;
+  if ((int)(blockIdx.x >> 3) >= per_xcd) return;
+  const int logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  if (logical >= total) return;
+  const i32x4_t item = items[logical];
+  const int bh = item[0], nb = item[1], sg = item[2], slot = item[3];
+  if (slot < -1) return;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int kh = wave & 1, dh = wave >> 1;
   const int g = lane >> 5, r = lane & 31;
@@ -368,7 +470,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
 
   const int* mylist = list + ((size_t)bh * Nblk + nb) * Mblk;
-  const int ntile = count[(size_t)bh * Nblk + nb] * SUB;
+  // this work item's part of the list, in tiles of TQ query rows
+  const int tile0 = sg * seg * SUB;
+  const int ntile = min(count[(size_t)bh * Nblk + nb], (sg + 1) * seg) * SUB;
 
   i16x8_t qreg[NLD], doreg[NLD];
   float lreg = 0.f, dreg = 0.f;
@@ -409,13 +513,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int tr_row = (lane & 15) >> 2;
   const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
 
-  int row_next = ntile > 1 ? tile_row0(1) : 0;
-  if (ntile > 0) {
-    load_tile(tile_row0(0));
+  int row_next = tile0 + 1 < ntile ? tile_row0(tile0 + 1) : 0;
+  if (tile0 < ntile) {
+    load_tile(tile_row0(tile0));
     store_tile();
   }
   __syncthreads();
-  for (int ti = 0; ti < ntile; ++ti) {
+  for (int ti = tile0; ti < ntile; ++ti) {
     if (ti + 1 < ntile) {
       load_tile(row_next);
       row_next = ti + 2 < ntile ? tile_row0(ti + 2) : 0;
@@ -503,6 +607,22 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     if (ti + 1 < ntile) store_tile();
     __syncthreads();                       // next tile visible
   }
+  if (slot >= 0) {
+    // one segment of a long list: fp32 partial [dk | dv][64][D], added up by bwd_dkdv_reduce_kernel
+    float* pk = part + (size_t)slot * (2 * 64 * D) + (size_t)(kh * 32 + r) * D;
+    float* pv = pk + 64 * D;
+#pragma unroll
+    for (int dt = 0; dt < DH; ++dt)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; ++i4) {
+        const int d0 = 32 * (DH * dh + dt) + 8 * i4 + 4 * g;
+        *reinterpret_cast<f32x4_t*>(pk + d0) = f32x4_t{dkacc[dt][4 * i4 + 0] * qk_scale, dkacc[dt][4 * i4 + 1] * qk_scale,
+                                                       dkacc[dt][4 * i4 + 2] * qk_scale, dkacc[dt][4 * i4 + 3] * qk_scale};
+        *reinterpret_cast<f32x4_t*>(pv + d0) =
+            f32x4_t{dvacc[dt][4 * i4 + 0], dvacc[dt][4 * i4 + 1], dvacc[dt][4 * i4 + 2], dvacc[dt][4 * i4 + 3]};
+      }
+    return;
+  }
   if (kok) {
     uint16_t* dkrow = dk + head_off + (size_t)krow * pitch;
     uint16_t* dvrow = dv + head_off + (size_t)krow * pitch;
@@ -533,22 +653,36 @@ void launch_col_lists(const int8_t* sparse_map, int* list, int* count, int BH, i
 }
 
 struct BwdWs {
-  size_t delta, count, list, total;
+  int seg;                  // longest stretch of a key block's list one workgroup walks
+  int64_t max_items, max_slots;
+  size_t delta, count, list, nseg, slot0, items, totals, part, total;
 };
-static BwdWs bwd_ws(int BH, int L, int BLKQ, int BLKK) {
+static BwdWs bwd_ws(int BH, int L, int D, int BLKQ, int BLKK, int topk) {
   const int64_t M = cdiv(L, BLKQ), N = cdiv(L, BLKK);
   BwdWs w;
+  // A segment is at most a quarter of the list entries an average resident workgroup (2 per compute unit) walks, and
+  // at least 64: balanced maps are never cut, and the fp32 partials of the worst case stay bounded (the lists of one
+  // head hold M*topk entries in all, so at most 2*M*topk/seg segments belong to lists longer than seg).
+  const int64_t entries = (int64_t)BH * M * topk;
+  int64_t seg = (entries + 2047) / 2048;     // 512 resident workgroups, a quarter of the average each
+  if (seg < 64) seg = 64;
+  w.seg = (int)seg;
+  w.max_items = (int64_t)BH * N + entries / seg;
+  w.max_slots = 2 * entries / seg;
   size_t off = 0;
-  w.delta = off; off += align_up((int64_t)BH * L * 4, 256);
-  w.count = off; off += align_up((int64_t)BH * N * 4, 256);
-  w.list = off;  off += align_up((int64_t)BH * N * M * 4, 256);
+  w.delta = off;  off += align_up((int64_t)BH * L * 4, 256);
+  w.count = off;  off += align_up((int64_t)BH * N * 4, 256);
+  w.list = off;   off += align_up((int64_t)BH * N * M * 4, 256);
+  w.nseg = off;   off += align_up((int64_t)BH * N * 4, 256);
+  w.slot0 = off;  off += align_up((int64_t)BH * N * 4, 256);
+  w.items = off;  off += align_up(w.max_items * 16, 256);
+  w.totals = off; off += 256;
+  w.part = off;   off += align_up(w.max_slots * 2 * 64 * D * 4, 256);
   w.total = off;
   return w;
 }
 int64_t sparse_bwd_workspace_bytes(int BH, int L, int D, int BLKQ, int BLKK, int topk) {
-  (void)D;
-  (void)topk;
-  return (int64_t)bwd_ws(BH, L, BLKQ, BLKK).total;
+  return (int64_t)bwd_ws(BH, L, D, BLKQ, BLKK, topk).total;
 }
 
 template <typename Tag, int D, int BLKQ>
@@ -556,7 +690,7 @@ static int bwd_impl(const void* q, const void* k, const void* v, const void* o, 
                     const int8_t* sparse_map, const void* lut, int lut64, void* dq, void* dk, void* dv,
                     const RowLayout& lin, const RowLayout& ldo, int BH, int L, int topk, float qk_scale, char* ws,
                     hipStream_t st) {
-  const BwdWs w = bwd_ws(BH, L, BLKQ, 64);
+  const BwdWs w = bwd_ws(BH, L, D, BLKQ, 64, topk);
   const int Mblk = cdiv(L, BLKQ), Nblk = cdiv(L, 64);
   float* delta = (float*)(ws + w.delta);
   int* count = (int*)(ws + w.count);
@@ -566,22 +700,30 @@ static int bwd_impl(const void* q, const void* k, const void* v, const void* o, 
   hipLaunchKernelGGL((bwd_delta_kernel<Tag, D>), dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, st,
                      (const uint16_t*)o, (const uint16_t*)d_o, ldo, delta, rows, L);
   launch_col_lists(sparse_map, list, count, BH, Mblk, Nblk, st);
+  int* nseg = (int*)(ws + w.nseg);
+  int* slot0 = (int*)(ws + w.slot0);
+  i32x4_t* items = (i32x4_t*)(ws + w.items);
+  int* totals = (int*)(ws + w.totals);
+  float* part = (float*)(ws + w.part);
+  hipLaunchKernelGGL(bwd_segments_kernel, dim3(1), dim3(1024), 0, st, count, nseg, slot0, items, totals, BH * Nblk, Nblk, w.seg,
+                     (int)w.max_items, (int)w.max_slots);
   const int total_q = BH * Mblk;
-  const int total_k = BH * Nblk;
   const bool contig = lin.sl == D && ldo.sl == D;
 #define SLA_BWD_LAUNCH(CONTIG)                                                                                              \
   hipLaunchKernelGGL((bwd_dq_kernel<Tag, D, BLKQ, CONTIG>), dim3(xcd_grid(total_q)), dim3(BLKQ * 2), 0, st,                 \
                      (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse, delta, lut,     \
                      lut64, (uint16_t*)dq, lin, ldo, L, Mblk, topk, qk_scale, total_q);                                    \
-  hipLaunchKernelGGL((bwd_dkdv_kernel<Tag, D, BLKQ, CONTIG>), dim3(xcd_grid(total_k)), dim3(256), 0, st, (const uint16_t*)q, \
-                     (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse, delta, list, count, (uint16_t*)dk,  \
-                     (uint16_t*)dv, lin, ldo, L, Mblk, Nblk, qk_scale, total_k);
+  hipLaunchKernelGGL((bwd_dkdv_kernel<Tag, D, BLKQ, CONTIG>), dim3(xcd_grid(w.max_items)), dim3(256), 0, st,               \
+                     (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse, delta, list,    \
+                     count, items, totals, part, w.seg, (uint16_t*)dk, (uint16_t*)dv, lin, ldo, L, Mblk, Nblk, qk_scale);
   if (contig) {
     SLA_BWD_LAUNCH(true)
   } else {
     SLA_BWD_LAUNCH(false)
   }
 #undef SLA_BWD_LAUNCH
+  hipLaunchKernelGGL((bwd_dkdv_reduce_kernel<Tag, D>), dim3(Nblk, BH), dim3(256), 0, st, nseg, slot0, part, (uint16_t*)dk,
+                     (uint16_t*)dv, lin, L, Nblk, (int)w.max_slots);
   return check_launch("sparse_attn_bwd");
 }
 

@@ -95,3 +95,31 @@ def test_more_query_blocks_than_one_round_of_the_list_builder(dev):
     for name, a, b in zip(("dq", "dk", "dv"), (dq, dk, dv), refs):
         assert max_abs(a, b) <= TOL_ABS, name
         assert cos_sim(a, b) >= TOL_COS, name
+
+
+@pytest.mark.parametrize("L,D,BLKQ,T,sinks", [(12800, 64, 64, 8, 2), (12790, 128, 128, 6, 1), (9000, 128, 64, 5, 5)])
+def test_key_blocks_selected_by_every_query_block(dev, L, D, BLKQ, T, sinks):
+    """Attention "sinks": a few key blocks are in every look-up row, so their lists hold every query block and are cut
+    into segments whose fp32 partials a second kernel adds; the other key blocks keep short lists."""
+    g = torch.Generator().manual_seed(L + T)
+    q, k, v, do = (torch.randn(1, 2, L, D, generator=g).to(torch.bfloat16) for _ in range(4))
+    M, N = -(-L // BLKQ), -(-L // 64)
+    lut = torch.empty(1, 2, M, T, dtype=torch.int64)
+    for h in range(2):
+        for i in range(M):
+            rest = torch.randperm(N - sinks, generator=g)[:T - sinks] + sinks
+            lut[0, h, i] = torch.cat([torch.arange(sinks), rest]).sort().values
+    m = torch.zeros(1, 2, M, N, dtype=torch.int8).scatter_(-1, lut, 1)
+    assert int(m[0, 0, :, 0].sum()) == M > 64
+    o_ref, lse_ref = O.sparse_attn_fwd_gather(q, k, v, lut, BLKQ, 64)
+    refs = O.sparse_attn_bwd_gather(q, k, v, o_ref, do, lse_ref, lut, BLKQ, 64)
+    o, dq, dk, dv = _grads(q, k, v, do, m, lut, T, BLKQ, dev)
+    for name, a, b in zip(("dq", "dk", "dv"), (dq, dk, dv), refs):
+        # (a sink block's dK / dV rows are sums over all L queries: scale the absolute bound with their size)
+        scale = max(1.0, float(b.abs().max()) / 8)
+        assert max_abs(a, b) <= TOL_ABS * scale, (name, max_abs(a, b), scale)
+        assert cos_sim(a, b) >= TOL_COS, name
+    # the sink rows themselves, separately (they are a small part of the tensor)
+    rows = slice(0, sinks * 64)
+    for a, b in ((dk, refs[1]), (dv, refs[2])):
+        assert cos_sim(a[:, :, rows], b[:, :, rows]) >= TOL_COS
