@@ -32,13 +32,13 @@ def dev():
 
 
 def cos_sim(a, b):
-    a = a.double().flatten()
-    b = b.double().flatten()
+    a = a.detach().double().flatten()
+    b = b.detach().double().flatten()
     return float((a @ b) / (a.norm() * b.norm() + 1e-300))
 
 
 def max_abs(a, b):
-    return float((a.double() - b.double()).abs().max())
+    return float((a.detach().double() - b.detach().double()).abs().max())
 
 
 @pytest.fixture(autouse=True)
