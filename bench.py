@@ -196,6 +196,12 @@ def main():
                 cmod.proj_l.weight.copy_(w)
                 cmod.proj_l.bias.copy_(b)
                 extra["sla_fwd_complement_mode_ms"] = time_region(torch, lambda: cmod(q, k, v), args.steps, args.warmup)
+
+            def cfwd_bwd():
+                o = cmod(qg, kg, vg)
+                o.backward(do)
+                qg.grad = kg.grad = vg.grad = None
+            extra["sla_fwd_bwd_complement_mode_ms"] = time_region(torch, cfwd_bwd, max(args.steps // 2, 1), min(args.warmup, 2))
         except (AssertionError, RuntimeError, NotImplementedError) as e:
             extra["sla_fwd_complement_mode_ms"] = None
             extra["complement_note"] = str(e)[:200]

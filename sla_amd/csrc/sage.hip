@@ -516,7 +516,7 @@ static int prepare_impl(const void* q, const void* k, const void* v, int dtype, 
                      (const uint16_t*)(ws + w.colmean), k8, ks, pk, L, N);
   launch_map_from_pooled(dtype, pq, pk, ws + p.score, BH, M, N, D, topk, sparse_map, lut, lut64, st);
   int rc = check_launch("sage_prepare");
-  if (rc) return rc;
+  if (rc || !v) return rc;
   return quant_v_impl<Tag, D>(v, BH, L, v8, vs, ws, st);
 }
 
@@ -567,8 +567,10 @@ extern "C" int sage_prepare(const void* q, const void* k, const void* v, int dty
   SLA_REQUIRE(N <= 8192, SLA_ERR_UNSUPPORTED, "more than 8192 key blocks (%d)", N);
   SLA_REQUIRE(lut_elem_bytes == 4 || lut_elem_bytes == 8, SLA_ERR_BAD_ARG, "lut_elem_bytes must be 4 or 8, got %d",
               lut_elem_bytes);
-  SLA_REQUIRE(q && k && v && sparse_map && (lut || topk == 0) && q_int8 && q_scale && k_int8 && k_scale && v_fp8 && v_scale &&
-                  workspace,
+  // (v, v_fp8 and v_scale may all three be NULL: the caller then quantises v itself with sage_quant_v, e.g. on another
+  //  stream)
+  SLA_REQUIRE(q && k && sparse_map && (lut || topk == 0) && q_int8 && q_scale && k_int8 && k_scale && workspace &&
+                  ((v && v_fp8 && v_scale) || (!v && !v_fp8 && !v_scale)),
               SLA_ERR_BAD_ARG, "null pointer");
   SLA_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)lut | (uintptr_t)q_int8 | (uintptr_t)k_int8 |
                (uintptr_t)v_fp8 | (uintptr_t)workspace) % 16 == 0,

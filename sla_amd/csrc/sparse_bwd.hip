@@ -117,21 +117,29 @@ __global__ __launch_bounds__(64 * COL_NW) void bwd_col_lists_kernel(const int8_t
 // segment is one work item.  item = {bh, key block, segment, slot}: slot < 0 for a key block with a single segment
 // (the workgroup writes dK / dV itself), otherwise the index of the fp32 partial this segment writes; the partials
 // of a key block occupy consecutive slots and are added in segment order by bwd_dkdv_reduce_kernel.
-// One workgroup of 1024 threads walks all (head, key block) pairs in order with a running prefix sum.
+// One workgroup of 1024 threads walks all (head, key block) pairs in order, eight per thread and round, with a running
+// prefix sum.
 __global__ __launch_bounds__(1024) void bwd_segments_kernel(const int* __restrict__ count, int* __restrict__ nseg,
                                                             int* __restrict__ slot0, i32x4_t* __restrict__ items,
                                                             int* __restrict__ totals, int nblocks, int Nblk, int seg,
                                                             int max_items, int max_slots) {
+  constexpr int EPT = 8;                      // consecutive (head, key block) pairs per thread and round
   __shared__ int wsum[2][16];
   __shared__ int base[2];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   if (tid == 0) base[0] = base[1] = 0;
   __syncthreads();
-  for (int i0 = 0; i0 < nblocks; i0 += 1024) {
-    const int i = i0 + tid;
-    const int ns = i < nblocks ? max(1, (count[i] + seg - 1) / seg) : 0;
-    const int ms = ns > 1 ? ns : 0;
-    int a = ns, b = ms;                       // inclusive scans inside the wave
+  for (int i0 = 0; i0 < nblocks; i0 += 1024 * EPT) {
+    const int first = i0 + tid * EPT;
+    int ns[EPT];
+    int own_a = 0, own_b = 0;
+#pragma unroll
+    for (int e = 0; e < EPT; ++e) {
+      ns[e] = first + e < nblocks ? max(1, (count[first + e] + seg - 1) / seg) : 0;
+      own_a += ns[e];
+      own_b += ns[e] > 1 ? ns[e] : 0;
+    }
+    int a = own_a, b = own_b;                 // inclusive scans inside the wave
 #pragma unroll
     for (int o = 1; o < 64; o <<= 1) {
       const int ta = __shfl_up(a, o), tb = __shfl_up(b, o);
@@ -153,18 +161,25 @@ __global__ __launch_bounds__(1024) void bwd_segments_kernel(const int* __restric
       ta += wsum[0][w];
       tb += wsum[1][w];
     }
-    if (i < nblocks) {
-      const int first_item = base[0] + pa + a - ns, first_slot = base[1] + pb + b - ms;
-      nseg[i] = ns;
-      slot0[i] = first_slot;
-      const int bh = i / Nblk, nb = i - bh * Nblk;
-      // (a map whose rows hold more ones than the topk the workspace was sized for cannot overrun the tables: its
-      //  surplus items are dropped)
-      for (int sg = 0; sg < ns; ++sg)
-        if (first_item + sg < max_items && first_slot + ms <= max_slots)
-          items[first_item + sg] = i32x4_t{bh, nb, sg, ns > 1 ? first_slot + sg : -1};
-        else if (first_item + sg < max_items)
-          items[first_item + sg] = i32x4_t{bh, nb, sg, -2};
+    int first_item = base[0] + pa + a - own_a, first_slot = base[1] + pb + b - own_b;
+#pragma unroll
+    for (int e = 0; e < EPT; ++e) {
+      const int i = first + e;
+      if (i < nblocks) {
+        const int ms = ns[e] > 1 ? ns[e] : 0;
+        nseg[i] = ns[e];
+        slot0[i] = first_slot;
+        const int bh = i / Nblk, nb = i - bh * Nblk;
+        // (a map whose rows hold more ones than the topk the workspace was sized for cannot overrun the tables: its
+        //  surplus items are dropped)
+        for (int sg = 0; sg < ns[e]; ++sg)
+          if (first_item + sg < max_items && first_slot + ms <= max_slots)
+            items[first_item + sg] = i32x4_t{bh, nb, sg, ns[e] > 1 ? first_slot + sg : -1};
+          else if (first_item + sg < max_items)
+            items[first_item + sg] = i32x4_t{bh, nb, sg, -2};
+        first_item += ns[e];
+        first_slot += ms;
+      }
     }
     __syncthreads();
     if (tid == 0) {

@@ -146,6 +146,16 @@ class _StateBuild:
         with torch.cuda.stream(side):
             self.ws = linear_state_fwd(k, v, weight, fmap)
 
+    def also(self, fn, *args):
+        """Runs ``fn(*args)`` behind the state build, on the same side stream; its results are ready after ``join``."""
+        if self.side is None:
+            return fn(*args)
+        with torch.cuda.stream(self.side):
+            res = fn(*args)
+        for t in (res if isinstance(res, tuple) else (res,)):
+            t.record_stream(torch.cuda.current_stream(t.device))
+        return res
+
     def join(self):
         if self.side is not None:
             torch.cuda.current_stream(self.ws.device).wait_stream(self.side)

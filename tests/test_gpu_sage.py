@@ -45,6 +45,10 @@ def test_one_call_preparation_equals_the_separate_calls(dev, L, D, ratio, dtype)
     qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
     m, lut, T, q8, qs, k8, ks, v8, vs = sage_prepare(qd, kd, vd, ratio)
     assert T == T_ref and torch.equal(lut.cpu(), lut_ref) and torch.equal(m.cpu(), m_ref)
+    # without v: the same map and q / k results, the v part left to the caller
+    m3, lut3, T3, q8c, qsc, k8c, ksc, none_a, none_b = sage_prepare(qd, kd, None, ratio)
+    assert none_a is None and none_b is None and T3 == T and torch.equal(lut3, lut) and torch.equal(m3, m)
+    assert torch.equal(q8c, q8) and torch.equal(qsc, qs) and torch.equal(k8c, k8) and torch.equal(ksc, ks)
     m2, lut2, T2 = get_block_map(qd, kd, ratio, 128, 64)
     assert T2 == T and torch.equal(lut2, lut) and torch.equal(m2, m)
     q8b, qsb, k8b, ksb = quant_qk(qd, kd)
