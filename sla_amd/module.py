@@ -206,6 +206,7 @@ class SparseLinearAttention(nn.Module):
             q, k, v: (B, H, L, D).
             return_sparsity: also return real_topk / n_key_blocks (reference core.py:102-103).
         """
+        _lib.require_gpu(q, k, v)          # no CPU path: refuse loudly before anything touches a stream
         dtype = q.dtype
         needs_grad = torch.is_grad_enabled() and any(
             t.requires_grad for t in (q, k, v, self.proj_l.weight, self.proj_l.bias))

@@ -129,6 +129,7 @@ class SageSparseLinearAttention(nn.Module):
 
     @torch.no_grad()
     def forward(self, q, k, v, return_sparsity=False):
+        _lib.require_gpu(q, k, v)          # no CPU path: refuse loudly before anything touches a stream
         dtype = q.dtype
         q = q.contiguous()
         k = k.contiguous()
