@@ -14,24 +14,40 @@ from __future__ import annotations
 import torch.nn as nn
 
 from .module import SparseLinearAttention
+from .sage import SageSparseLinearAttention
 
 
 class SLASelfAttention(nn.Module):
     def __init__(self, dim, num_heads, topk, feature_map="softmax", BLKQ=64, BLKK=64, use_bf16=True, qkv_bias=True,
-                 linear_mode="global"):
+                 linear_mode="global", quantized=False):
+        """``quantized=True`` puts ``SageSparseLinearAttention`` (INT8 / FP8, inference only, 128/64 blocks) in the place
+        of ``SparseLinearAttention``; the parameter names are the same, so a block fine-tuned with the 16-bit operator
+        loads into a quantised one (the pairing the reference's README describes: train with SLA, serve with SageSLA)."""
         super().__init__()
         if dim % num_heads != 0:
             raise ValueError(f"dim {dim} is not a multiple of num_heads {num_heads}")
         self.num_heads = num_heads
         self.head_dim = dim // num_heads
         self.qkv = nn.Linear(dim, 3 * dim, bias=qkv_bias)
-        self.attn = SparseLinearAttention(self.head_dim, topk, feature_map, BLKQ, BLKK, use_bf16=use_bf16,
-                                          linear_mode=linear_mode)
+        self.quantized = quantized
+        if quantized:
+            if linear_mode != "global":
+                raise NotImplementedError("the quantised operator has the global linear branch only")
+            self.attn = SageSparseLinearAttention(self.head_dim, topk, feature_map, use_bf16=use_bf16)
+        else:
+            self.attn = SparseLinearAttention(self.head_dim, topk, feature_map, BLKQ, BLKK, use_bf16=use_bf16,
+                                              linear_mode=linear_mode)
         self.proj = nn.Linear(dim, dim)
 
     def forward(self, x):
         """x: (B, L, dim) -> (B, L, dim)."""
         B, L, C = x.shape
         H, D = self.num_heads, self.head_dim
-        o = self.attn.forward_packed(self.qkv(x).view(B, L, 3, H, D))      # (B, L, H, D)
+        qkv = self.qkv(x).view(B, L, 3, H, D)
+        if self.quantized:
+            # (the quantisers take contiguous (B, H, L, D) tensors: one layout copy in, one out)
+            q, k, v = qkv.permute(2, 0, 3, 1, 4).contiguous()
+            o = self.attn(q, k, v).transpose(1, 2)
+        else:
+            o = self.attn.forward_packed(qkv)                               # (B, L, H, D)
         return self.proj(o.reshape(B, L, C))

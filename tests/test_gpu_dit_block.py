@@ -46,3 +46,24 @@ def test_gradients_reach_all_parameters(dev):
     assert x.grad is not None and torch.isfinite(x.grad.float()).all()
     for n, p in blk.named_parameters():
         assert p.grad is not None and torch.isfinite(p.grad.float()).all() and float(p.grad.float().abs().max()) > 0, n
+
+
+def test_quantised_block_loads_the_16_bit_block_and_agrees(dev):
+    """Train with SLA, serve with SageSLA: same parameter names, outputs agree to the quantised operator's bound
+    (both blocks at 128/64 blocks, so both attend to the same key blocks)."""
+    torch.manual_seed(3)
+    kw = dict(dim=256, num_heads=2, topk=0.25, feature_map="softmax")
+    blk = SLASelfAttention(BLKQ=128, BLKK=64, **kw).to(dev).to(torch.bfloat16)
+    blk.attn.proj_l.float()
+    with torch.no_grad():
+        blk.attn.proj_l.weight.normal_(0, 128 ** -0.5)
+        blk.attn.proj_l.bias.normal_(0, 0.1)
+    qblk = SLASelfAttention(quantized=True, **kw).to(dev).to(torch.bfloat16)
+    qblk.attn.proj_l.float()
+    qblk.load_state_dict(blk.state_dict())
+    x = torch.randn(2, 1000, 256, device=dev, dtype=torch.bfloat16)
+    with torch.no_grad():
+        y, yq = blk(x), qblk(x)
+    assert yq.shape == y.shape and cos_sim(yq.cpu(), y.cpu()) >= 0.995
+    with pytest.raises(NotImplementedError):
+        SLASelfAttention(quantized=True, linear_mode="complement", **kw)
