@@ -231,6 +231,21 @@ int sage_sparse_attn_fwd(const int8_t* q_int8, const float* q_scale, const int8_
                          int lut_elem_bytes, void* o, int out_dtype, int B, int H, int L, int D, int BLKQ,
                          int BLKK, int topk, float qk_scale, void* stream);
 
+/* The SageSLA path on row-contiguous views (same stride convention as the other *_strided entry points):
+ * q, k, v may be (B, L, H, D) activations or slices of a packed projection; the quantised tensors are always written
+ * as contiguous (B, H, L, D), which is what sage_sparse_attn_fwd reads; sla_linear_out_fwd_strided reads q and
+ * writes out where the caller's tensors lie (the residual, i.e. the attention output, is contiguous (B, H, L, D)).
+ * They spare the caller the layout copies of bench_kernel.py:68-71 around the quantised operator. */
+int sage_prepare_strided(const void* q, const void* k, const void* v, const int64_t* qkv_strides, int dtype, int B, int H,
+                         int L, int D, int BLKQ, int BLKK, int topk, int8_t* sparse_map, void* lut, int lut_elem_bytes,
+                         int8_t* q_int8, float* q_scale, int8_t* k_int8, float* k_scale, uint8_t* v_fp8, float* v_scale,
+                         void* workspace, int64_t workspace_bytes, void* stream);
+int sage_quant_v_strided(const void* v, const int64_t* v_strides, int dtype, int B, int H, int L, int D, uint8_t* v_fp8,
+                         float* v_scale, void* workspace, int64_t workspace_bytes, void* stream);
+int sla_linear_out_fwd_strided(const void* q, const int64_t* q_strides, const float* bias, const void* residual, void* out,
+                               const int64_t* out_strides, int dtype, int fmap, int B, int H, int L, int D,
+                               void* workspace, int64_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

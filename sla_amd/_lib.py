@@ -56,6 +56,10 @@ SIGNATURES = {
     "sage_prepare": (_I, [_P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I64, _P]),
     "sage_quant_v": (_I, [_P, _I, _I, _I, _I, _I, _P, _P, _P, _I64, _P]),
     "sage_sparse_attn_fwd": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _P]),
+    "sage_prepare_strided": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I64,
+                                  _P]),
+    "sage_quant_v_strided": (_I, [_P, _P, _I, _I, _I, _I, _I, _P, _P, _P, _I64, _P]),
+    "sla_linear_out_fwd_strided": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I64, _P]),
 }
 
 _lib = None

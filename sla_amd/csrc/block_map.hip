@@ -423,9 +423,9 @@ static void launch_colmean_reduce(float* chunk_sums, float* group_sums, typename
 }
 
 template <typename IO>
-static void launch_k_colmean_t(const void* k, int BH, int L, int D, float* chunk_sums, float* group_sums,
-                               typename IO::raw* colmean, hipStream_t st) {
-  launch_pool<IO, 0>(k, contiguous_layout(BH, L, D), nullptr, chunk_sums, BH, L, D, KMEAN_CHUNK, st);
+static void launch_k_colmean_t(const void* k, const RowLayout& lay, int BH, int L, int D, float* chunk_sums,
+                               float* group_sums, typename IO::raw* colmean, hipStream_t st) {
+  launch_pool<IO, 0>(k, lay, nullptr, chunk_sums, BH, L, D, KMEAN_CHUNK, st);
   launch_colmean_reduce<IO>(chunk_sums, group_sums, colmean, BH, L, D, st);
 }
 
@@ -461,16 +461,17 @@ int64_t k_colmean_scratch_floats(int BH, int L, int D) {
   const int64_t nchunk = cdiv(L, KMEAN_CHUNK), ngroup = cdiv((int)nchunk, KMEAN_GROUP);
   return (int64_t)BH * (nchunk + ngroup) * D;
 }
-void launch_k_colmean(const void* k, int dtype, int BH, int L, int D, float* scratch, void* colmean, hipStream_t st) {
+void launch_k_colmean(const void* k, const RowLayout& lay, int dtype, int BH, int L, int D, float* scratch, void* colmean,
+                      hipStream_t st) {
   const int64_t nchunk = cdiv(L, KMEAN_CHUNK);
   float* chunk_sums = scratch;
   float* group_sums = scratch + (int64_t)BH * nchunk * D;
   if (dtype == SLA_F32)
-    launch_k_colmean_t<IoF32>(k, BH, L, D, chunk_sums, group_sums, (float*)colmean, st);
+    launch_k_colmean_t<IoF32>(k, lay, BH, L, D, chunk_sums, group_sums, (float*)colmean, st);
   else if (dtype == SLA_BF16)
-    launch_k_colmean_t<IoBf16>(k, BH, L, D, chunk_sums, group_sums, (uint16_t*)colmean, st);
+    launch_k_colmean_t<IoBf16>(k, lay, BH, L, D, chunk_sums, group_sums, (uint16_t*)colmean, st);
   else
-    launch_k_colmean_t<IoF16>(k, BH, L, D, chunk_sums, group_sums, (uint16_t*)colmean, st);
+    launch_k_colmean_t<IoF16>(k, lay, BH, L, D, chunk_sums, group_sums, (uint16_t*)colmean, st);
 }
 
 // Scores and top-k selection from block means computed elsewhere (the quantisers of the SageSLA path

@@ -42,11 +42,14 @@ __global__ __launch_bounds__(256) void linear_fold_kernel(const uint16_t* __rest
 
 // ---- kernel 4: output --------------------------------------------------------------------
 // grid (ceil(L / (128*TILES)), BH), 256 threads = 4 waves x 32 queries, TILES steps per workgroup.
-template <typename Tag, int D>
+// CONTIG: q and out are contiguous (B, H, L, D): the row pitch is the compile-time D.
+template <typename Tag, int D, bool CONTIG>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void linear_out_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ kvwt,
                                                          const uint16_t* __restrict__ z, const float* __restrict__ bias,
                                                          const uint16_t* __restrict__ residual, uint16_t* __restrict__ out,
-                                                         int L, int fmap, int tiles_per_wg) {
+                                                         const RowLayout lq, const RowLayout lout, int L, int fmap,
+                                                         int tiles_per_wg) {
+  // (lq, lout: where the rows of q and of out lie; the residual is a contiguous (B, H, L, D) tensor)
   using E = Elem<Tag>;
   constexpr int DC = D / 16;
   constexpr int DT = D / 32;
@@ -74,11 +77,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   }
   __syncthreads();
 
-  const uint16_t* qh = q + (size_t)bh * L * D;
+  const uint16_t* qh = q + (CONTIG ? (size_t)bh * L * D : lq.head(bh));
+  uint16_t* const oh = out + (CONTIG ? (size_t)bh * L * D : lout.head(bh));
+  const size_t pitch_q = CONTIG ? (size_t)D : (size_t)lq.sl, pitch_o = CONTIG ? (size_t)D : (size_t)lout.sl;
   uint16_t* stage = sStage[wave];
   const int first_row = blockIdx.x * tiles_per_wg * 128 + wave * 32;
   TileRows<D> qt;                      // q rows of the tile about to be processed, fetched one tile ahead
-  if (first_row < L) qt.fetch(qh + (size_t)first_row * D, min(32, L - first_row), lane);
+  if (first_row < L) qt.fetch(qh + (size_t)first_row * pitch_q, min(32, L - first_row), lane, pitch_q);
   for (int tt = 0; tt < tiles_per_wg; ++tt) {
     const int row0 = first_row + tt * 128;
     if (row0 >= L) break;
@@ -97,7 +102,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     wave_lds_fence();
     TileRows<D> res;
     if (residual) res.fetch(residual + off, rows_valid, lane);
-    if (tt + 1 < tiles_per_wg && row0 + 128 < L) qt.fetch(qh + (size_t)(row0 + 128) * D, min(32, L - row0 - 128), lane);
+    if (tt + 1 < tiles_per_wg && row0 + 128 < L)
+      qt.fetch(qh + (size_t)(row0 + 128) * pitch_q, min(32, L - row0 - 128), lane, pitch_q);
     float row_mx, row_inv;
     phi_row_pair<Tag, DC>(fmap, f, row_mx, row_inv);
     // divisor: 1e-5 + sum_d round16(fq*z), each step rounded to 16 bit as the reference's tensors are
@@ -131,7 +137,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
       for (int i = 0; i < 16; ++i) val[t][i] = pin_f32(__builtin_fmaf(acc[i], inv_den, sBias[32 * t + 8 * (i >> 2) + 4 * g + (i & 3)]));   // as in the fused epilogue
     }
-    store_acc_tile<E, D>(stage, val, out + off, residual ? &res : nullptr, rows_valid, lane);
+    store_acc_tile<E, D>(stage, val, oh + (size_t)row0 * pitch_o, residual ? &res : nullptr, rows_valid, lane, pitch_o);
   }
 }
 
@@ -150,13 +156,19 @@ static int linear_state_impl(const void* k, const void* v, const RowLayout& lay,
 }
 
 template <typename Tag, int D>
-static int linear_out_impl(const void* q, const float* bias, const void* residual, void* out, int fmap, int BH, int L,
-                           char* ws, hipStream_t st) {
+static int linear_out_impl(const void* q, const RowLayout& lq, const float* bias, const void* residual, void* out,
+                           const RowLayout& lout, int fmap, int BH, int L, char* ws, hipStream_t st) {
   const LinWs w = lin_ws(BH, L, D);
   const int tiles = balanced_tiles(cdiv(L, 128), BH, 2);
-  hipLaunchKernelGGL((linear_out_kernel<Tag, D>), dim3(cdiv(L, 128 * tiles), BH), dim3(256), 0, st, (const uint16_t*)q,
-                     (const uint16_t*)(ws + w.kvwt), (const uint16_t*)(ws + w.z), bias, (const uint16_t*)residual,
-                     (uint16_t*)out, L, fmap, tiles);
+  if (lq.sl == D && lout.sl == D && lq.sh == (int64_t)L * D && lout.sh == (int64_t)L * D && lq.sb == lq.sh * lq.H &&
+      lout.sb == lout.sh * lout.H)
+    hipLaunchKernelGGL((linear_out_kernel<Tag, D, true>), dim3(cdiv(L, 128 * tiles), BH), dim3(256), 0, st, (const uint16_t*)q,
+                       (const uint16_t*)(ws + w.kvwt), (const uint16_t*)(ws + w.z), bias, (const uint16_t*)residual,
+                       (uint16_t*)out, lq, lout, L, fmap, tiles);
+  else
+    hipLaunchKernelGGL((linear_out_kernel<Tag, D, false>), dim3(cdiv(L, 128 * tiles), BH), dim3(256), 0, st, (const uint16_t*)q,
+                       (const uint16_t*)(ws + w.kvwt), (const uint16_t*)(ws + w.z), bias, (const uint16_t*)residual,
+                       (uint16_t*)out, lq, lout, L, fmap, tiles);
   return check_launch("linear_out_fwd");
 }
 
@@ -220,9 +232,15 @@ extern "C" int sla_linear_state_fwd_strided(const void* k, const void* v, const 
   return linear_state_entry(k, v, kv_strides, weight, dtype, fmap, B, H, L, D, workspace, workspace_bytes, stream);
 }
 
-extern "C" int sla_linear_out_fwd(const void* q, const float* bias, const void* residual, void* out, int dtype, int fmap,
-                                  int B, int H, int L, int D, void* workspace, int64_t workspace_bytes, void* stream) {
+static int linear_out_entry(const void* q, const int64_t* q_strides, const float* bias, const void* residual, void* out,
+                            const int64_t* out_strides, int dtype, int fmap, int B, int H, int L, int D, void* workspace,
+                            int64_t workspace_bytes, void* stream) {
   int rc = validate_linear(dtype, fmap, B, H, L, D);
+  if (rc) return rc;
+  RowLayout lq, lout;
+  rc = make_layout(q_strides, B, H, L, D, 2, &lq);
+  if (rc) return rc;
+  rc = make_layout(out_strides, B, H, L, D, 2, &lout);
   if (rc) return rc;
   SLA_REQUIRE(q && bias && out, SLA_ERR_BAD_ARG, "null pointer");
   SLA_REQUIRE(((uintptr_t)q | (uintptr_t)out | (uintptr_t)residual) % 16 == 0, SLA_ERR_BAD_ARG,
@@ -232,7 +250,7 @@ extern "C" int sla_linear_out_fwd(const void* q, const float* bias, const void* 
   if (rc) return rc;
   hipStream_t st = (hipStream_t)stream;
   char* ws = (char*)workspace;
-#define SLA_LIN_CASE(TAG, DD) return linear_out_impl<TAG, DD>(q, bias, residual, out, fmap, BH, L, ws, st)
+#define SLA_LIN_CASE(TAG, DD) return linear_out_impl<TAG, DD>(q, lq, bias, residual, out, lout, fmap, BH, L, ws, st)
   if (dtype == SLA_BF16) {
     if (D == 128) SLA_LIN_CASE(bf16_tag, 128);
     SLA_LIN_CASE(bf16_tag, 64);
@@ -240,6 +258,19 @@ extern "C" int sla_linear_out_fwd(const void* q, const float* bias, const void* 
   if (D == 128) SLA_LIN_CASE(f16_tag, 128);
   SLA_LIN_CASE(f16_tag, 64);
 #undef SLA_LIN_CASE
+}
+
+extern "C" int sla_linear_out_fwd(const void* q, const float* bias, const void* residual, void* out, int dtype, int fmap,
+                                  int B, int H, int L, int D, void* workspace, int64_t workspace_bytes, void* stream) {
+  return linear_out_entry(q, nullptr, bias, residual, out, nullptr, dtype, fmap, B, H, L, D, workspace, workspace_bytes, stream);
+}
+
+extern "C" int sla_linear_out_fwd_strided(const void* q, const int64_t* q_strides, const float* bias, const void* residual,
+                                          void* out, const int64_t* out_strides, int dtype, int fmap, int B, int H, int L,
+                                          int D, void* workspace, int64_t workspace_bytes, void* stream) {
+  SLA_REQUIRE(q_strides && out_strides, SLA_ERR_BAD_ARG, "null strides");
+  return linear_out_entry(q, q_strides, bias, residual, out, out_strides, dtype, fmap, B, H, L, D, workspace, workspace_bytes,
+                          stream);
 }
 
 extern "C" int sla_linear_fwd(const void* q, const void* k, const void* v, const float* weight, const float* bias,

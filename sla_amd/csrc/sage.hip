@@ -15,7 +15,8 @@
 namespace sla {
 
 int64_t k_colmean_scratch_floats(int BH, int L, int D);
-void launch_k_colmean(const void* k, int dtype, int BH, int L, int D, float* scratch, void* colmean, hipStream_t st);
+void launch_k_colmean(const void* k, const RowLayout& lay, int dtype, int BH, int L, int D, float* scratch, void* colmean,
+                      hipStream_t st);
 void launch_map_from_pooled(int dtype, const void* pq, const void* pk, void* score, int BH, int M, int N, int D, int topk,
                             int8_t* sparse_map, void* lut, int lut64, hipStream_t st);
 
@@ -25,9 +26,10 @@ void launch_map_from_pooled(int dtype, const void* pq, const void* pk, void* sco
 // get_block_map pools it: utils.py:55-58 of the reference), summed row by row in fp32 and divided once,
 // exactly as the pooling kernel of the mask builder does, so the block is read from memory once for both.
 template <typename Tag, int D, int BLK, bool SUB_MEAN, bool POOL>
-__global__ __launch_bounds__(256) void quant_int8_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ colmean,
-                                                         int8_t* __restrict__ xq, float* __restrict__ scale,
-                                                         uint16_t* __restrict__ pooled, int L, int nblk) {
+__global__ __launch_bounds__(256) void quant_int8_kernel(const uint16_t* __restrict__ x, const RowLayout lay,
+                                                         const uint16_t* __restrict__ colmean, int8_t* __restrict__ xq,
+                                                         float* __restrict__ scale, uint16_t* __restrict__ pooled, int L,
+                                                         int nblk) {
   using E = Elem<Tag>;
   constexpr int CPR = D / 8;
   constexpr int RPP = 256 / CPR;
@@ -53,7 +55,7 @@ __global__ __launch_bounds__(256) void quant_int8_kernel(const uint16_t* __restr
     const int grow = blk * BLK + lrow + p * RPP;
     i16x8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
     const bool ok = grow < L;
-    if (ok) v = *reinterpret_cast<const i16x8_t*>(x + ((size_t)bh * L + grow) * D + lcol);
+    if (ok) v = *reinterpret_cast<const i16x8_t*>(x + lay.head(bh) + (size_t)grow * (size_t)lay.sl + lcol);
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       val[p][e] = ok ? E::to_float((uint16_t)v[e]) - cm[e] : 0.f;
@@ -110,8 +112,8 @@ __global__ __launch_bounds__(256) void quant_int8_kernel(const uint16_t* __restr
 // pass 1: per (chunk of 256 rows, bh) column abs-max -> partial; pass 2: reduce partials;
 // pass 3: v_fp8 = e4m3(v / scale).
 template <typename Tag, int D>
-__global__ __launch_bounds__(256) void v_amax_partial_kernel(const uint16_t* __restrict__ v, float* __restrict__ part, int L,
-                                                             int rows_per_chunk) {
+__global__ __launch_bounds__(256) void v_amax_partial_kernel(const uint16_t* __restrict__ v, const RowLayout lay,
+                                                             float* __restrict__ part, int L, int rows_per_chunk) {
   using E = Elem<Tag>;
   constexpr int CPR = D / 8;
   constexpr int RPP = 256 / CPR;
@@ -124,7 +126,7 @@ __global__ __launch_bounds__(256) void v_amax_partial_kernel(const uint16_t* __r
 #pragma unroll
   for (int e = 0; e < 8; ++e) am[e] = 0.f;
   for (int row = chunk * rows_per_chunk + lrow; row < r_end; row += RPP) {
-    const i16x8_t x = *reinterpret_cast<const i16x8_t*>(v + ((size_t)bh * L + row) * D + lcol);
+    const i16x8_t x = *reinterpret_cast<const i16x8_t*>(v + lay.head(bh) + (size_t)row * (size_t)lay.sl + lcol);
 #pragma unroll
     for (int e = 0; e < 8; ++e) am[e] = fmaxf(am[e], fabsf(E::to_float((uint16_t)x[e])));
   }
@@ -163,8 +165,8 @@ static __device__ __forceinline__ uint32_t cvt4_fp8(float a, float b, float c, f
 }
 
 template <typename Tag, int D>
-__global__ __launch_bounds__(256) void v_quant_fp8_kernel(const uint16_t* __restrict__ v, const float* __restrict__ v_scale,
-                                                          uint8_t* __restrict__ v8, int L) {
+__global__ __launch_bounds__(256) void v_quant_fp8_kernel(const uint16_t* __restrict__ v, const RowLayout lay,
+                                                          const float* __restrict__ v_scale, uint8_t* __restrict__ v8, int L) {
   using E = Elem<Tag>;
   constexpr int CPR = D / 8;
   constexpr int RPP = 256 / CPR;
@@ -172,7 +174,7 @@ __global__ __launch_bounds__(256) void v_quant_fp8_kernel(const uint16_t* __rest
   const int row = blockIdx.x * RPP + threadIdx.x / CPR;
   const int lcol = (threadIdx.x % CPR) * 8;
   if (row >= L) return;
-  const i16x8_t x = *reinterpret_cast<const i16x8_t*>(v + ((size_t)bh * L + row) * D + lcol);
+  const i16x8_t x = *reinterpret_cast<const i16x8_t*>(v + lay.head(bh) + (size_t)row * (size_t)lay.sl + lcol);
   float f[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) f[e] = E::to_float((uint16_t)x[e]) / v_scale[(size_t)bh * D + lcol + e];
@@ -486,10 +488,11 @@ static int quant_qk_impl(const void* q, const void* k, int dtype, int BH, int L,
                          float* ks, char* ws, hipStream_t st) {
   const SageWs w = sage_ws(BH, L, D);
   const int M = cdiv(L, 128), N = cdiv(L, 64);
-  launch_k_colmean(k, dtype, BH, L, D, (float*)(ws + w.chunk_sums), ws + w.colmean, st);
-  hipLaunchKernelGGL((quant_int8_kernel<Tag, D, 128, false, false>), dim3(M, BH), dim3(256), 0, st, (const uint16_t*)q, nullptr,
-                     q8, qs, nullptr, L, M);
-  hipLaunchKernelGGL((quant_int8_kernel<Tag, D, 64, true, false>), dim3(N, BH), dim3(256), 0, st, (const uint16_t*)k,
+  const RowLayout lay = contiguous_layout(BH, L, D);
+  launch_k_colmean(k, lay, dtype, BH, L, D, (float*)(ws + w.chunk_sums), ws + w.colmean, st);
+  hipLaunchKernelGGL((quant_int8_kernel<Tag, D, 128, false, false>), dim3(M, BH), dim3(256), 0, st, (const uint16_t*)q, lay,
+                     nullptr, q8, qs, nullptr, L, M);
+  hipLaunchKernelGGL((quant_int8_kernel<Tag, D, 64, true, false>), dim3(N, BH), dim3(256), 0, st, (const uint16_t*)k, lay,
                      (const uint16_t*)(ws + w.colmean), k8, ks, nullptr, L, N);
   return check_launch("sage_quant_qk");
 }
@@ -498,10 +501,12 @@ static int quant_qk_impl(const void* q, const void* k, int dtype, int BH, int L,
 // and the quantiser both subtract it) and the quantisers emit the block means the scores are made of, so
 // q is read once and k twice instead of q twice and k four times.
 template <typename Tag, int D>
-static int quant_v_impl(const void* v, int BH, int L, uint8_t* v8, float* vs, char* ws, hipStream_t st);
+static int quant_v_impl(const void* v, const RowLayout& lay, int BH, int L, uint8_t* v8, float* vs, char* ws, hipStream_t st);
 
+// (lay: where the rows of q, k, v lie; the quantised outputs are always contiguous (B, H, L, D))
 template <typename Tag, int D>
-static int prepare_impl(const void* q, const void* k, const void* v, int dtype, int BH, int L, int topk, int8_t* sparse_map,
+static int prepare_impl(const void* q, const void* k, const void* v, const RowLayout& lay, int dtype, int BH, int L, int topk,
+                        int8_t* sparse_map,
                         void* lut, int lut64, int8_t* q8, float* qs, int8_t* k8, float* ks, uint8_t* v8, float* vs, char* ws,
                         hipStream_t st) {
   const SageWs w = sage_ws(BH, L, D);
@@ -509,26 +514,27 @@ static int prepare_impl(const void* q, const void* k, const void* v, int dtype, 
   const int M = cdiv(L, 128), N = cdiv(L, 64);
   uint16_t* pq = (uint16_t*)(ws + p.pq);
   uint16_t* pk = (uint16_t*)(ws + p.pk);
-  launch_k_colmean(k, dtype, BH, L, D, (float*)(ws + w.chunk_sums), ws + w.colmean, st);
-  hipLaunchKernelGGL((quant_int8_kernel<Tag, D, 128, false, true>), dim3(M, BH), dim3(256), 0, st, (const uint16_t*)q, nullptr,
-                     q8, qs, pq, L, M);
-  hipLaunchKernelGGL((quant_int8_kernel<Tag, D, 64, true, true>), dim3(N, BH), dim3(256), 0, st, (const uint16_t*)k,
+  launch_k_colmean(k, lay, dtype, BH, L, D, (float*)(ws + w.chunk_sums), ws + w.colmean, st);
+  hipLaunchKernelGGL((quant_int8_kernel<Tag, D, 128, false, true>), dim3(M, BH), dim3(256), 0, st, (const uint16_t*)q, lay,
+                     nullptr, q8, qs, pq, L, M);
+  hipLaunchKernelGGL((quant_int8_kernel<Tag, D, 64, true, true>), dim3(N, BH), dim3(256), 0, st, (const uint16_t*)k, lay,
                      (const uint16_t*)(ws + w.colmean), k8, ks, pk, L, N);
   launch_map_from_pooled(dtype, pq, pk, ws + p.score, BH, M, N, D, topk, sparse_map, lut, lut64, st);
   int rc = check_launch("sage_prepare");
   if (rc || !v) return rc;
-  return quant_v_impl<Tag, D>(v, BH, L, v8, vs, ws, st);
+  return quant_v_impl<Tag, D>(v, lay, BH, L, v8, vs, ws, st);
 }
 
 template <typename Tag, int D>
-static int quant_v_impl(const void* v, int BH, int L, uint8_t* v8, float* vs, char* ws, hipStream_t st) {
+static int quant_v_impl(const void* v, const RowLayout& lay, int BH, int L, uint8_t* v8, float* vs, char* ws, hipStream_t st) {
   const SageWs w = sage_ws(BH, L, D);
   float* part = (float*)(ws + w.v_part);
-  hipLaunchKernelGGL((v_amax_partial_kernel<Tag, D>), dim3(w.nchunk_v, BH), dim3(256), 0, st, (const uint16_t*)v, part, L,
+  hipLaunchKernelGGL((v_amax_partial_kernel<Tag, D>), dim3(w.nchunk_v, BH), dim3(256), 0, st, (const uint16_t*)v, lay, part, L,
                      w.rows_per_chunk_v);
   hipLaunchKernelGGL(v_scale_kernel, dim3(BH), dim3(1024), 0, st, part, vs, w.nchunk_v, D);
   constexpr int RPP = 256 / (D / 8);
-  hipLaunchKernelGGL((v_quant_fp8_kernel<Tag, D>), dim3(cdiv(L, RPP), BH), dim3(256), 0, st, (const uint16_t*)v, vs, v8, L);
+  hipLaunchKernelGGL((v_quant_fp8_kernel<Tag, D>), dim3(cdiv(L, RPP), BH), dim3(256), 0, st, (const uint16_t*)v, lay, vs, v8,
+                     L);
   return check_launch("sage_quant_v");
 }
 
@@ -556,11 +562,14 @@ extern "C" int sage_quant_qk(const void* q, const void* k, int dtype, int B, int
   return quant_qk_impl<f16_tag, 64>(q, k, dtype, BH, L, q_int8, q_scale, k_int8, k_scale, ws, st);
 }
 
-extern "C" int sage_prepare(const void* q, const void* k, const void* v, int dtype, int B, int H, int L, int D, int BLKQ,
-                            int BLKK, int topk, int8_t* sparse_map, void* lut, int lut_elem_bytes, int8_t* q_int8,
-                            float* q_scale, int8_t* k_int8, float* k_scale, uint8_t* v_fp8, float* v_scale, void* workspace,
-                            int64_t workspace_bytes, void* stream) {
+static int prepare_entry(const void* q, const void* k, const void* v, const int64_t* qkv_strides, int dtype, int B, int H, int L,
+                         int D, int BLKQ, int BLKK, int topk, int8_t* sparse_map, void* lut, int lut_elem_bytes, int8_t* q_int8,
+                         float* q_scale, int8_t* k_int8, float* k_scale, uint8_t* v_fp8, float* v_scale, void* workspace,
+                         int64_t workspace_bytes, void* stream) {
   int rc = validate_sage(dtype, B, H, L, D, BLKQ, BLKK);
+  if (rc) return rc;
+  RowLayout lay;
+  rc = make_layout(qkv_strides, B, H, L, D, 2, &lay);
   if (rc) return rc;
   const int N = cdiv(L, 64);
   SLA_REQUIRE(topk >= 0 && topk <= N, SLA_ERR_BAD_ARG, "topk=%d outside [0, %d]", topk, N);
@@ -582,8 +591,8 @@ extern "C" int sage_prepare(const void* q, const void* k, const void* v, int dty
   char* ws = (char*)workspace;
   const int lut64 = lut_elem_bytes == 8;
 #define SLA_PREP_CASE(TAG, DD) \
-  return prepare_impl<TAG, DD>(q, k, v, dtype, BH, L, topk, sparse_map, lut, lut64, q_int8, q_scale, k_int8, k_scale, v_fp8, \
-                               v_scale, ws, st)
+  return prepare_impl<TAG, DD>(q, k, v, lay, dtype, BH, L, topk, sparse_map, lut, lut64, q_int8, q_scale, k_int8, k_scale, \
+                               v_fp8, v_scale, ws, st)
   if (dtype == SLA_BF16) {
     if (D == 128) SLA_PREP_CASE(bf16_tag, 128);
     SLA_PREP_CASE(bf16_tag, 64);
@@ -593,9 +602,29 @@ extern "C" int sage_prepare(const void* q, const void* k, const void* v, int dty
 #undef SLA_PREP_CASE
 }
 
-extern "C" int sage_quant_v(const void* v, int dtype, int B, int H, int L, int D, uint8_t* v_fp8, float* v_scale,
-                            void* workspace, int64_t workspace_bytes, void* stream) {
+extern "C" int sage_prepare(const void* q, const void* k, const void* v, int dtype, int B, int H, int L, int D, int BLKQ,
+                            int BLKK, int topk, int8_t* sparse_map, void* lut, int lut_elem_bytes, int8_t* q_int8,
+                            float* q_scale, int8_t* k_int8, float* k_scale, uint8_t* v_fp8, float* v_scale, void* workspace,
+                            int64_t workspace_bytes, void* stream) {
+  return prepare_entry(q, k, v, nullptr, dtype, B, H, L, D, BLKQ, BLKK, topk, sparse_map, lut, lut_elem_bytes, q_int8, q_scale,
+                       k_int8, k_scale, v_fp8, v_scale, workspace, workspace_bytes, stream);
+}
+
+extern "C" int sage_prepare_strided(const void* q, const void* k, const void* v, const int64_t* qkv_strides, int dtype, int B,
+                                    int H, int L, int D, int BLKQ, int BLKK, int topk, int8_t* sparse_map, void* lut,
+                                    int lut_elem_bytes, int8_t* q_int8, float* q_scale, int8_t* k_int8, float* k_scale,
+                                    uint8_t* v_fp8, float* v_scale, void* workspace, int64_t workspace_bytes, void* stream) {
+  SLA_REQUIRE(qkv_strides, SLA_ERR_BAD_ARG, "null strides");
+  return prepare_entry(q, k, v, qkv_strides, dtype, B, H, L, D, BLKQ, BLKK, topk, sparse_map, lut, lut_elem_bytes, q_int8,
+                       q_scale, k_int8, k_scale, v_fp8, v_scale, workspace, workspace_bytes, stream);
+}
+
+static int quant_v_entry(const void* v, const int64_t* v_strides, int dtype, int B, int H, int L, int D, uint8_t* v_fp8,
+                         float* v_scale, void* workspace, int64_t workspace_bytes, void* stream) {
   int rc = validate_sage(dtype, B, H, L, D, 128, 64);
+  if (rc) return rc;
+  RowLayout lay;
+  rc = make_layout(v_strides, B, H, L, D, 2, &lay);
   if (rc) return rc;
   SLA_REQUIRE(v && v_fp8 && v_scale && workspace, SLA_ERR_BAD_ARG, "null pointer");
   SLA_REQUIRE(((uintptr_t)v | (uintptr_t)v_fp8 | (uintptr_t)workspace) % 16 == 0, SLA_ERR_BAD_ARG,
@@ -605,11 +634,22 @@ extern "C" int sage_quant_v(const void* v, int dtype, int B, int H, int L, int D
   hipStream_t st = (hipStream_t)stream;
   char* ws = (char*)workspace;
   if (dtype == SLA_BF16) {
-    if (D == 128) return quant_v_impl<bf16_tag, 128>(v, BH, L, v_fp8, v_scale, ws, st);
-    return quant_v_impl<bf16_tag, 64>(v, BH, L, v_fp8, v_scale, ws, st);
+    if (D == 128) return quant_v_impl<bf16_tag, 128>(v, lay, BH, L, v_fp8, v_scale, ws, st);
+    return quant_v_impl<bf16_tag, 64>(v, lay, BH, L, v_fp8, v_scale, ws, st);
   }
-  if (D == 128) return quant_v_impl<f16_tag, 128>(v, BH, L, v_fp8, v_scale, ws, st);
-  return quant_v_impl<f16_tag, 64>(v, BH, L, v_fp8, v_scale, ws, st);
+  if (D == 128) return quant_v_impl<f16_tag, 128>(v, lay, BH, L, v_fp8, v_scale, ws, st);
+  return quant_v_impl<f16_tag, 64>(v, lay, BH, L, v_fp8, v_scale, ws, st);
+}
+
+extern "C" int sage_quant_v(const void* v, int dtype, int B, int H, int L, int D, uint8_t* v_fp8, float* v_scale,
+                            void* workspace, int64_t workspace_bytes, void* stream) {
+  return quant_v_entry(v, nullptr, dtype, B, H, L, D, v_fp8, v_scale, workspace, workspace_bytes, stream);
+}
+
+extern "C" int sage_quant_v_strided(const void* v, const int64_t* v_strides, int dtype, int B, int H, int L, int D,
+                                    uint8_t* v_fp8, float* v_scale, void* workspace, int64_t workspace_bytes, void* stream) {
+  SLA_REQUIRE(v_strides, SLA_ERR_BAD_ARG, "null strides");
+  return quant_v_entry(v, v_strides, dtype, B, H, L, D, v_fp8, v_scale, workspace, workspace_bytes, stream);
 }
 
 extern "C" int sage_sparse_attn_fwd(const int8_t* q_int8, const float* q_scale, const int8_t* k_int8,

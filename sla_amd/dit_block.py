@@ -45,9 +45,10 @@ class SLASelfAttention(nn.Module):
         H, D = self.num_heads, self.head_dim
         qkv = self.qkv(x).view(B, L, 3, H, D)
         if self.quantized:
-            # (the quantisers take contiguous (B, H, L, D) tensors: one layout copy in, one out)
-            q, k, v = qkv.permute(2, 0, 3, 1, 4).contiguous()
-            o = self.attn(q, k, v).transpose(1, 2)
+            # (B, H, L, D) views of the packed projection: the quantisers read them where they lie and the output
+            # comes back in (B, L, H, D) memory order
+            q, k, v = (qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+            o = self.attn(q, k, v).permute(0, 2, 1, 3)
         else:
             o = self.attn.forward_packed(qkv)                               # (B, L, H, D)
         return self.proj(o.reshape(B, L, C))

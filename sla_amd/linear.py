@@ -44,14 +44,25 @@ def linear_state_fwd(k, v, weight, fmap: str):
 
 
 def linear_out_fwd(q, bias, residual, state_ws, fmap: str):
-    """Second half of :func:`linear_fwd`: ``residual + proj(phi(q) state / divisor)``."""
+    """Second half of :func:`linear_fwd`: ``residual + proj(phi(q) state / divisor)``.
+
+    ``q`` may be a row-contiguous view (see ``_lib.row_strided``); the output then has q's memory order.
+    ``residual`` is always a contiguous (B, H, L, D) tensor."""
     _lib.require_gpu(q, bias, state_ws)
     B, H, L, D = q.shape
     dt = _lib.dtype_code(q.dtype)
-    out = torch.empty_like(q)
-    rc = _lib.load().sla_linear_out_fwd(q.data_ptr(), bias.data_ptr(), 0 if residual is None else residual.data_ptr(),
-                                        out.data_ptr(), dt, _lib.FMAP[fmap], B, H, L, D, state_ws.data_ptr(),
-                                        state_ws.numel(), _lib.stream_ptr(q.device))
+    res_ptr = 0 if residual is None else residual.data_ptr()
+    assert residual is None or residual.is_contiguous()
+    if q.is_contiguous():
+        out = torch.empty_like(q)
+        rc = _lib.load().sla_linear_out_fwd(q.data_ptr(), bias.data_ptr(), res_ptr, out.data_ptr(), dt, _lib.FMAP[fmap], B, H,
+                                            L, D, state_ws.data_ptr(), state_ws.numel(), _lib.stream_ptr(q.device))
+    else:
+        assert _lib.row_strided(q), "q must be contiguous or a row-contiguous view"
+        out = _lib.empty_like_rows(q)
+        rc = _lib.load().sla_linear_out_fwd_strided(q.data_ptr(), _lib.strides_arg(q), bias.data_ptr(), res_ptr, out.data_ptr(),
+                                                    _lib.strides_arg(out), dt, _lib.FMAP[fmap], B, H, L, D,
+                                                    state_ws.data_ptr(), state_ws.numel(), _lib.stream_ptr(q.device))
     _lib.check(rc)
     return out
 

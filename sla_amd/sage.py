@@ -36,21 +36,28 @@ def quant_qk(q, k):
 
 
 def quant_v(v):
-    """Per-channel FP8 e4m3 v.  Returns (v_fp8 (B,H,L,D) float8_e4m3fn, v_scale (B,H,D) fp32)."""
+    """Per-channel FP8 e4m3 v (contiguous or a row-contiguous view).  Returns (v_fp8 (B,H,L,D) float8_e4m3fn, contiguous,
+    v_scale (B,H,D) fp32)."""
     _lib.require_gpu(v)
     B, H, L, D = v.shape
     dt = _lib.dtype_code(v.dtype)
     ws = _lib.workspace(_lib.WS_SAGE_QUANT, dt, B, H, L, D, SAGE_BLKQ, SAGE_BLKK, 0, v.device)
     v8 = torch.empty((B, H, L, D), dtype=torch.float8_e4m3fn, device=v.device)
     vs = torch.empty((B, H, D), dtype=torch.float32, device=v.device)
-    rc = _lib.load().sage_quant_v(v.data_ptr(), dt, B, H, L, D, v8.data_ptr(), vs.data_ptr(), ws.data_ptr(), ws.numel(),
-                                  _lib.stream_ptr(v.device))
+    if v.is_contiguous():
+        rc = _lib.load().sage_quant_v(v.data_ptr(), dt, B, H, L, D, v8.data_ptr(), vs.data_ptr(), ws.data_ptr(), ws.numel(),
+                                      _lib.stream_ptr(v.device))
+    else:
+        assert _lib.row_strided(v), "v must be contiguous or a row-contiguous view"
+        rc = _lib.load().sage_quant_v_strided(v.data_ptr(), _lib.strides_arg(v), dt, B, H, L, D, v8.data_ptr(), vs.data_ptr(),
+                                              ws.data_ptr(), ws.numel(), _lib.stream_ptr(v.device))
     _lib.check(rc)
     return v8, vs
 
 
 def sage_prepare(q, k, v, topk_ratio):
-    """Block map, INT8 q / k and FP8 v in one library call (q, k, v already in the compute dtype).
+    """Block map, INT8 q / k and FP8 v in one library call (q, k, v already in the compute dtype; contiguous, or
+    row-contiguous views with common strides: the quantised tensors are contiguous (B, H, L, D) either way).
 
     Returns ``(sparse_map, lut, T, q_int8, q_scale, k_int8, k_scale, v_fp8, v_scale)``, identical to
     ``get_block_map`` + ``quant_qk`` + ``quant_v`` on the same tensors; the k column mean and the block
@@ -58,10 +65,13 @@ def sage_prepare(q, k, v, topk_ratio):
     v part is left out (``v_fp8`` and ``v_scale`` are returned as None) for a caller that runs ``quant_v`` elsewhere.
     """
     _lib.require_gpu(q, k)
-    assert q.is_contiguous() and k.is_contiguous() and q.shape == k.shape and q.dtype == k.dtype
+    tensors = (q, k) if v is None else (q, k, v)
+    contiguous = all(t.is_contiguous() for t in tensors)
+    assert contiguous or _lib.row_strided(*tensors), "q, k, v must be contiguous or share row-contiguous strides"
+    assert q.shape == k.shape and q.dtype == k.dtype
     if v is not None:
         _lib.require_gpu(v)
-        assert v.is_contiguous() and v.shape == q.shape and v.dtype == q.dtype
+        assert v.shape == q.shape and v.dtype == q.dtype
     B, H, L, D = q.shape
     dt = _lib.dtype_code(q.dtype)
     M, N = (L + SAGE_BLKQ - 1) // SAGE_BLKQ, (L + SAGE_BLKK - 1) // SAGE_BLKK
@@ -78,10 +88,14 @@ def sage_prepare(q, k, v, topk_ratio):
     if v is not None:
         v8 = torch.empty((B, H, L, D), dtype=torch.float8_e4m3fn, device=dev)
         vs = torch.empty((B, H, D), dtype=torch.float32, device=dev)
-    rc = _lib.load().sage_prepare(q.data_ptr(), k.data_ptr(), None if v is None else v.data_ptr(), dt, B, H, L, D, SAGE_BLKQ,
-                                  SAGE_BLKK, T, sparse_map.data_ptr(), lut.data_ptr(), 8, q8.data_ptr(), qs.data_ptr(),
-                                  k8.data_ptr(), ks.data_ptr(), None if v is None else v8.data_ptr(),
-                                  None if v is None else vs.data_ptr(), ws.data_ptr(), ws.numel(), _lib.stream_ptr(dev))
+    tail = (dt, B, H, L, D, SAGE_BLKQ, SAGE_BLKK, T, sparse_map.data_ptr(), lut.data_ptr(), 8, q8.data_ptr(), qs.data_ptr(),
+            k8.data_ptr(), ks.data_ptr(), None if v is None else v8.data_ptr(), None if v is None else vs.data_ptr(),
+            ws.data_ptr(), ws.numel(), _lib.stream_ptr(dev))
+    vp = None if v is None else v.data_ptr()
+    if contiguous:
+        rc = _lib.load().sage_prepare(q.data_ptr(), k.data_ptr(), vp, *tail)
+    else:
+        rc = _lib.load().sage_prepare_strided(q.data_ptr(), k.data_ptr(), vp, _lib.strides_arg(q), *tail)
     _lib.check(rc)
     return sparse_map, lut, T, q8, qs, k8, ks, v8, vs
 
@@ -131,9 +145,13 @@ class SageSparseLinearAttention(nn.Module):
     def forward(self, q, k, v, return_sparsity=False):
         _lib.require_gpu(q, k, v)          # no CPU path: refuse loudly before anything touches a stream
         dtype = q.dtype
-        q = q.contiguous()
-        k = k.contiguous()
-        v = v.contiguous()
+        # (B, L, H, D) activations or slices of a packed projection, viewed as (B, H, L, D), are read where they lie
+        # and the output is written in the same order; anything else is copied as in the reference (core.py:85-87)
+        in_place = (q.dtype == k.dtype == v.dtype == self.dtype and _lib.row_strided(q, k, v))
+        if not in_place:
+            q = q.contiguous()
+            k = k.contiguous()
+            v = v.contiguous()
         headdim = q.size(-1)
         assert headdim in [64, 128], "headdim should be in [64, 128]. For other headdim, you can use padding and specify the softmax scale."
         # The k/v half of the linear branch runs on a side stream beside the preparation and the attention

@@ -120,7 +120,18 @@ def test_other_entry_points_validate():
     assert lib.sla_sparse_attn_linear_fwd_strided(FAKE, FAKE, FAKE, st(65536, 128, 256), FAKE, 8, FAKE, 1 << 30, FAKE, None,
                                                   FAKE, st(65536, 128, 4), FAKE, 1, 0, 1, 2, 256, 128, 64, 64, 1, 0.1,
                                                   None) == _lib.ERR_BAD_ARG
+    assert lib.sla_linear_out_fwd_strided(FAKE, st(65536, 128, 256), FAKE, None, FAKE, st(65536, 128, 100), 1, 0, 1, 2, 256, 128,
+                                          FAKE, 1 << 30, None) == _lib.ERR_BAD_ARG
+    assert lib.sla_linear_out_fwd_strided(FAKE, None, FAKE, None, FAKE, st(65536, 128, 256), 1, 0, 1, 2, 256, 128, FAKE, 1 << 30,
+                                          None) == _lib.ERR_BAD_ARG and "strides" in _lib.last_error()
+    assert lib.sage_quant_v_strided(FAKE, st(65536, 128, 260), 1, 1, 2, 256, 128, FAKE, FAKE, FAKE, 1 << 30,
+                                    None) == _lib.ERR_BAD_ARG and "16-byte" in _lib.last_error()
+    assert lib.sage_prepare_strided(FAKE, FAKE, None, st(65536, 128, 64), 1, 1, 2, 256, 128, 128, 64, 1, FAKE, FAKE, 8, FAKE, FAKE,
+                                    FAKE, FAKE, None, None, FAKE, 1 << 30, None) == _lib.ERR_BAD_ARG
     # one-call SageSLA preparation: block sizes, topk range and workspace are checked before any launch
+    # (v and its two outputs may be left out together, not separately)
+    assert lib.sage_prepare(FAKE, FAKE, None, 1, 1, 1, 256, 128, 128, 64, 2, FAKE, FAKE, 8, FAKE, FAKE, FAKE, FAKE, FAKE, None,
+                            FAKE, 1 << 30, None) == _lib.ERR_BAD_ARG
     prep = lambda BLKQ, topk, ws: lib.sage_prepare(FAKE, FAKE, FAKE, 1, 1, 1, 256, 128, BLKQ, 64, topk, FAKE, FAKE, 8, FAKE,  # noqa: E731
                                                    FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, ws, None)
     assert prep(64, 1, 1 << 30) == _lib.ERR_UNSUPPORTED

@@ -107,3 +107,43 @@ def test_packed_training_equals_the_contiguous_route(dev, B, H, L, D, BLKQ, fmap
     # inference through the same entry
     with torch.no_grad():
         assert torch.equal(mod.forward_packed(qkv), out.detach())
+
+
+@pytest.mark.parametrize("kind", ["blhd", "packed"])
+@pytest.mark.parametrize("B,H,L,D,fmap,dtype", [(2, 3, 700, 128, "elu", torch.bfloat16), (1, 2, 333, 64, "softmax", torch.float16)])
+def test_quantised_module_reads_views_in_place(dev, kind, B, H, L, D, fmap, dtype):
+    """SageSLA on (B, L, H, D) activations / packed projections viewed as (B, H, L, D): bit for bit what the contiguous
+    copies give (quantisers, state build and output kernel all read the views), output in the views' memory order."""
+    from sla_amd import SageSparseLinearAttention
+    from sla_amd.sage import quant_v, sage_prepare
+    q, k, v = _views(kind, B, H, L, D, dtype, dev, L + 1)
+    mod = SageSparseLinearAttention(D, 0.3, fmap, use_bf16=dtype == torch.bfloat16).to(dev)
+    w, b = make_proj(D)
+    with torch.no_grad():
+        mod.proj_l.weight.copy_(w)
+        mod.proj_l.bias.copy_(b)
+        ref = mod(q.contiguous(), k.contiguous(), v.contiguous())
+        out = mod(q, k, v)
+    assert out.shape == ref.shape and torch.equal(out, ref)
+    assert out.permute(0, 2, 1, 3).is_contiguous()
+    # the pieces: one-call preparation and the separate v quantiser on views
+    a = sage_prepare(q, k, v, 0.3)
+    c = sage_prepare(q.contiguous(), k.contiguous(), v.contiguous(), 0.3)
+    for x, y in zip(a, c):
+        assert x == y if isinstance(x, int) else torch.equal(x.view(torch.uint8) if x.dtype == torch.float8_e4m3fn else x,
+                                                             y.view(torch.uint8) if y.dtype == torch.float8_e4m3fn else y)
+    v8, vs = quant_v(v)
+    assert torch.equal(v8.view(torch.uint8), c[7].view(torch.uint8)) and torch.equal(vs, c[8])
+
+
+def test_quantised_block_inference_equals_block_with_copies(dev):
+    torch.manual_seed(5)
+    blk = SLASelfAttention(dim=256, num_heads=2, topk=0.25, feature_map="relu", quantized=True).to(dev).to(torch.bfloat16)
+    blk.attn.proj_l.float()
+    with torch.no_grad():
+        blk.attn.proj_l.weight.normal_(0, 128 ** -0.5)
+        x = torch.randn(2, 640, 256, device=dev, dtype=torch.bfloat16)
+        y = blk(x)
+        q, k, v = blk.qkv(x).view(2, 640, 3, 2, 128).permute(2, 0, 3, 1, 4).contiguous()
+        y_ref = blk.proj(blk.attn(q, k, v).transpose(1, 2).reshape(2, 640, 256))
+    assert torch.equal(y, y_ref)
