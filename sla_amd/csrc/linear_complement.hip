@@ -87,14 +87,25 @@ __global__ __launch_bounds__(256) void complement_total_kernel(const float* __re
 // `at(i)` is the block index of list entry i (`count` entries, subtracted in list order).  Two listed
 // states are in flight while a third is being subtracted (the gather is latency-bound: bytes in flight per
 // compute unit set its rate).
+// When the list names every block (`count == nblocks`) the difference is exactly zero by definition; it is
+// returned as such instead of as the rounding residue of two fp32 sums formed in different orders, which the
+// 1e-5 of the divisor would otherwise turn into an arbitrary result.
 template <typename Tag, int D, typename At>
 static __device__ __forceinline__ void gather_complement(float (&acc)[D * D / 8 / 256][8], float& zacc,
                                                          const float* __restrict__ total, const float* __restrict__ ztotal,
                                                          const uint16_t* __restrict__ blocks, const float* __restrict__ zblocks,
-                                                         int count, At at, int tid) {
+                                                         int count, int nblocks, At at, int tid) {
   using E = Elem<Tag>;
   constexpr int DD = D * D;
   constexpr int NCH = DD / 8 / 256;
+  if (count >= nblocks) {                    // (uniform over the workgroup)
+#pragma unroll
+    for (int c = 0; c < NCH; ++c)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[c][e] = 0.f;
+    zacc = 0.f;
+    return;
+  }
 #pragma unroll
   for (int c = 0; c < NCH; ++c) {
     const int idx = (tid + 256 * c) * 8;
@@ -204,7 +215,7 @@ __global__ __launch_bounds__(256) void complement_out_kernel(const uint16_t* __r
     float acc[NCH][8];
     float zacc;
     gather_complement<Tag, D>(acc, zacc, hall + (size_t)bh * DD, zall + (size_t)bh * D, hblk + (size_t)bh * N * DD,
-                              zblk + (size_t)bh * N * D, topk, lut_at, tid);
+                              zblk + (size_t)bh * N * D, topk, N, lut_at, tid);
     park_state<Tag, D, STR>(sH, acc, tid);
     // projection weight, 16 bit, columns in accumulator slot order
     for (int idx = tid; idx < DD; idx += 256) {
@@ -373,7 +384,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   float acc[NCH][8];
   float zacc;
   gather_complement<Tag, D>(acc, zacc, hall + (size_t)bh * DD, zall + (size_t)bh * D, hblk + (size_t)bh * N * DD,
-                            zblk + (size_t)bh * N * D, topk, lut_at, tid);
+                            zblk + (size_t)bh * N * D, topk, N, lut_at, tid);
   // G in B-operand order (d = 16c + 8g + j)
   i16x8_t gf[DC];
   if (active && G_IN_H) {
@@ -565,7 +576,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   float acc[NCH][8];
   float zacc;
   gather_complement<Tag, D>(acc, zacc, gall + (size_t)bh * DD, gzall + (size_t)bh * D, dhblk + (size_t)bh * Mblk * DD,
-                            dzblk + (size_t)bh * Mblk * D, count[(size_t)bh * N + nb], list_at, tid);
+                            dzblk + (size_t)bh * Mblk * D, count[(size_t)bh * N + nb], Mblk, list_at, tid);
   i16x8_t vf[DC];
   if (active) {
 #pragma unroll

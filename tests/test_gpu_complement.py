@@ -124,3 +124,22 @@ def test_module_trains_in_complement_mode(dev):
     lin = _oracle_grads(q, k, v, lut, w, b, do, "softmax", cfg.BLKQ)
     refs = [a + c for a, c in zip(sp, lin[:3])] + lin[3:]
     _check_grads((qd.grad, kd.grad, vd.grad, mod.proj_l.weight.grad, mod.proj_l.bias.grad), refs)
+
+
+def test_everything_selected_leaves_the_bias_and_no_gradient(dev):
+    """topk = 1: the complement is empty.  The difference of the two state sums is then exactly zero (not their
+    rounding residue, which the 1e-5 of the divisor would amplify): the branch is the bias, and only the bias has a gradient."""
+    from sla_amd import _attention
+    gen = torch.Generator().manual_seed(17)
+    q, k, v, g = (torch.randn(1, 2, 333, 128, generator=gen).to(torch.bfloat16).to(dev) for _ in range(4))
+    w, b = (t.to(dev) for t in make_proj(128))
+    for BLKQ in (64, 128):
+        M, N = -(-333 // BLKQ), 6
+        lut = torch.arange(N, device=dev).expand(1, 2, M, N).contiguous()
+        m = torch.ones(1, 2, M, N, dtype=torch.int8, device=dev)
+        out = linear_complement_fwd(q, k, v, lut, N, w, b, None, "elu", BLKQ, 64)
+        assert torch.equal(out, b.to(torch.bfloat16).expand_as(out))
+        dq, dk, dv, dw, db = linear_complement_bwd(q, k, v, m, lut, N, w, b, g, "elu", BLKQ, 64)
+        for t in (dq, dk, dv, dw):
+            assert int(torch.count_nonzero(t)) == 0
+        assert max_abs(db.cpu(), g.float().sum((0, 1, 2)).cpu()) <= 1e-2 * float(g.float().sum((0, 1, 2)).abs().max())
