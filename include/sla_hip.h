@@ -100,7 +100,10 @@ int sla_sparse_attn_linear_fwd(const void* q, const void* k, const void* v, cons
                                int BLKQ, int BLKK, int topk, float qk_scale, void* stream);
 
 /* Block-sparse FlashAttention backward: delta, dQ over the look-up table, dK/dV
- * over per-key-block lists built from the int8 map.
+ * over per-key-block lists built from the int8 map.  sparse_map and lut are the pair sla_block_map_fwd
+ * produced: every map row holds `topk` ones, the same blocks the look-up row names (the workspace,
+ * SLA_WS_SPARSE_BWD, is sized from topk; lists of key blocks that very many query blocks selected are cut
+ * into segments whose fp32 partials are added in a fixed order, so the result does not depend on scheduling).
  * Replaces _attention.backward + _attn_bwd_preprocess/_dq/_dkdv,
  * sparse_linear_attention/kernel.py:85-237, 277-320. */
 int sla_sparse_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o,
