@@ -50,3 +50,26 @@ def test_cfg2_gradients(dev, fmap):
         scale = max(1.0, float(r.abs().max()))
         assert max_abs(a.cpu(), r) <= TOL_ABS * scale, (name, max_abs(a.cpu(), r), scale)
         assert cos_sim(a.cpu(), r) >= TOL_COS, name
+
+
+@pytest.mark.parametrize("mode", ["global", "complement"])
+def test_forward_and_gradients_are_bit_reproducible(dev, mode):
+    """No atomics anywhere on the path: two runs give the same bits, also with a key block that every query block
+    selects (its list is cut into segments whose partial sums are added in a fixed order)."""
+    cfg = CONFIGS["cfg2"]
+    d = make_inputs(cfg, H=2)
+    d["k"][:, :, :64] += 3 * d["q"].float().mean(-2, keepdim=True).to(d["k"].dtype)   # pulls key block 0 into most rows
+    w, b = make_proj(cfg.D)
+    mod = SparseLinearAttention(cfg.D, cfg.topk, "elu", cfg.BLKQ, cfg.BLKK, linear_mode=mode).to(dev)
+    with torch.no_grad():
+        mod.proj_l.weight.copy_(w)
+        mod.proj_l.bias.copy_(b)
+    runs = []
+    for _ in range(2):
+        qd, kd, vd = (d[x].to(dev).requires_grad_(True) for x in "qkv")
+        mod.zero_grad()
+        o = mod(qd, kd, vd)
+        o.backward(d["do"].to(dev))
+        runs.append([t.detach().clone() for t in (o, qd.grad, kd.grad, vd.grad, mod.proj_l.weight.grad, mod.proj_l.bias.grad)])
+    for a, c in zip(*runs):
+        assert torch.equal(a, c)
