@@ -82,32 +82,14 @@ __global__ __launch_bounds__(256) void complement_total_kernel(const float* __re
   }
 }
 
-// A D x D state `total - sum of the listed blocks` in fp32 registers: thread t of 256 owns the 16-byte chunks
-// t + 256 c of the (row-major, 16-bit) block states, and element t of the z vectors when t < D.
-// `at(i)` is the block index of list entry i (`count` entries, subtracted in list order).  Two listed
-// states are in flight while a third is being subtracted (the gather is latency-bound: bytes in flight per
-// compute unit set its rate).
-// When the list names every block (`count == nblocks`) the difference is exactly zero by definition; it is
-// returned as such instead of as the rounding residue of two fp32 sums formed in different orders, which the
-// 1e-5 of the divisor would otherwise turn into an arbitrary result.
-template <typename Tag, int D, typename At>
-static __device__ __forceinline__ void gather_complement(float (&acc)[D * D / 8 / 256][8], float& zacc,
-                                                         const float* __restrict__ total, const float* __restrict__ ztotal,
-                                                         const uint16_t* __restrict__ blocks, const float* __restrict__ zblocks,
-                                                         int count, int nblocks, At at, int tid) {
-  using E = Elem<Tag>;
-  constexpr int DD = D * D;
-  constexpr int NCH = DD / 8 / 256;
-  if (count >= nblocks) {                    // (uniform over the workgroup)
+// A D x D state held in fp32 registers: thread t of 256 owns the 16-byte chunks t + 256 c of the (row-major, 16-bit)
+// block states, and element t of the z vectors when t < D.
+template <int D>
+static __device__ __forceinline__ void state_from_total(float (&acc)[D * D / 8 / 256][8], float& zacc,
+                                                        const float* __restrict__ total, const float* __restrict__ ztotal,
+                                                        int tid) {
 #pragma unroll
-    for (int c = 0; c < NCH; ++c)
-#pragma unroll
-      for (int e = 0; e < 8; ++e) acc[c][e] = 0.f;
-    zacc = 0.f;
-    return;
-  }
-#pragma unroll
-  for (int c = 0; c < NCH; ++c) {
+  for (int c = 0; c < D * D / 8 / 256; ++c) {
     const int idx = (tid + 256 * c) * 8;
     const f32x4_t a = *reinterpret_cast<const f32x4_t*>(total + idx);
     const f32x4_t b = *reinterpret_cast<const f32x4_t*>(total + idx + 4);
@@ -118,21 +100,29 @@ static __device__ __forceinline__ void gather_complement(float (&acc)[D * D / 8 
     }
   }
   zacc = tid < D ? ztotal[tid] : 0.f;
+}
+
+// Adds or subtracts `count` listed block states, in list order.  `at(i)` is list entry i: a block index j >= 0 means
+// "subtract block j", ~j (negative) means "add block j".  Two listed states are in flight while a third is being
+// applied (the gather is latency-bound: bytes in flight per compute unit set its rate).
+template <typename Tag, int D, typename At>
+static __device__ __forceinline__ void apply_states(float (&acc)[D * D / 8 / 256][8], float& zacc,
+                                                    const uint16_t* __restrict__ blocks, const float* __restrict__ zblocks,
+                                                    int count, At at, int tid) {
+  using E = Elem<Tag>;
+  constexpr int DD = D * D;
+  constexpr int NCH = DD / 8 / 256;
   i16x8_t ring[2][NCH];
   float zring[2] = {0.f, 0.f};
+  float sgn[2] = {0.f, 0.f};
   auto fetch = [&](int slot, int i) {
-    const int nb = at(i);
+    const int e = at(i);
+    const int nb = e < 0 ? ~e : e;
+    sgn[slot] = e < 0 ? 1.0f : -1.0f;
     const uint16_t* p = blocks + (size_t)nb * DD;
 #pragma unroll
     for (int c = 0; c < NCH; ++c) ring[slot][c] = *reinterpret_cast<const i16x8_t*>(p + (tid + 256 * c) * 8);
     zring[slot] = tid < D ? zblocks[(size_t)nb * D + tid] : 0.f;
-  };
-  auto consume = [&](int slot) {
-#pragma unroll
-    for (int c = 0; c < NCH; ++c)
-#pragma unroll
-      for (int e = 0; e < 8; ++e) acc[c][e] -= E::to_float((uint16_t)ring[slot][c][e]);
-    zacc -= zring[slot];
   };
   if (count > 0) fetch(0, 0);
   if (count > 1) fetch(1, 1);
@@ -141,24 +131,51 @@ static __device__ __forceinline__ void gather_complement(float (&acc)[D * D / 8 
     i16x8_t x[NCH];
 #pragma unroll
     for (int c = 0; c < NCH; ++c) x[c] = ring[0][c];
-    const float zx = zring[0];
+    const float zx = zring[0], sx = sgn[0];
     if (it + 2 < count) fetch(0, it + 2);
 #pragma unroll
     for (int c = 0; c < NCH; ++c)
 #pragma unroll
-      for (int e = 0; e < 8; ++e) acc[c][e] -= E::to_float((uint16_t)x[c][e]);
-    zacc -= zx;
+      for (int e = 0; e < 8; ++e) acc[c][e] += sx * E::to_float((uint16_t)x[c][e]);
+    zacc += sx * zx;
 #pragma unroll
     for (int c = 0; c < NCH; ++c) x[c] = ring[1][c];
-    const float zy = zring[1];
+    const float zy = zring[1], sy = sgn[1];
     if (it + 3 < count) fetch(1, it + 3);
 #pragma unroll
     for (int c = 0; c < NCH; ++c)
 #pragma unroll
-      for (int e = 0; e < 8; ++e) acc[c][e] -= E::to_float((uint16_t)x[c][e]);
-    zacc -= zy;
+      for (int e = 0; e < 8; ++e) acc[c][e] += sy * E::to_float((uint16_t)x[c][e]);
+    zacc += sy * zy;
   }
-  if (it < count) consume(0);
+  if (it < count) {
+#pragma unroll
+    for (int c = 0; c < NCH; ++c)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[c][e] += sgn[0] * E::to_float((uint16_t)ring[0][c][e]);
+    zacc += sgn[0] * zring[0];
+  }
+}
+
+// `total - sum of the listed blocks` (list entries are block indices, subtracted in list order).
+// When the list names every block (`count == nblocks`) the difference is exactly zero by definition; it is
+// returned as such instead of as the rounding residue of two fp32 sums formed in different orders, which the
+// 1e-5 of the divisor would otherwise turn into an arbitrary result.
+template <typename Tag, int D, typename At>
+static __device__ __forceinline__ void gather_complement(float (&acc)[D * D / 8 / 256][8], float& zacc,
+                                                         const float* __restrict__ total, const float* __restrict__ ztotal,
+                                                         const uint16_t* __restrict__ blocks, const float* __restrict__ zblocks,
+                                                         int count, int nblocks, At at, int tid) {
+  if (count >= nblocks) {                    // (uniform over the workgroup)
+#pragma unroll
+    for (int c = 0; c < D * D / 8 / 256; ++c)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[c][e] = 0.f;
+    zacc = 0.f;
+    return;
+  }
+  state_from_total<D>(acc, zacc, total, ztotal, tid);
+  apply_states<Tag, D>(acc, zacc, blocks, zblocks, count, at, tid);
 }
 
 // The gathered state, rounded to 16 bit, into an LDS matrix of D rows with row stride STR (same row-major
@@ -177,10 +194,59 @@ static __device__ __forceinline__ void park_state(uint16_t* sH, const float (&ac
   }
 }
 
-// 1-D grid over (head, query block) with the XCD-aware remap of the attention kernels: neighbouring query
-// blocks select mostly the same key blocks, so their state reads hit the same XCD's L2.  256 threads.
+// Look-up rows of neighbouring query blocks share most of their entries, so a workgroup walks a run of COMPL_RUN
+// consecutive query blocks of one head and keeps H_i in fp32 registers: the first block of the run gathers
+// `total - its T selected states`, every later block only applies the difference of its look-up row against the
+// previous one (adds back the states that dropped out, subtracts the new ones).  The difference lists are formed in
+// a fixed order (dropped entries in the previous row's order, then new entries in this row's order), so results do
+// not depend on scheduling.  Rows longer than COMPL_TMAX fall back to the full gather for every block.
+constexpr int COMPL_RUN = 4;
+constexpr int COMPL_TMAX = 256;
+
+// The signed difference list between the previous look-up row (sPrev) and this one (sCur), both `T` entries in LDS:
+// sList[0 .. ndrop) = ~j for the blocks j only the previous row names, sList[ndrop .. ndrop + nnew) = j for the blocks
+// only this row names.  Returns ndrop + nnew.  All 256 threads call it; contains workgroup barriers.
+static __device__ __forceinline__ int lut_difference(const int* sPrev, const int* sCur, int* sList, int (*sCnt)[4], int T,
+                                                     int tid) {
+  const int lane = tid & 63, wave = tid >> 6;
+  bool isdrop = false, isnew = false;
+  int p = 0, c = 0;
+  if (tid < T) {
+    p = sPrev[tid];
+    c = sCur[tid];
+    bool found_p = false, found_c = false;
+    for (int u = 0; u < T; ++u) {
+      found_p |= sCur[u] == p;
+      found_c |= sPrev[u] == c;
+    }
+    isdrop = !found_p;
+    isnew = !found_c;
+  }
+  const unsigned long long bd = __ballot(isdrop), bn = __ballot(isnew);
+  if (lane == 0) {
+    sCnt[0][wave] = __popcll(bd);
+    sCnt[1][wave] = __popcll(bn);
+  }
+  __syncthreads();
+  int ndrop = 0, nnew = 0, before_d = 0, before_n = 0;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    before_d += w < wave ? sCnt[0][w] : 0;
+    before_n += w < wave ? sCnt[1][w] : 0;
+    ndrop += sCnt[0][w];
+    nnew += sCnt[1][w];
+  }
+  const unsigned long long lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+  if (isdrop) sList[before_d + __popcll(bd & lt_mask)] = ~p;
+  if (isnew) sList[ndrop + before_n + __popcll(bn & lt_mask)] = c;
+  __syncthreads();
+  return ndrop + nnew;
+}
+
+// 1-D grid over (head, run of COMPL_RUN query blocks) with the XCD-aware remap of the attention kernels: neighbouring
+// runs select mostly the same key blocks, so their state reads hit the same XCD's L2.  256 threads.
 template <typename Tag, int D, int BLKQ>
-__global__ __launch_bounds__(256) void complement_out_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ hblk,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void complement_out_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ hblk,
                                                              const float* __restrict__ zblk, const float* __restrict__ hall,
                                                              const float* __restrict__ zall, const void* __restrict__ lut,
                                                              int lut64, const float* __restrict__ weight,
@@ -198,120 +264,150 @@ __global__ __launch_bounds__(256) void complement_out_kernel(const uint16_t* __r
   __shared__ __attribute__((aligned(16))) uint16_t sW[D * STR];    // W [e][d2 in accumulator slot order]
   __shared__ float sBias[D];
   __shared__ float sZ[D];
+  __shared__ int sPrev[COMPL_TMAX], sCur[COMPL_TMAX], sList[2 * COMPL_TMAX];
+  __shared__ int sCnt[2][4];
 
   const int logical = xcd_remap(blockIdx.x, gridDim.x, total);
   if (logical < 0) return;
-  const int bh = logical / Mblk, mb = logical - bh * Mblk;
+  const int runs = (Mblk + COMPL_RUN - 1) / COMPL_RUN;
+  const int bh = logical / runs, mb0 = (logical - bh * runs) * COMPL_RUN;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int g = lane >> 5, r = lane & 31;
-  const size_t lut_row = ((size_t)bh * Mblk + mb) * topk;
-  auto lut_at = [&](int i) -> int {
-    return lut64 ? (int)reinterpret_cast<const long long*>(lut)[lut_row + i]
-                 : reinterpret_cast<const int*>(lut)[lut_row + i];
-  };
 
-  // ---- H_i = total - selected, fp32, then 16 bit into LDS ----
-  {
-    float acc[NCH][8];
-    float zacc;
-    gather_complement<Tag, D>(acc, zacc, hall + (size_t)bh * DD, zall + (size_t)bh * D, hblk + (size_t)bh * N * DD,
-                              zblk + (size_t)bh * N * D, topk, N, lut_at, tid);
+  // projection weight, 16 bit, columns in accumulator slot order; bias
+  for (int idx = tid; idx < DD; idx += 256) {
+    const int e = idx / D, d = idx % D;
+    sW[e * STR + slot_order_pos(d)] = E::from_float(weight[idx]);
+  }
+  if (tid < D) sBias[tid] = round16<Tag>(bias[tid]);
+
+  const uint16_t* hb = hblk + (size_t)bh * N * DD;
+  const float* zb = zblk + (size_t)bh * N * D;
+  const bool diffable = topk <= COMPL_TMAX && topk < N;
+  float acc[NCH][8];
+  float zacc;
+#pragma nounroll
+  for (int step = 0; step < COMPL_RUN; ++step) {
+    const int mb = mb0 + step;
+    if (mb >= Mblk) break;
+    const size_t lut_row = ((size_t)bh * Mblk + mb) * topk;
+    auto lut_at = [&](int i) -> int {
+      return lut64 ? (int)reinterpret_cast<const long long*>(lut)[lut_row + i]
+                   : reinterpret_cast<const int*>(lut)[lut_row + i];
+    };
+    // ---- H_i in fp32: total - selected for the first block of the run, the previous block's H plus the difference of
+    // the two look-up rows afterwards ----
+    const bool full = step == 0 || !diffable;          // (uniform over the workgroup)
+    int count = topk;
+    if (full) {
+      if (diffable && tid < topk) sPrev[tid] = lut_at(tid);       // (read after the barriers below)
+      if (topk >= N) {
+        count = 0;                                                // everything selected: exactly zero, see gather_complement
+#pragma unroll
+        for (int c = 0; c < NCH; ++c)
+#pragma unroll
+          for (int e = 0; e < 8; ++e) acc[c][e] = 0.f;
+        zacc = 0.f;
+      } else {
+        state_from_total<D>(acc, zacc, hall + (size_t)bh * DD, zall + (size_t)bh * D, tid);
+      }
+    } else {
+      if (tid < topk) sCur[tid] = lut_at(tid);
+      __syncthreads();
+      count = lut_difference(sPrev, sCur, sList, sCnt, topk, tid);
+      if (tid < topk) sPrev[tid] = sCur[tid];                     // (every thread has passed the barriers of lut_difference)
+    }
+    auto entry_at = [&](int i) -> int { return full ? lut_at(i) : sList[i]; };
+    apply_states<Tag, D>(acc, zacc, hb, zb, count, entry_at, tid);
     park_state<Tag, D, STR>(sH, acc, tid);
-    // projection weight, 16 bit, columns in accumulator slot order
-    for (int idx = tid; idx < DD; idx += 256) {
-      const int e = idx / D, d = idx % D;
-      sW[e * STR + slot_order_pos(d)] = E::from_float(weight[idx]);
-    }
-    if (tid < D) {
-      sZ[tid] = round16<Tag>(zacc);
-      sBias[tid] = round16<Tag>(bias[tid]);
-    }
-  }
-  __syncthreads();
-  if (wave >= BLKQ / 32) return;
-
-  // ---- this wave's 32 queries ----
-  const int qrow = mb * BLKQ + wave * 32 + r;
-  const bool ok = qrow < L;
-  const size_t off = ((size_t)bh * L + qrow) * D;
-  float f[DC][8];
+    if (tid < D) sZ[tid] = round16<Tag>(zacc);
+    __syncthreads();
+    if (wave < BLKQ / 32) {
+      // ---- this wave's 32 queries ----
+      const int qrow = mb * BLKQ + wave * 32 + r;
+      const bool ok = qrow < L;
+      const size_t off = ((size_t)bh * L + qrow) * D;
+      float f[DC][8];
 #pragma unroll
-  for (int c = 0; c < DC; ++c) {
-    i16x8_t x = {0, 0, 0, 0, 0, 0, 0, 0};
-    if (ok) x = *reinterpret_cast<const i16x8_t*>(q + off + 16 * c + 8 * g);
+      for (int c = 0; c < DC; ++c) {
+        i16x8_t x = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (ok) x = *reinterpret_cast<const i16x8_t*>(q + off + 16 * c + 8 * g);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) f[c][j] = E::to_float((uint16_t)x[j]);
-  }
-  float row_mx, row_inv;
-  phi_row_pair<Tag, DC>(fmap, f, row_mx, row_inv);
-  float den = 0.f;
-  i16x8_t qf[DC];
-#pragma unroll
-  for (int c = 0; c < DC; ++c) {
-    i32x4_t pw;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) den += round16<Tag>(f[c][j] * sZ[16 * c + 8 * g + j]);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) pw[j] = (int)E::pack2(f[c][2 * j], f[c][2 * j + 1]);
-    qf[c] = __builtin_bit_cast(i16x8_t, pw);
-  }
-  den += __shfl_xor(den, 32);
-  den = round16<Tag>(1e-5f + round16<Tag>(den));
-  const float inv_den = 1.0f / den;
-
-  // N^T = H_i^T phi(Q)^T ; Y^T = round(round(N^T) / den) packed straight into B-operand fragments
-  i16x8_t yf[DT][2];
-#pragma unroll
-  for (int t = 0; t < DT; ++t) {
-    f32x16_t nacc;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) nacc[i] = 0.f;
-#pragma unroll
-    for (int c = 0; c < DC; ++c) {
-      const i16x8_t a = *reinterpret_cast<const i16x8_t*>(&sH[(32 * t + r) * STR + 16 * c + 8 * g]);
-      nacc = E::mfma32(a, qf[c], nacc);
-    }
-#pragma unroll
-    for (int c2 = 0; c2 < 2; ++c2) {
-      i32x4_t pw;
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        pw[j] = (int)E::pack2(round16<Tag>(nacc[8 * c2 + 2 * j]) * inv_den, round16<Tag>(nacc[8 * c2 + 2 * j + 1]) * inv_den);
-      yf[t][c2] = __builtin_bit_cast(i16x8_t, pw);
-    }
-  }
-  // OUT^T = W Y^T : contraction chunk (t, c2) covers d2 = 32t + 16c2 .. +15 in slot order
-#pragma unroll
-  for (int et = 0; et < DT; ++et) {
-    f32x16_t oacc;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) oacc[i] = 0.f;
-#pragma unroll
-    for (int t = 0; t < DT; ++t)
-#pragma unroll
-      for (int c2 = 0; c2 < 2; ++c2) {
-        const i16x8_t a = *reinterpret_cast<const i16x8_t*>(&sW[(32 * et + r) * STR + 16 * (2 * t + c2) + 8 * g]);
-        oacc = E::mfma32(a, yf[t][c2], oacc);
+        for (int j = 0; j < 8; ++j) f[c][j] = E::to_float((uint16_t)x[j]);
       }
-    if (ok) {
+      float row_mx, row_inv;
+      phi_row_pair<Tag, DC>(fmap, f, row_mx, row_inv);
+      float den = 0.f;
+      i16x8_t qf[DC];
 #pragma unroll
-      for (int i4 = 0; i4 < 4; ++i4) {
-        const int e0 = 32 * et + 8 * i4 + 4 * g;
-        float y[4];
+      for (int c = 0; c < DC; ++c) {
+        i32x4_t pw;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) y[j] = round16<Tag>(oacc[4 * i4 + j] + sBias[e0 + j]);
-        if (residual) {
-          const i32x2_t rv = *reinterpret_cast<const i32x2_t*>(residual + off + e0);
-          const uint16_t* rp = reinterpret_cast<const uint16_t*>(&rv);
+        for (int j = 0; j < 8; ++j) den += round16<Tag>(f[c][j] * sZ[16 * c + 8 * g + j]);
 #pragma unroll
-          for (int j = 0; j < 4; ++j) y[j] += E::to_float(rp[j]);
+        for (int j = 0; j < 4; ++j) pw[j] = (int)E::pack2(f[c][2 * j], f[c][2 * j + 1]);
+        qf[c] = __builtin_bit_cast(i16x8_t, pw);
+      }
+      den += __shfl_xor(den, 32);
+      den = round16<Tag>(1e-5f + round16<Tag>(den));
+      const float inv_den = 1.0f / den;
+
+      // N^T = H_i^T phi(Q)^T ; Y^T = round(round(N^T) / den) packed straight into B-operand fragments
+      i16x8_t yf[DT][2];
+#pragma unroll
+      for (int t = 0; t < DT; ++t) {
+        f32x16_t nacc;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) nacc[i] = 0.f;
+#pragma unroll
+        for (int c = 0; c < DC; ++c) {
+          const i16x8_t a = *reinterpret_cast<const i16x8_t*>(&sH[(32 * t + r) * STR + 16 * c + 8 * g]);
+          nacc = E::mfma32(a, qf[c], nacc);
         }
-        i32x2_t w;
-        w[0] = (int)E::pack2(y[0], y[1]);
-        w[1] = (int)E::pack2(y[2], y[3]);
-        *reinterpret_cast<i32x2_t*>(out + off + e0) = w;
+#pragma unroll
+        for (int c2 = 0; c2 < 2; ++c2) {
+          i32x4_t pw;
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            pw[j] = (int)E::pack2(round16<Tag>(nacc[8 * c2 + 2 * j]) * inv_den, round16<Tag>(nacc[8 * c2 + 2 * j + 1]) * inv_den);
+          yf[t][c2] = __builtin_bit_cast(i16x8_t, pw);
+        }
+      }
+      // OUT^T = W Y^T : contraction chunk (t, c2) covers d2 = 32t + 16c2 .. +15 in slot order
+#pragma unroll
+      for (int et = 0; et < DT; ++et) {
+        f32x16_t oacc;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) oacc[i] = 0.f;
+#pragma unroll
+        for (int t = 0; t < DT; ++t)
+#pragma unroll
+          for (int c2 = 0; c2 < 2; ++c2) {
+            const i16x8_t a = *reinterpret_cast<const i16x8_t*>(&sW[(32 * et + r) * STR + 16 * (2 * t + c2) + 8 * g]);
+            oacc = E::mfma32(a, yf[t][c2], oacc);
+          }
+        if (ok) {
+#pragma unroll
+          for (int i4 = 0; i4 < 4; ++i4) {
+            const int e0 = 32 * et + 8 * i4 + 4 * g;
+            float y[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) y[j] = round16<Tag>(oacc[4 * i4 + j] + sBias[e0 + j]);
+            if (residual) {
+              const i32x2_t rv = *reinterpret_cast<const i32x2_t*>(residual + off + e0);
+              const uint16_t* rp = reinterpret_cast<const uint16_t*>(&rv);
+#pragma unroll
+              for (int j = 0; j < 4; ++j) y[j] += E::to_float(rp[j]);
+            }
+            i32x2_t w;
+            w[0] = (int)E::pack2(y[0], y[1]);
+            w[1] = (int)E::pack2(y[2], y[3]);
+            *reinterpret_cast<i32x2_t*>(out + off + e0) = w;
+          }
+        }
       }
     }
+    __syncthreads();                       // H_i^T and z_i are rewritten by the next block of the run
   }
 }
 
@@ -703,7 +799,7 @@ static int complement_impl(const void* q, const void* k, const void* v, const vo
                      hgrp, zgrp, N, D);
   hipLaunchKernelGGL(complement_total_kernel, dim3(cdiv(D * D, 256), BH), dim3(256), 0, st, hgrp, zgrp, hall, zall, w.ngroup,
                      D);
-  const int total = BH * Mblk;
+  const int total = BH * cdiv(Mblk, COMPL_RUN);
   hipLaunchKernelGGL((complement_out_kernel<Tag, D, BLKQ>), dim3(xcd_grid(total)), dim3(256), 0, st, (const uint16_t*)q, hblk,
                      zblk, hall, zall, lut, lut64, weight, bias, (const uint16_t*)residual, (uint16_t*)out, L, Mblk, N, topk,
                      fmap, total);
