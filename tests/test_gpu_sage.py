@@ -102,3 +102,39 @@ def test_module_cfg5_two_heads(dev):
         SageSparseLinearAttention(128, 0.1, BLKQ=64, BLKK=64)
     with pytest.raises(NotImplementedError):
         SageSparseLinearAttention(128, 0.1, feature_map="hedgehog")
+
+
+def test_quantised_forward_in_a_hip_graph(dev):
+    """The quantised forward is capturable too (under capture the k/v state build and the v quantiser stay on the
+    capturing stream); every replay is checked against the eager result, with eager work between the replays."""
+    cfg = CONFIGS["cfg2"]
+    d = make_inputs(cfg, H=2)
+    w, b = make_proj(cfg.D)
+    mod = SageSparseLinearAttention(cfg.D, cfg.topk, "elu").to(dev)
+    q, k, v = (d[x].to(dev) for x in "qkv")
+    with torch.no_grad():
+        mod.proj_l.weight.copy_(w)
+        mod.proj_l.bias.copy_(b)
+        ref = mod(q, k, v)
+        torch.cuda.synchronize()
+        s = torch.cuda.Stream(device=dev)
+        s.wait_stream(torch.cuda.current_stream(dev))
+        with torch.cuda.stream(s):
+            mod(q, k, v)                      # warm-up on the capture stream
+        torch.cuda.current_stream(dev).wait_stream(s)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            out = mod(q, k, v)
+        for i in range(3):
+            out.zero_()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out, ref), f"replay {i}"
+            assert torch.equal(mod(q, k, v), ref)   # eager work between the replays
+            torch.cuda.synchronize()
+        v2 = torch.roll(v, 5, dims=2)
+        ref2 = mod(q, k, v2)
+        v.copy_(v2)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, ref2)
