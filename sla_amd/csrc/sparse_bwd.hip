@@ -228,7 +228,7 @@ __global__ __launch_bounds__(256) void bwd_dkdv_reduce_kernel(const int* __restr
 // CONTIG: all tensors are contiguous (B, H, L, D); the row pitch is then the compile-time D and every in-tile
 // offset folds into an instruction immediate (the strided variant pays a few registers for the run-time pitch).
 template <typename Tag, int D, int BLKQ, bool CONTIG>
-__global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))) void bwd_dq_kernel(
+__global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(D == 64 ? 3 : 2, D == 64 ? 3 : 2))) void bwd_dq_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ k, const uint16_t* __restrict__ v,
     const uint16_t* __restrict__ d_o, const float* __restrict__ lse, const float* __restrict__ delta,
     const void* __restrict__ lut, int lut64, uint16_t* __restrict__ dq, const RowLayout lin, const RowLayout ldo, int L,
@@ -416,7 +416,7 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
 // dV^T += dO^T P and dK^T += Q^T dS.  Splitting the accumulators this way keeps a wave at 256 registers,
 // so two waves share a SIMD.
 template <typename Tag, int D, int BLKQ, bool CONTIG>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void bwd_dkdv_kernel(
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 64 ? 3 : 2, D == 64 ? 3 : 2))) void bwd_dkdv_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ k, const uint16_t* __restrict__ v,
     const uint16_t* __restrict__ d_o, const float* __restrict__ lse, const float* __restrict__ delta,
     const int* __restrict__ list, const int* __restrict__ count, const i32x4_t* __restrict__ items,
