@@ -194,11 +194,14 @@ __global__ __launch_bounds__(1024) void colmean_fused_kernel(const float* __rest
 
 // score[bh][m][n] = round_dtype( sum_d pq[m][d]*pk[n][d] ), d ascending, every product and every sum rounded to fp32.
 // 64x64 outputs per workgroup, 4x4 per thread, operands staged through LDS 32 columns at a time.
-template <typename IO>
+// VECD (D a multiple of 32): every thread fetches eight adjacent d of one row of each operand with 16-byte loads,
+// one chunk ahead of the chunk being accumulated.
+template <typename IO, bool VECD>
 __global__ __launch_bounds__(256) void score_kernel(const typename IO::raw* __restrict__ pq,
                                                     const typename IO::raw* __restrict__ pk,
                                                     typename IO::raw* __restrict__ score, int M, int N, int D) {
   constexpr int TS = 64, DC = 32, LD = TS + 4;
+  constexpr int NV = 8 / IO::VEC;          // 16-byte loads per eight elements
   __shared__ __attribute__((aligned(16))) float sa[DC][LD];
   __shared__ __attribute__((aligned(16))) float sb[DC][LD];
   const int bh = blockIdx.z;
@@ -212,15 +215,41 @@ __global__ __launch_bounds__(256) void score_kernel(const typename IO::raw* __re
     for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
   const typename IO::raw* aq = pq + (size_t)bh * M * D;
   const typename IO::raw* bk = pk + (size_t)bh * N * D;
+  const int lrow = tid >> 2, lseg = (tid & 3) * 8;
+  Vec16<IO> va[NV], vb[NV];
+  auto fetch = [&](int d0) {
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+#pragma unroll
+      for (int e = 0; e < IO::VEC; ++e) {
+        va[v].e[e] = 0;
+        vb[v].e[e] = 0;
+      }
+      if (m0 + lrow < M) va[v] = reinterpret_cast<const Vec16<IO>*>(aq + (size_t)(m0 + lrow) * D + d0 + lseg)[v];
+      if (n0 + lrow < N) vb[v] = reinterpret_cast<const Vec16<IO>*>(bk + (size_t)(n0 + lrow) * D + d0 + lseg)[v];
+    }
+  };
+  if (VECD) fetch(0);
   for (int d0 = 0; d0 < D; d0 += DC) {
     __syncthreads();
-    for (int idx = tid; idx < TS * DC; idx += 256) {
-      const int row = idx / DC, dd = idx % DC;
-      const bool dok = d0 + dd < D;
-      sa[dd][row] = (m0 + row < M && dok) ? IO::ld(aq[(size_t)(m0 + row) * D + d0 + dd]) : 0.f;
-      sb[dd][row] = (n0 + row < N && dok) ? IO::ld(bk[(size_t)(n0 + row) * D + d0 + dd]) : 0.f;
+    if (VECD) {
+#pragma unroll
+      for (int v = 0; v < NV; ++v)
+#pragma unroll
+        for (int e = 0; e < IO::VEC; ++e) {
+          sa[lseg + v * IO::VEC + e][lrow] = IO::ld(va[v].e[e]);
+          sb[lseg + v * IO::VEC + e][lrow] = IO::ld(vb[v].e[e]);
+        }
+    } else {
+      for (int idx = tid; idx < TS * DC; idx += 256) {
+        const int row = idx / DC, dd = idx % DC;
+        const bool dok = d0 + dd < D;
+        sa[dd][row] = (m0 + row < M && dok) ? IO::ld(aq[(size_t)(m0 + row) * D + d0 + dd]) : 0.f;
+        sb[dd][row] = (n0 + row < N && dok) ? IO::ld(bk[(size_t)(n0 + row) * D + d0 + dd]) : 0.f;
+      }
     }
     __syncthreads();
+    if (VECD && d0 + DC < D) fetch(d0 + DC);
     const int dn = min(DC, D - d0);
     for (int dd = 0; dd < dn; ++dd) {
       const f32x4_t a = *reinterpret_cast<const f32x4_t*>(&sa[dd][ty * 4]);
@@ -251,6 +280,16 @@ __global__ __launch_bounds__(256) void score_kernel(const typename IO::raw* __re
       if (n < N) out[(size_t)m * N + n] = IO::st(acc[i][j]);
     }
   }
+}
+
+template <typename IO>
+static void launch_score(const typename IO::raw* pq, const typename IO::raw* pk, typename IO::raw* score, int BH, int M, int N,
+                         int D, hipStream_t st) {
+  const dim3 grid(cdiv(N, 64), cdiv(M, 64), BH);
+  if (D % 32 == 0)
+    hipLaunchKernelGGL((score_kernel<IO, true>), grid, dim3(256), 0, st, pq, pk, score, M, N, D);
+  else
+    hipLaunchKernelGGL((score_kernel<IO, false>), grid, dim3(256), 0, st, pq, pk, score, M, N, D);
 }
 
 // Monotone map float -> uint32 (larger float = larger key); -0.0 is folded onto +0.0.  The LOW_BIT
@@ -449,7 +488,7 @@ static int block_map_impl(const void* q, const void* k, const RowLayout& lay, in
   }
   launch_colmean_reduce<IO>(chunk_sums, (float*)(ws + w.group_sums), colmean, BH, L, D, st);
   launch_pool<IO, 2>(k, lay, colmean, pk, BH, L, D, BLKK, st);
-  hipLaunchKernelGGL((score_kernel<IO>), dim3(cdiv(N, 64), cdiv(M, 64), BH), dim3(256), 0, st, pq, pk, score, M, N, D);
+  launch_score<IO>(pq, pk, score, BH, M, N, D, st);
   // topk == 0 selects nothing: the kernel then only clears the map row.
   launch_topk<IO>(score, sparse_map, lut, lut64, N, topk, (size_t)BH * M, st);
   return check_launch("block map");
@@ -478,14 +517,11 @@ void launch_k_colmean(const void* k, const RowLayout& lay, int dtype, int BH, in
 // produce them on the way): pq (BH, M, D), pk (BH, N, D) in `dtype`; score: (BH, M, N) elements of `dtype`.
 void launch_map_from_pooled(int dtype, const void* pq, const void* pk, void* score, int BH, int M, int N, int D, int topk,
                             int8_t* sparse_map, void* lut, int lut64, hipStream_t st) {
-  const dim3 grid(cdiv(N, 64), cdiv(M, 64), BH);
   if (dtype == SLA_BF16) {
-    hipLaunchKernelGGL((score_kernel<IoBf16>), grid, dim3(256), 0, st, (const uint16_t*)pq, (const uint16_t*)pk,
-                       (uint16_t*)score, M, N, D);
+    launch_score<IoBf16>((const uint16_t*)pq, (const uint16_t*)pk, (uint16_t*)score, BH, M, N, D, st);
     launch_topk<IoBf16>((const uint16_t*)score, sparse_map, lut, lut64, N, topk, (size_t)BH * M, st);
   } else {
-    hipLaunchKernelGGL((score_kernel<IoF16>), grid, dim3(256), 0, st, (const uint16_t*)pq, (const uint16_t*)pk,
-                       (uint16_t*)score, M, N, D);
+    launch_score<IoF16>((const uint16_t*)pq, (const uint16_t*)pk, (uint16_t*)score, BH, M, N, D, st);
     launch_topk<IoF16>((const uint16_t*)score, sparse_map, lut, lut64, N, topk, (size_t)BH * M, st);
   }
 }
