@@ -165,30 +165,33 @@ __global__ __launch_bounds__(128) void colmean_kernel(const float* __restrict__ 
   colmean[(size_t)bh * D + d] = IO::st(acc / (float)L);
 }
 
-// Levels 2 and 3 in one workgroup per head when the group sums fit in LDS: thread (gi, d) = (tid / D, tid % D)
-// forms group sums gi, gi + 1024/D, ...; thread d < D then adds the groups in ascending order.
-constexpr int COLMEAN_LDS_FLOATS = 12288;
+// Levels 2 and 3 in one launch when the group sums of a column slab fit in LDS: one workgroup per (head, slab of
+// COLMEAN_SLAB columns), thread (gi, c) = (tid / COLMEAN_SLAB, tid % COLMEAN_SLAB) forms group sums gi, gi + 16, ...
+// of its column; the first COLMEAN_SLAB threads then add the groups in ascending order.  (Small workgroups: the
+// launch has to find room beside the memory-bound kernels that run on other streams at the same time.)
+constexpr int COLMEAN_SLAB = 16;
+constexpr int COLMEAN_MAX_GROUPS = 256;
 template <typename IO>
-__global__ __launch_bounds__(1024) void colmean_fused_kernel(const float* __restrict__ chunk_sums,
-                                                             typename IO::raw* __restrict__ colmean, int nchunk, int ngroup,
-                                                             int D, int L) {
-  __shared__ float gs[COLMEAN_LDS_FLOATS];
-  const int bh = blockIdx.x, tid = threadIdx.x;
-  const int d = tid % D, gstep = 1024 / D;
-  for (int g = tid / D; g < ngroup; g += gstep) {
+__global__ __launch_bounds__(256) void colmean_fused_kernel(const float* __restrict__ chunk_sums,
+                                                            typename IO::raw* __restrict__ colmean, int nchunk, int ngroup,
+                                                            int D, int L) {
+  __shared__ float gs[COLMEAN_MAX_GROUPS * COLMEAN_SLAB];
+  const int bh = blockIdx.y, tid = threadIdx.x;
+  const int c = tid % COLMEAN_SLAB, d = blockIdx.x * COLMEAN_SLAB + c;
+  for (int g = tid / COLMEAN_SLAB; g < ngroup; g += 256 / COLMEAN_SLAB) {
     const int c0 = g * KMEAN_GROUP;
     const int n = min(KMEAN_GROUP, nchunk - c0);
     const float* p = chunk_sums + ((size_t)bh * nchunk + c0) * D + d;
     float acc = 0.f;
 #pragma unroll 8
     for (int i = 0; i < n; ++i) acc = acc + p[(size_t)i * D];
-    gs[g * D + d] = acc;
+    gs[g * COLMEAN_SLAB + c] = acc;
   }
   __syncthreads();
-  if (tid < D) {
+  if (tid < COLMEAN_SLAB) {
     float acc = 0.f;
-    for (int g = 0; g < ngroup; ++g) acc = acc + gs[g * D + tid];
-    colmean[(size_t)bh * D + tid] = IO::st(acc / (float)L);
+    for (int g = 0; g < ngroup; ++g) acc = acc + gs[g * COLMEAN_SLAB + tid];
+    colmean[(size_t)bh * D + d] = IO::st(acc / (float)L);
   }
 }
 
@@ -453,8 +456,9 @@ template <typename IO>
 static void launch_colmean_reduce(float* chunk_sums, float* group_sums, typename IO::raw* colmean, int BH, int L, int D,
                                   hipStream_t st) {
   const int nchunk = cdiv(L, KMEAN_CHUNK), ngroup = cdiv(nchunk, KMEAN_GROUP);
-  if (D <= 1024 && 1024 % D == 0 && ngroup * D <= COLMEAN_LDS_FLOATS) {
-    hipLaunchKernelGGL((colmean_fused_kernel<IO>), dim3(BH), dim3(1024), 0, st, chunk_sums, colmean, nchunk, ngroup, D, L);
+  if (D % COLMEAN_SLAB == 0 && ngroup <= COLMEAN_MAX_GROUPS) {
+    hipLaunchKernelGGL((colmean_fused_kernel<IO>), dim3(D / COLMEAN_SLAB, BH), dim3(256), 0, st, chunk_sums, colmean, nchunk,
+                       ngroup, D, L);
     return;
   }
   hipLaunchKernelGGL(colmean_group_kernel, dim3(ngroup, BH), dim3(128), 0, st, chunk_sums, group_sums, nchunk, ngroup, D);

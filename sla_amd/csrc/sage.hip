@@ -76,6 +76,7 @@ __global__ __launch_bounds__(256) void quant_int8_kernel(const uint16_t* __restr
   amax = fmaxf(fmaxf(sred[0], sred[1]), fmaxf(sred[2], sred[3]));
   const float sc = fmaxf(amax, 1e-30f) / 127.0f;
   if (tid == 0) scale[(size_t)bh * nblk + blk] = sc;
+  const float inv_sc = 1.0f / sc;
   if (POOL && tid < D) {   // one column per thread (the barrier above also covers the tile)
     const int nrows = min(BLK, L - blk * BLK);
     float acc = 0.f;
@@ -100,7 +101,12 @@ __global__ __launch_bounds__(256) void quant_int8_kernel(const uint16_t* __restr
     int8_t* b = reinterpret_cast<int8_t*>(&w);
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      float r = rintf(val[p][e] / sc);
+      // round(val / sc) through the reciprocal: the product is within two units in the last place of the quotient
+      // (< 3e-5 for |quotient| <= 127), so both round to the same integer unless the product lies that close to a
+      // half-integer; those few elements take the division itself.
+      const float t = val[p][e] * inv_sc;
+      float r = rintf(t);
+      if (fabsf(t - r) > 0.4999f) r = rintf(val[p][e] / sc);
       r = fminf(fmaxf(r, -127.f), 127.f);
       b[e] = (int8_t)(int)r;
     }

@@ -35,6 +35,29 @@ def test_quantisers_bit_exact(dev, L, D):
     assert torch.equal(v8.cpu().view(torch.uint8), v8r.view(torch.uint8))
 
 
+def test_int8_quantiser_near_half_integers(dev):
+    """The kernel rounds x * (1 / scale) and takes the division only where that product lies close to a half-integer.
+    Two million elements hold a few hundred such quotients by chance; block 0 of q is planted with exact ties
+    (scale 1: values k + 0.5 round to even) and block 1 with a scale of 3 / 127, whose reciprocal is inexact."""
+    g = torch.Generator().manual_seed(5)
+    q = torch.randn(1, 2, 8192, 128, generator=g)
+    k = torch.randn(1, 2, 8192, 128, generator=g) + torch.randn(1, 2, 1, 128, generator=g)
+    halves = (torch.arange(128 * 128) % 253 - 126).float() + 0.5        # -125.5 .. 126.5, exact in bf16
+    q[0, 0, :128] = halves.view(128, 128)
+    q[0, 0, 0, 0] = 127.0
+    q[0, 0, 128:256] = (torch.arange(128 * 128) % 255 - 127).float().view(128, 128) * (3.0 / 254.0)
+    q[0, 0, 128, 0] = 3.0
+    q, k = q.to(torch.bfloat16), k.to(torch.bfloat16)
+    q8r, qsr, k8r, ksr, _ = O.sage_quant_qk(q, k, 128, 64)
+    quotient = q[0, 0].float().view(64, 128 * 128) / qsr[0, 0].view(64, 1)
+    assert int(((quotient - quotient.round()).abs() > 0.4999).sum()) > 100     # the slow path is exercised
+    q8, qs, k8, ks = quant_qk(q.to(dev), k.to(dev))
+    assert torch.equal(qs.cpu(), qsr) and torch.equal(ks.cpu(), ksr)
+    assert torch.equal(q8.cpu(), q8r) and torch.equal(k8.cpu(), k8r)
+    *_, q8p, qsp, k8p, ksp, _, _ = sage_prepare(q.to(dev), k.to(dev), None, 0.25)
+    assert torch.equal(q8p.cpu(), q8r) and torch.equal(k8p.cpu(), k8r)
+
+
 @pytest.mark.parametrize("L,D,ratio,dtype", [(512, 128, 0.5, torch.bfloat16), (1000, 128, 0.3, torch.bfloat16),
                                               (333, 64, 0.5, torch.float16), (2048, 128, 0.1, torch.float16),
                                               (100, 64, 1.0, torch.bfloat16)])
