@@ -147,20 +147,21 @@ __global__ __launch_bounds__(256) void v_amax_partial_kernel(const uint16_t* __r
   }
 }
 
-// grid (BH), 1024 threads: thread (cg, d) = (tid / D, tid % D) takes the maximum over chunks cg, cg + 1024/D, ...;
-// the 1024/D partial maxima per column meet in LDS.
-__global__ __launch_bounds__(1024) void v_scale_kernel(const float* __restrict__ part, float* __restrict__ v_scale, int nchunk,
-                                                      int D) {
-  __shared__ float sm[1024];
-  const int bh = blockIdx.x, tid = threadIdx.x;
-  const int d = tid % D, cg = tid / D, ncg = 1024 / D;
+// grid (D / 16, BH), 256 threads: thread (cg, c) = (tid / 16, tid % 16) takes the maximum of column 16 blockIdx.x + c
+// over chunks cg, cg + 16, ...; the 16 partial maxima per column meet in LDS.  (Small workgroups: the launch has to
+// find room beside the memory-bound kernels of the other stream.)
+__global__ __launch_bounds__(256) void v_scale_kernel(const float* __restrict__ part, float* __restrict__ v_scale, int nchunk,
+                                                     int D) {
+  __shared__ float sm[256];
+  const int bh = blockIdx.y, tid = threadIdx.x;
+  const int d = blockIdx.x * 16 + (tid & 15), cg = tid >> 4;
   float a = 0.f;
-  for (int c = cg; c < nchunk; c += ncg) a = fmaxf(a, part[((size_t)bh * nchunk + c) * D + d]);
+  for (int c = cg; c < nchunk; c += 16) a = fmaxf(a, part[((size_t)bh * nchunk + c) * D + d]);
   sm[tid] = a;
   __syncthreads();
-  if (tid < D) {
-    for (int j = 1; j < ncg; ++j) a = fmaxf(a, sm[j * D + tid]);
-    v_scale[(size_t)bh * D + tid] = fmaxf(a, 1e-30f) / 448.0f;
+  if (tid < 16) {
+    for (int j = 1; j < 16; ++j) a = fmaxf(a, sm[j * 16 + tid]);
+    v_scale[(size_t)bh * D + d] = fmaxf(a, 1e-30f) / 448.0f;
   }
 }
 
@@ -537,7 +538,7 @@ static int quant_v_impl(const void* v, const RowLayout& lay, int BH, int L, uint
   float* part = (float*)(ws + w.v_part);
   hipLaunchKernelGGL((v_amax_partial_kernel<Tag, D>), dim3(w.nchunk_v, BH), dim3(256), 0, st, (const uint16_t*)v, lay, part, L,
                      w.rows_per_chunk_v);
-  hipLaunchKernelGGL(v_scale_kernel, dim3(BH), dim3(1024), 0, st, part, vs, w.nchunk_v, D);
+  hipLaunchKernelGGL(v_scale_kernel, dim3(D / 16, BH), dim3(256), 0, st, part, vs, w.nchunk_v, D);
   constexpr int RPP = 256 / (D / 8);
   hipLaunchKernelGGL((v_quant_fp8_kernel<Tag, D>), dim3(cdiv(L, RPP), BH), dim3(256), 0, st, (const uint16_t*)v, lay, vs, v8,
                      L);
