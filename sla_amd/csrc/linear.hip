@@ -24,14 +24,17 @@ namespace sla {
 // kvwt[bh][e][d1] = round16( sum_d2 round16(W[e][d2]) * KVT[d2][d1] ), fp32 accumulation in ascending d2.
 // (phi(Q) KV / den) W^T = (phi(Q) (KV W^T)) / den, so the output kernel needs one product per query tile.
 // grid (D*D/256, BH): thread (e, d1); the 256 threads of a workgroup share at most two rows e.
+// The workgroups of head 0 also leave the 16-bit transposed weight wt[d][e] that a backward reads (what
+// linear_prep_weight_kernel writes), which saves the forward one launch in its chain of small kernels.
 template <typename Tag>
 __global__ __launch_bounds__(256) void linear_fold_kernel(const uint16_t* __restrict__ kvt, const float* __restrict__ weight,
-                                                          uint16_t* __restrict__ kvwt, int D) {
+                                                          uint16_t* __restrict__ kvwt, uint16_t* __restrict__ wt, int D) {
   using E = Elem<Tag>;
   const int bh = blockIdx.y;
   const int i = blockIdx.x * 256 + threadIdx.x;
   if (i >= D * D) return;
   const int e = i / D, d1 = i % D;
+  if (bh == 0) wt[d1 * D + e] = E::from_float(weight[i]);
   const uint16_t* s = kvt + (size_t)bh * D * D + d1;
   const float* w = weight + (size_t)e * D;
   float acc = 0.f;
@@ -149,9 +152,9 @@ template <typename Tag, int D>
 static int linear_state_impl(const void* k, const void* v, const RowLayout& lay, const float* weight, int fmap, int BH, int L,
                              char* ws, hipStream_t st) {
   const LinWs w = lin_ws(BH, L, D);
-  launch_state_build<Tag, D>(k, v, lay, weight, fmap, BH, L, ws, w, st);
+  launch_state_build<Tag, D>(k, v, lay, weight, fmap, BH, L, ws, w, st, false);
   hipLaunchKernelGGL((linear_fold_kernel<Tag>), dim3(cdiv(D * D, 256), BH), dim3(256), 0, st,
-                     (const uint16_t*)(ws + w.kvt), weight, (uint16_t*)(ws + w.kvwt), D);
+                     (const uint16_t*)(ws + w.kvt), weight, (uint16_t*)(ws + w.kvwt), (uint16_t*)(ws + w.wt), D);
   return check_launch("linear_state_fwd");
 }
 

@@ -244,7 +244,7 @@ static inline LinWs lin_ws(int BH, int L, int D) {
 // Streams K and V once and leaves KVT, KVP, z (16 bit) and the 16-bit transposed weight in the workspace.
 template <typename Tag, int D>
 static inline void launch_state_build(const void* k, const void* v, const RowLayout& lay, const float* weight, int fmap,
-                                      int BH, int L, char* ws, const LinWs& w, hipStream_t st) {
+                                      int BH, int L, char* ws, const LinWs& w, hipStream_t st, bool copy_weight = true) {
   float* kv_part = (float*)(ws + w.kv_part);
   float* z_part = (float*)(ws + w.z_part);
   uint16_t* kvt = (uint16_t*)(ws + w.kvt);
@@ -253,8 +253,10 @@ static inline void launch_state_build(const void* k, const void* v, const RowLay
                      (const uint16_t*)v, lay, kv_part, z_part, L, w.rows_per_split, fmap);
   hipLaunchKernelGGL((linear_state_reduce_kernel<Tag>), dim3(cdiv(D * D, 256), BH), dim3(256), 0, st, kv_part, z_part, kvt,
                      (uint16_t*)(ws + w.kvp), z, w.nsplit, D * D, D);
-  hipLaunchKernelGGL((linear_prep_weight_kernel<Tag>), dim3(cdiv(D * D, 256)), dim3(256), 0, st, weight,
-                     (uint16_t*)(ws + w.wt), D);
+  // (copy_weight = false: the caller's next kernel writes the 16-bit transposed weight on the side)
+  if (copy_weight)
+    hipLaunchKernelGGL((linear_prep_weight_kernel<Tag>), dim3(cdiv(D * D, 256)), dim3(256), 0, st, weight,
+                       (uint16_t*)(ws + w.wt), D);
 }
 
 }  // namespace sla
