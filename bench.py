@@ -26,13 +26,50 @@ if ROOT not in sys.path:
 PEAK_BF16_TFLOPS = 2500.0     # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0
 
-# HBM bytes per launch of the dominant kernel, from two `rocprofv3 --pmc` runs of this script
-# (FETCH_SIZE, then WRITE_SIZE; summaries under profiles/), each scaled by what the same counter reads for
-# the 1 GiB-read / 1 GiB-write elementwise kernel of --pmc-calibration (FETCH_SIZE x2.0, WRITE_SIZE x1.0).
-# It is a property of the kernel and the workload, not re-measured by a plain bench run.
-MEASURED_TRAFFIC_BYTES = {
-    "cfg3": {"kernel": "sparse_fwd_kernel<FUSED>", "fetch": 208656.1 * 1024 * 2.0, "write": 99869.7 * 1024 * 1.0},
-}
+PEAK_I8F8_TOPS = 5000.0        # MI355X dense int8 / fp8 MFMA
+
+# HBM bytes per launch of the dominant kernel come from two `rocprofv3 --pmc` runs of this script (FETCH_SIZE, then
+# WRITE_SIZE), each scaled by what the same counter reads for the 1 GiB-read / 1 GiB-write elementwise kernel of
+# --pmc-calibration.  A plain bench run cannot re-measure them, so the figures live in a small file next to the
+# profiler summaries, stamped with a fingerprint of the kernel's sources: when the kernel changes the stamp no
+# longer matches and `traffic` is reported as null until the counters have been read again (--record-traffic).
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "sparse_fwd_cfg3_hbm_traffic.json")
+KERNEL_SOURCES = ("sla_amd/csrc/sparse_fwd.hip", "sla_amd/csrc/common.h", "sla_amd/csrc/linear_state.h",
+                  "sla_amd/csrc/linear_common.h")
+
+
+def kernel_fingerprint() -> str:
+    import hashlib
+    h = hashlib.sha256()
+    for rel in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, rel), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(workload: str):
+    """(bytes per launch, note) from the committed counter readings, or (None, why not)."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            t = json.load(f)
+    except (OSError, ValueError):
+        return None, "no counter readings recorded"
+    if t.get("workload") != workload:
+        return None, f"counter readings are for {t.get('workload')}"
+    if t.get("kernel_sources_sha256_16") != kernel_fingerprint():
+        return None, "the kernel's sources changed after the counters were read"
+    return (t["fetch_size_kib"] * 1024 * t["fetch_factor"] + t["write_size_kib"] * 1024 * t["write_factor"],
+            "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a copy kernel of known size")
+
+
+def record_traffic(values):
+    fetch_kib, write_kib, fetch_factor, write_factor = values
+    t = {"workload": "cfg3", "kernel": "sparse_fwd_kernel<FUSED>", "fetch_size_kib": fetch_kib, "write_size_kib": write_kib,
+         "fetch_factor": fetch_factor, "write_factor": write_factor, "kernel_sources_sha256_16": kernel_fingerprint(),
+         "kernel_sources": list(KERNEL_SOURCES)}
+    with open(TRAFFIC_FILE, "w") as f:
+        json.dump(t, f, indent=1)
+        f.write("\n")
 
 
 def _events(torch):
@@ -80,6 +117,91 @@ def cpu_baseline(cfg, heads, torch):
                       f"{dt:.2f} s wall", "ms_per_step_scaled_to_all_heads": dt * 1e3 * cfg.H / heads}
 
 
+def other_configs(torch, dev, steps):
+    """The figures of the other benchmark configurations (a handful of steps each, inputs generated on the device):
+    the quantised forward on cfg5, forward and forward + backward on cfg4, the sparse backward alone on cfg3, and
+    the reference-convention kernel benchmark (evaluate/bench_kernel.py)."""
+    import dataclasses
+    import importlib.util
+    from sla_amd import SageSparseLinearAttention, SparseLinearAttention, get_block_map
+    from sla_amd.inputs import CONFIGS, make_inputs_on_device, make_proj
+    from sla_amd.sage import sage_attn_fwd, sage_prepare, quant_v
+    from sla_amd.sparse_attn import sparse_attn_bwd, sparse_attn_fwd
+    ex = {}
+    w, b = make_proj(128)
+
+    def seeded(mod):
+        with torch.no_grad():
+            mod.proj_l.weight.copy_(w)
+            mod.proj_l.bias.copy_(b)
+        return mod
+
+    # ---- cfg3: sparse backward alone (delta, lists, dq, dk/dv): 7 products per selected tile executed ----
+    cfg = CONFIGS["cfg3"]
+    q, k, v, do = make_inputs_on_device(cfg, dev, 3, True)
+    m, lut, T = get_block_map(q, k, cfg.topk, cfg.BLKQ, cfg.BLKK)
+    o, lse = sparse_attn_fwd(q, k, v, lut, T, cfg.BLKQ, cfg.BLKK, cfg.D ** -0.5)
+    ms = time_region(torch, lambda: sparse_attn_bwd(q, k, v, o, do, lse, m, lut, T, cfg.BLKQ, cfg.BLKK, cfg.D ** -0.5),
+                     steps, 2, preheat_s=0.05)
+    tiles = cfg.B * cfg.H * (-(-cfg.L // cfg.BLKQ)) * T
+    ex["cfg3_sparse_bwd_ms"] = ms
+    ex["cfg3_sparse_bwd_mfma_frac"] = 14.0 * tiles * cfg.BLKQ * 64 * cfg.D / ms / 1e9 / PEAK_BF16_TFLOPS
+    del q, k, v, do, o, lse, m, lut
+
+    # ---- cfg5: SageSLA module forward, and its attention kernel against the int8 / fp8 peak ----
+    cfg = CONFIGS["cfg5"]
+    q, k, v, _ = make_inputs_on_device(cfg, dev, 5, False)
+    sage = seeded(SageSparseLinearAttention(cfg.D, cfg.topk, cfg.feature_map).to(dev))
+    with torch.no_grad():
+        ex["cfg5_sage_fwd_ms"] = time_region(torch, lambda: sage(q, k, v), steps, 2, preheat_s=0.05)
+        m, lut, T, q8, qs, k8, ks, _, _ = sage_prepare(q, k, None, cfg.topk)
+        v8, vs = quant_v(v)
+        ms = time_region(torch, lambda: sage_attn_fwd(q8, qs, k8, ks, v8, vs, lut, T, torch.bfloat16), steps, 2,
+                         preheat_s=0.05)
+    ops = 4.0 * cfg.B * cfg.H * (-(-cfg.L // 128)) * T * 128 * 64 * cfg.D
+    ex["cfg5_sage_attention_kernel_ms"] = ms
+    ex["cfg5_sage_attention_kernel_frac_of_5_pops"] = ops / ms / 1e9 / PEAK_I8F8_TOPS
+    ex["cfg5_sage_effective_tflops"] = 4.0 * cfg.B * cfg.H * cfg.L * cfg.L * cfg.D / ex["cfg5_sage_fwd_ms"] / 1e9
+    del q8, k8, v8, m, lut, sage
+    # the 16-bit module on the same inputs and block sizes
+    mod = seeded(SparseLinearAttention(cfg.D, cfg.topk, cfg.feature_map, cfg.BLKQ, cfg.BLKK).to(dev))
+    with torch.no_grad():
+        ex["cfg5_sla_bf16_fwd_ms"] = time_region(torch, lambda: mod(q, k, v), steps, 2, preheat_s=0.05)
+    del q, k, v, mod
+
+    # ---- cfg4: module forward and forward + backward ----
+    cfg = CONFIGS["cfg4"]
+    q, k, v, do = make_inputs_on_device(cfg, dev, 4, True)
+    mod = seeded(SparseLinearAttention(cfg.D, cfg.topk, cfg.feature_map, cfg.BLKQ, cfg.BLKK).to(dev))
+    dense = 4.0 * cfg.B * cfg.H * cfg.L * cfg.L * cfg.D
+    with torch.no_grad():
+        ex["cfg4_sla_fwd_ms"] = time_region(torch, lambda: mod(q, k, v), steps, 1, preheat_s=0.05)
+        ms = time_region(torch, lambda: get_block_map(q, k, cfg.topk, cfg.BLKQ, cfg.BLKK), steps, 1, preheat_s=0.05)
+    ex["cfg4_fwd_effective_tflops"] = dense / ex["cfg4_sla_fwd_ms"] / 1e9
+    ex["cfg4_mask_ms"] = ms
+    ex["cfg4_mask_hbm_gbs"] = 2.0 * q.numel() * 2 / ms / 1e6
+    qg, kg, vg = (t.requires_grad_(True) for t in (q, k, v))
+
+    def fwd_bwd():
+        mod(qg, kg, vg).backward(do)
+        qg.grad = kg.grad = vg.grad = None
+    ex["cfg4_sla_fwd_bwd_ms"] = time_region(torch, fwd_bwd, steps, 1, preheat_s=0.05)
+    ex["cfg4_fwd_bwd_effective_tflops"] = 3.5 * dense / ex["cfg4_sla_fwd_bwd_ms"] / 1e9
+    del q, k, v, do, qg, kg, vg, mod
+    torch.cuda.empty_cache()
+
+    # ---- the reference's own kernel benchmark: B2 H16 L32760 D128 randn, sparsity .95, BLKQ 128 ----
+    spec = importlib.util.spec_from_file_location("bench_kernel", os.path.join(ROOT, "evaluate", "bench_kernel.py"))
+    bk = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bk)
+    for r in bk.run(iters=steps, warmup=2):
+        ex[f"bench_kernel_{r['mode']}_ms"] = r["ms"]
+        ex[f"bench_kernel_{r['mode']}_effective_tflops"] = r["effective_tflops"]
+        if "attention_kernel_ms" in r:
+            ex["bench_kernel_attention_kernel_ms"] = r["attention_kernel_ms"]
+    return ex
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -91,7 +213,14 @@ def main():
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run one plain 1 GiB read + 1 GiB write elementwise kernel, the known-size reference for "
                          "scaling the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
+    ap.add_argument("--record-traffic", type=float, nargs=4, metavar=("FETCH_KIB", "WRITE_KIB", "FETCH_FACTOR", "WRITE_FACTOR"),
+                    help="store the FETCH_SIZE / WRITE_SIZE readings (KiB per dispatch of the dominant kernel) and the "
+                         "calibration factors of two rocprofv3 --pmc runs, stamped with the kernel sources' fingerprint; "
+                         "needs no GPU")
     args = ap.parse_args()
+    if args.record_traffic:
+        record_traffic(args.record_traffic)
+        return
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (heads shard with no collective in "
               "forward); run with --gpus 1", file=sys.stderr)
@@ -137,6 +266,7 @@ def main():
     # executed MFMA work: QK^T and PV over the selected tiles + phi(q) KVW of the epilogue
     sparse_flops = 4.0 * B * H * M * T * cfg.BLKQ * cfg.BLKK * D + 2.0 * B * H * L * D * D
     achieved = sparse_flops / ms_sparse / 1e9
+    traffic, traffic_note = measured_traffic(cfg.name)
     out = {
         "metric": "sla_forward_effective_tflops",
         "value": eff_tflops,
@@ -148,8 +278,7 @@ def main():
                    "B": B, "H": H, "L": L, "D": D, "topk": cfg.topk, "T": T},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / PEAK_BF16_TFLOPS,
-                     "traffic": (sum(v for k_, v in MEASURED_TRAFFIC_BYTES[cfg.name].items() if k_ != "kernel")
-                                 if cfg.name in MEASURED_TRAFFIC_BYTES else None),
+                     "traffic": traffic, "traffic_note": traffic_note,
                      "traffic_unit": "HBM bytes per launch (fetch + write)", "kernel": "sparse_fwd_kernel<FUSED=true>",
                      "flops_per_launch": sparse_flops, "ms_per_launch": ms_sparse},
     }
@@ -205,6 +334,8 @@ def main():
         except (AssertionError, RuntimeError, NotImplementedError) as e:
             extra["sla_fwd_complement_mode_ms"] = None
             extra["complement_note"] = str(e)[:200]
+    if not args.no_extras and cfg.name == "cfg3":
+        extra.update(other_configs(torch, dev, max(args.steps // 10, 3)))
     if args.pmc_calibration:
         x = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
         y = torch.empty_like(x)

@@ -46,6 +46,42 @@ def time_ms(fn, warmup=5, iters=20):
     return e0.elapsed_time(e1) / iters
 
 
+def run(batch=2, heads=16, seq=32760, dim=128, sparsity=0.95, blkq=128, iters=20, warmup=5):
+    """Times the two modes; returns the two result dicts (``mode`` "fwd" and "bwd")."""
+    dev = torch.device("cuda:0")
+    torch.manual_seed(42)
+    shape = (batch, heads, seq, dim)
+    q, k, v = (torch.randn(shape, dtype=torch.bfloat16, device=dev, requires_grad=True) for _ in range(3))
+    do = torch.randn_like(v)
+    with torch.no_grad():
+        sparse_map, lut, real_topk = get_block_map(q, k, topk_ratio=1 - sparsity, BLKQ=blkq, BLKK=64)
+
+    def fwd():
+        return _attention.apply(q, k, v, sparse_map, lut, real_topk, blkq, 64), calc_linear(q, k, v)
+
+    def fwd_attention_only():
+        with torch.no_grad():
+            return _attention.apply(q, k, v, sparse_map, lut, real_topk, blkq, 64)
+
+    dense_flops = 4.0 * batch * heads * seq * seq * dim
+    common = {"B": batch, "H": heads, "L": seq, "D": dim, "sparsity": sparsity, "BLKQ": blkq, "BLKK": 64, "T": real_topk,
+              "dtype": "bf16", "data": "randn, seed 42"}
+    ms = time_ms(fwd, warmup=warmup, iters=iters)
+    ms_attn = time_ms(fwd_attention_only, warmup=warmup, iters=iters)
+    results = [{"mode": "fwd", "ms": ms, "effective_tflops": dense_flops / ms * 1e-9, "attention_kernel_ms": ms_attn,
+                **common}]
+    o_s, o_l = fwd()
+    o = o_s + o_l
+
+    def bwd():
+        q.grad = k.grad = v.grad = None
+        o.backward(do, retain_graph=True)
+
+    ms = time_ms(bwd, warmup=warmup, iters=iters)
+    results.append({"mode": "bwd", "ms": ms, "effective_tflops": 2.5 * dense_flops / ms * 1e-9, **common})
+    return results
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--batch", type=int, default=2)
@@ -58,37 +94,8 @@ def main():
     args = ap.parse_args()
     if not torch.cuda.is_available():
         sys.exit("evaluate/bench_kernel.py needs a GPU")
-    dev = torch.device("cuda:0")
-    torch.manual_seed(42)
-    shape = (args.batch, args.heads, args.seq, args.dim)
-    q, k, v = (torch.randn(shape, dtype=torch.bfloat16, device=dev, requires_grad=True) for _ in range(3))
-    do = torch.randn_like(v)
-    with torch.no_grad():
-        sparse_map, lut, real_topk = get_block_map(q, k, topk_ratio=1 - args.sparsity, BLKQ=args.blkq, BLKK=64)
-
-    def fwd():
-        return _attention.apply(q, k, v, sparse_map, lut, real_topk, args.blkq, 64), calc_linear(q, k, v)
-
-    def fwd_attention_only():
-        with torch.no_grad():
-            return _attention.apply(q, k, v, sparse_map, lut, real_topk, args.blkq, 64)
-
-    dense_flops = 4.0 * args.batch * args.heads * args.seq * args.seq * args.dim
-    common = {"B": args.batch, "H": args.heads, "L": args.seq, "D": args.dim, "sparsity": args.sparsity,
-              "BLKQ": args.blkq, "BLKK": 64, "T": real_topk, "dtype": "bf16", "data": "randn, seed 42"}
-    ms = time_ms(fwd, iters=args.iters)
-    ms_attn = time_ms(fwd_attention_only, iters=args.iters)
-    print(json.dumps({"mode": "fwd", "ms": ms, "effective_tflops": dense_flops / ms * 1e-9,
-                      "attention_kernel_ms": ms_attn, **common}))
-    o_s, o_l = fwd()
-    o = o_s + o_l
-
-    def bwd():
-        q.grad = k.grad = v.grad = None
-        o.backward(do, retain_graph=True)
-
-    ms = time_ms(bwd, iters=args.iters)
-    print(json.dumps({"mode": "bwd", "ms": ms, "effective_tflops": 2.5 * dense_flops / ms * 1e-9, **common}))
+    for r in run(args.batch, args.heads, args.seq, args.dim, args.sparsity, args.blkq, args.iters):
+        print(json.dumps(r))
 
 
 if __name__ == "__main__":

@@ -209,10 +209,13 @@ int sage_quant_qk(const void* q, const void* k, int dtype, int B, int H, int L, 
                   int64_t workspace_bytes, void* stream);
 
 /* SageSLA: per-channel FP8 e4m3 quantisation of v.  v_fp8 (B,H,L,D) e4m3fn bytes,
- * v_scale (B,H,D) fp32 = max_L|v| / 448.
+ * v_scale (B,H,D) fp32 = max_L|v| / v_range, v_fp8 = e4m3fn(v / v_scale), so |v_fp8| <= v_range.
+ * v_range in (0, 448]: the reference's call passes 2.25 (SageSLA/core.py:129, sized for fp16 accumulators of the
+ * PV product); this library's modules pass 448, the whole e4m3 range, because sage_sparse_attn_fwd accumulates
+ * in fp32.  sage_sparse_attn_fwd takes either: it only multiplies by v_scale at the end.
  * Replaces spas_sage_attn._fused.transpose_pad_permute_cuda + scale_fuse_quant_cuda,
  * SageSLA/core.py:123-129. */
-int sage_quant_v(const void* v, int dtype, int B, int H, int L, int D, uint8_t* v_fp8, float* v_scale,
+int sage_quant_v(const void* v, int dtype, int B, int H, int L, int D, uint8_t* v_fp8, float* v_scale, float v_range,
                  void* workspace, int64_t workspace_bytes, void* stream);
 
 /* SageSLA: everything the quantised attention kernel needs, in one call: the block map of
@@ -223,7 +226,7 @@ int sage_quant_v(const void* v, int dtype, int B, int H, int L, int D, uint8_t* 
  * Replaces get_block_map + k.mean + get_vanilla_qk_quant + the v quantisation, SageSLA/core.py:96-129. */
 int sage_prepare(const void* q, const void* k, const void* v, int dtype, int B, int H, int L, int D, int BLKQ,
                  int BLKK, int topk, int8_t* sparse_map, void* lut, int lut_elem_bytes, int8_t* q_int8, float* q_scale,
-                 int8_t* k_int8, float* k_scale, uint8_t* v_fp8, float* v_scale, void* workspace,
+                 int8_t* k_int8, float* k_scale, uint8_t* v_fp8, float* v_scale, float v_range, void* workspace,
                  int64_t workspace_bytes, void* stream);
 
 /* SageSLA: quantised block-sparse attention, INT8 QK^T and FP8 PV on the matrix cores.
@@ -242,9 +245,9 @@ int sage_sparse_attn_fwd(const int8_t* q_int8, const float* q_scale, const int8_
 int sage_prepare_strided(const void* q, const void* k, const void* v, const int64_t* qkv_strides, int dtype, int B, int H,
                          int L, int D, int BLKQ, int BLKK, int topk, int8_t* sparse_map, void* lut, int lut_elem_bytes,
                          int8_t* q_int8, float* q_scale, int8_t* k_int8, float* k_scale, uint8_t* v_fp8, float* v_scale,
-                         void* workspace, int64_t workspace_bytes, void* stream);
+                         float v_range, void* workspace, int64_t workspace_bytes, void* stream);
 int sage_quant_v_strided(const void* v, const int64_t* v_strides, int dtype, int B, int H, int L, int D, uint8_t* v_fp8,
-                         float* v_scale, void* workspace, int64_t workspace_bytes, void* stream);
+                         float* v_scale, float v_range, void* workspace, int64_t workspace_bytes, void* stream);
 int sla_linear_out_fwd_strided(const void* q, const int64_t* q_strides, const float* bias, const void* residual, void* out,
                                const int64_t* out_strides, int dtype, int fmap, int B, int H, int L, int D,
                                void* workspace, int64_t workspace_bytes, void* stream);

@@ -428,6 +428,7 @@ def sla_forward_autograd(q, k, v, weight, bias, sparse_map, fmap, BLKQ, BLKK,
 # --------------------------------------------------------------------------
 
 FP8_E4M3_MAX = 448.0
+SAGE_V_RANGE_REFERENCE = 2.25      # the constant the reference passes at SageSLA/core.py:129
 
 
 def sage_quant_qk(q, k, BLKQ=128, BLKK=64):
@@ -460,8 +461,9 @@ def sage_quant_v(v, fp8_max=FP8_E4M3_MAX):
     """Per-channel FP8 e4m3 quantisation of V (SageSLA/core.py:123-129).
 
     ``scale[b,h,d] = max_L |v| / fp8_max`` and ``v_fp8 = e4m3fn(v / scale)``.
-    The reference passes 2.25 as the range so that its fp16 accumulators stay
-    finite; with fp32 accumulation the full e4m3 range 448 is used here.
+    The reference passes ``fp8_max = 2.25`` (``SAGE_V_RANGE_REFERENCE``) so that
+    its fp16 accumulators stay finite; the default here is the full e4m3 range
+    448, which the HIP modules use because their PV product accumulates in fp32.
     Returns (v_fp8 float8_e4m3fn (B,H,L,D), v_scale fp32 (B,H,D)).
     """
     v32 = v.to(torch.float32)
@@ -471,19 +473,19 @@ def sage_quant_v(v, fp8_max=FP8_E4M3_MAX):
     return v8, scale
 
 
-def sage_sparse_attn_fwd(q, k, v, lut, BLKQ=128, BLKK=64, qk_scale=None, heads=None):
+def sage_sparse_attn_fwd(q, k, v, lut, BLKQ=128, BLKK=64, qk_scale=None, heads=None, v_range=FP8_E4M3_MAX):
     """Quantised block-sparse attention: INT8 QK^T, FP8 P and V, fp32 softmax.
 
     S = (q_int8 . k_int8) * q_scale * k_scale * qk_scale (exact int32 dot);
     softmax over the selected blocks; P scaled to the e4m3 range
-    (p * 448 rounded to e4m3fn), V per-channel e4m3fn; O = (P8 . V8) * v_scale / (448 * l).
-    The row sum l uses unrounded fp32 probabilities.
+    (p * 448 rounded to e4m3fn), V per-channel e4m3fn with range ``v_range``;
+    O = (P8 . V8) * v_scale / (448 * l).  The row sum l uses unrounded fp32 probabilities.
     """
     B, H, L, D = q.shape
     if qk_scale is None:
         qk_scale = D ** -0.5
     q8, qs, k8, ksc, _ = sage_quant_qk(q, k, BLKQ, BLKK)
-    v8, vs = sage_quant_v(v)
+    v8, vs = sage_quant_v(v, v_range)
     M = (L + BLKQ - 1) // BLKQ
     N = (L + BLKK - 1) // BLKK
     T = lut.shape[-1]

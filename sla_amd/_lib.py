@@ -53,12 +53,12 @@ SIGNATURES = {
                                        _I, _I, _I, _P, _I64, _P]),
     "sla_linear_bwd": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P, _I64, _P]),
     "sage_quant_qk": (_I, [_P, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _I64, _P]),
-    "sage_prepare": (_I, [_P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I64, _P]),
-    "sage_quant_v": (_I, [_P, _I, _I, _I, _I, _I, _P, _P, _P, _I64, _P]),
+    "sage_prepare": (_I, [_P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _I, _P, _P, _P, _P, _P, _P, _F, _P, _I64, _P]),
+    "sage_quant_v": (_I, [_P, _I, _I, _I, _I, _I, _P, _P, _F, _P, _I64, _P]),
     "sage_sparse_attn_fwd": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _P]),
-    "sage_prepare_strided": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I64,
-                                  _P]),
-    "sage_quant_v_strided": (_I, [_P, _P, _I, _I, _I, _I, _I, _P, _P, _P, _I64, _P]),
+    "sage_prepare_strided": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _I, _P, _P, _P, _P, _P, _P, _F, _P,
+                                  _I64, _P]),
+    "sage_quant_v_strided": (_I, [_P, _P, _I, _I, _I, _I, _I, _P, _P, _F, _P, _I64, _P]),
     "sla_linear_out_fwd_strided": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I64, _P]),
 }
 

@@ -560,7 +560,7 @@ static int block_map_entry(const void* q, const void* k, const int64_t* strides,
   if (rc) return rc;
   const int M = cdiv(L, BLKQ), N = cdiv(L, BLKK);
   SLA_REQUIRE(topk >= 0 && topk <= N, SLA_ERR_BAD_ARG, "topk=%d outside [0, %d]", topk, N);
-  SLA_REQUIRE(N <= 8192, SLA_ERR_UNSUPPORTED, "more than 8192 key blocks (%d)", N);
+  SLA_REQUIRE(N <= 4096, SLA_ERR_UNSUPPORTED, "more than 4096 key blocks (%d)", N);   // top-k rows of 4 waves in 64 KB of LDS
   SLA_REQUIRE((int64_t)BH * M < (1ll << 31), SLA_ERR_UNSUPPORTED, "too many query-block rows");
   SLA_REQUIRE(lut_elem_bytes == 4 || lut_elem_bytes == 8, SLA_ERR_BAD_ARG, "lut_elem_bytes must be 4 or 8, got %d",
               lut_elem_bytes);

@@ -33,8 +33,11 @@ int make_layout(const int64_t* strides, int B, int H, int L, int D, int elem_byt
   SLA_REQUIRE(sb % vec == 0 && sh % vec == 0 && sl % vec == 0, SLA_ERR_BAD_ARG,
               "strides (%lld, %lld, %lld) must be multiples of %lld elements (16-byte aligned rows)", (long long)sb,
               (long long)sh, (long long)sl, (long long)vec);
-  // rows of one head must not run into each other or into another head's rows of the same token
-  SLA_REQUIRE(sh >= D || sh >= (int64_t)L * sl, SLA_ERR_BAD_ARG, "head stride %lld overlaps rows of width D=%d", (long long)sh, D);
+  // rows of different heads must not overlap (the backward writes gradients through the same layout): either a
+  // head's rows end before the next head starts, or the heads are interleaved inside one token's row
+  SLA_REQUIRE(H == 1 || sh >= (int64_t)(L - 1) * sl + D || (sh >= D && sl >= (int64_t)(H - 1) * sh + D), SLA_ERR_BAD_ARG,
+              "strides (%lld, %lld, %lld): rows of different heads overlap (H=%d L=%d D=%d)", (long long)sb, (long long)sh,
+              (long long)sl, H, L, D);
   SLA_REQUIRE(((int64_t)(L - 1) * sl + D) * elem_bytes < (1ll << 32) - 65536, SLA_ERR_UNSUPPORTED,
               "one head spans 4 GiB or more with row stride %lld", (long long)sl);
   *out = RowLayout{sb, sh, sl, H};

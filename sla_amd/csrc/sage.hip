@@ -6,7 +6,7 @@
 // so the scheme below follows its published description, not its code:
 //   q_int8 = rint(q / sq), sq = max|q| / 127 over each block of BLKQ rows;
 //   k_int8 = rint((k - mean_L k) / sk), sk per block of BLKK rows;
-//   v_fp8  = e4m3(v / sv), sv[d] = max_L |v[:, d]| / 448;
+//   v_fp8  = e4m3(v / sv), sv[d] = max_L |v[:, d]| / v_range (448 by default; the reference's call passes 2.25);
 //   S = (q_int8 . k_int8) * sq * sk * scale ; P = softmax numerators over the selected blocks ;
 //   O = (e4m3(c P) . v_fp8) * sv / sum(e4m3(c P)), c = 112 with P <= 4 (reference maximum lagging by <= 2).
 // The look-up table of the bf16 path is used as is (no delta encoding is needed here).
@@ -151,7 +151,7 @@ __global__ __launch_bounds__(256) void v_amax_partial_kernel(const uint16_t* __r
 // over chunks cg, cg + 16, ...; the 16 partial maxima per column meet in LDS.  (Small workgroups: the launch has to
 // find room beside the memory-bound kernels of the other stream.)
 __global__ __launch_bounds__(256) void v_scale_kernel(const float* __restrict__ part, float* __restrict__ v_scale, int nchunk,
-                                                     int D) {
+                                                     int D, float v_range) {
   __shared__ float sm[256];
   const int bh = blockIdx.y, tid = threadIdx.x;
   const int d = blockIdx.x * 16 + (tid & 15), cg = tid >> 4;
@@ -161,7 +161,7 @@ __global__ __launch_bounds__(256) void v_scale_kernel(const float* __restrict__ 
   __syncthreads();
   if (tid < 16) {
     for (int j = 1; j < 16; ++j) a = fmaxf(a, sm[j * 16 + tid]);
-    v_scale[(size_t)bh * D + d] = fmaxf(a, 1e-30f) / 448.0f;
+    v_scale[(size_t)bh * D + d] = fmaxf(a, 1e-30f) / v_range;
   }
 }
 
@@ -490,6 +490,12 @@ static int validate_sage(int dtype, int B, int H, int L, int D, int BLKQ, int BL
   return SLA_OK;
 }
 
+// range of the e4m3 values v is quantised to: the format's largest finite value (448) or less
+static int validate_v_range(float v_range) {
+  SLA_REQUIRE(v_range > 0.f && v_range <= 448.f, SLA_ERR_BAD_ARG, "v_range=%g outside (0, 448]", (double)v_range);
+  return SLA_OK;
+}
+
 template <typename Tag, int D>
 static int quant_qk_impl(const void* q, const void* k, int dtype, int BH, int L, int8_t* q8, float* qs, int8_t* k8,
                          float* ks, char* ws, hipStream_t st) {
@@ -508,14 +514,15 @@ static int quant_qk_impl(const void* q, const void* k, int dtype, int BH, int L,
 // and the quantiser both subtract it) and the quantisers emit the block means the scores are made of, so
 // q is read once and k twice instead of q twice and k four times.
 template <typename Tag, int D>
-static int quant_v_impl(const void* v, const RowLayout& lay, int BH, int L, uint8_t* v8, float* vs, char* ws, hipStream_t st);
+static int quant_v_impl(const void* v, const RowLayout& lay, int BH, int L, uint8_t* v8, float* vs, float v_range, char* ws,
+                        hipStream_t st);
 
 // (lay: where the rows of q, k, v lie; the quantised outputs are always contiguous (B, H, L, D))
 template <typename Tag, int D>
 static int prepare_impl(const void* q, const void* k, const void* v, const RowLayout& lay, int dtype, int BH, int L, int topk,
                         int8_t* sparse_map,
-                        void* lut, int lut64, int8_t* q8, float* qs, int8_t* k8, float* ks, uint8_t* v8, float* vs, char* ws,
-                        hipStream_t st) {
+                        void* lut, int lut64, int8_t* q8, float* qs, int8_t* k8, float* ks, uint8_t* v8, float* vs, float v_range,
+                        char* ws, hipStream_t st) {
   const SageWs w = sage_ws(BH, L, D);
   const SagePrepWs p = sage_prep_ws(BH, L, D);
   const int M = cdiv(L, 128), N = cdiv(L, 64);
@@ -529,16 +536,17 @@ static int prepare_impl(const void* q, const void* k, const void* v, const RowLa
   launch_map_from_pooled(dtype, pq, pk, ws + p.score, BH, M, N, D, topk, sparse_map, lut, lut64, st);
   int rc = check_launch("sage_prepare");
   if (rc || !v) return rc;
-  return quant_v_impl<Tag, D>(v, lay, BH, L, v8, vs, ws, st);
+  return quant_v_impl<Tag, D>(v, lay, BH, L, v8, vs, v_range, ws, st);
 }
 
 template <typename Tag, int D>
-static int quant_v_impl(const void* v, const RowLayout& lay, int BH, int L, uint8_t* v8, float* vs, char* ws, hipStream_t st) {
+static int quant_v_impl(const void* v, const RowLayout& lay, int BH, int L, uint8_t* v8, float* vs, float v_range, char* ws,
+                        hipStream_t st) {
   const SageWs w = sage_ws(BH, L, D);
   float* part = (float*)(ws + w.v_part);
   hipLaunchKernelGGL((v_amax_partial_kernel<Tag, D>), dim3(w.nchunk_v, BH), dim3(256), 0, st, (const uint16_t*)v, lay, part, L,
                      w.rows_per_chunk_v);
-  hipLaunchKernelGGL(v_scale_kernel, dim3(D / 16, BH), dim3(256), 0, st, part, vs, w.nchunk_v, D);
+  hipLaunchKernelGGL(v_scale_kernel, dim3(D / 16, BH), dim3(256), 0, st, part, vs, w.nchunk_v, D, v_range);
   constexpr int RPP = 256 / (D / 8);
   hipLaunchKernelGGL((v_quant_fp8_kernel<Tag, D>), dim3(cdiv(L, RPP), BH), dim3(256), 0, st, (const uint16_t*)v, lay, vs, v8,
                      L);
@@ -571,16 +579,18 @@ extern "C" int sage_quant_qk(const void* q, const void* k, int dtype, int B, int
 
 static int prepare_entry(const void* q, const void* k, const void* v, const int64_t* qkv_strides, int dtype, int B, int H, int L,
                          int D, int BLKQ, int BLKK, int topk, int8_t* sparse_map, void* lut, int lut_elem_bytes, int8_t* q_int8,
-                         float* q_scale, int8_t* k_int8, float* k_scale, uint8_t* v_fp8, float* v_scale, void* workspace,
-                         int64_t workspace_bytes, void* stream) {
+                         float* q_scale, int8_t* k_int8, float* k_scale, uint8_t* v_fp8, float* v_scale, float v_range,
+                         void* workspace, int64_t workspace_bytes, void* stream) {
   int rc = validate_sage(dtype, B, H, L, D, BLKQ, BLKK);
+  if (rc) return rc;
+  rc = validate_v_range(v_range);
   if (rc) return rc;
   RowLayout lay;
   rc = make_layout(qkv_strides, B, H, L, D, 2, &lay);
   if (rc) return rc;
   const int N = cdiv(L, 64);
   SLA_REQUIRE(topk >= 0 && topk <= N, SLA_ERR_BAD_ARG, "topk=%d outside [0, %d]", topk, N);
-  SLA_REQUIRE(N <= 8192, SLA_ERR_UNSUPPORTED, "more than 8192 key blocks (%d)", N);
+  SLA_REQUIRE(N <= 4096, SLA_ERR_UNSUPPORTED, "more than 4096 key blocks (%d)", N);
   SLA_REQUIRE(lut_elem_bytes == 4 || lut_elem_bytes == 8, SLA_ERR_BAD_ARG, "lut_elem_bytes must be 4 or 8, got %d",
               lut_elem_bytes);
   // (v, v_fp8 and v_scale may all three be NULL: the caller then quantises v itself with sage_quant_v, e.g. on another
@@ -599,7 +609,7 @@ static int prepare_entry(const void* q, const void* k, const void* v, const int6
   const int lut64 = lut_elem_bytes == 8;
 #define SLA_PREP_CASE(TAG, DD) \
   return prepare_impl<TAG, DD>(q, k, v, lay, dtype, BH, L, topk, sparse_map, lut, lut64, q_int8, q_scale, k_int8, k_scale, \
-                               v_fp8, v_scale, ws, st)
+                               v_fp8, v_scale, v_range, ws, st)
   if (dtype == SLA_BF16) {
     if (D == 128) SLA_PREP_CASE(bf16_tag, 128);
     SLA_PREP_CASE(bf16_tag, 64);
@@ -611,24 +621,27 @@ static int prepare_entry(const void* q, const void* k, const void* v, const int6
 
 extern "C" int sage_prepare(const void* q, const void* k, const void* v, int dtype, int B, int H, int L, int D, int BLKQ,
                             int BLKK, int topk, int8_t* sparse_map, void* lut, int lut_elem_bytes, int8_t* q_int8,
-                            float* q_scale, int8_t* k_int8, float* k_scale, uint8_t* v_fp8, float* v_scale, void* workspace,
-                            int64_t workspace_bytes, void* stream) {
+                            float* q_scale, int8_t* k_int8, float* k_scale, uint8_t* v_fp8, float* v_scale, float v_range,
+                            void* workspace, int64_t workspace_bytes, void* stream) {
   return prepare_entry(q, k, v, nullptr, dtype, B, H, L, D, BLKQ, BLKK, topk, sparse_map, lut, lut_elem_bytes, q_int8, q_scale,
-                       k_int8, k_scale, v_fp8, v_scale, workspace, workspace_bytes, stream);
+                       k_int8, k_scale, v_fp8, v_scale, v_range, workspace, workspace_bytes, stream);
 }
 
 extern "C" int sage_prepare_strided(const void* q, const void* k, const void* v, const int64_t* qkv_strides, int dtype, int B,
                                     int H, int L, int D, int BLKQ, int BLKK, int topk, int8_t* sparse_map, void* lut,
                                     int lut_elem_bytes, int8_t* q_int8, float* q_scale, int8_t* k_int8, float* k_scale,
-                                    uint8_t* v_fp8, float* v_scale, void* workspace, int64_t workspace_bytes, void* stream) {
+                                    uint8_t* v_fp8, float* v_scale, float v_range, void* workspace,
+                                    int64_t workspace_bytes, void* stream) {
   SLA_REQUIRE(qkv_strides, SLA_ERR_BAD_ARG, "null strides");
   return prepare_entry(q, k, v, qkv_strides, dtype, B, H, L, D, BLKQ, BLKK, topk, sparse_map, lut, lut_elem_bytes, q_int8,
-                       q_scale, k_int8, k_scale, v_fp8, v_scale, workspace, workspace_bytes, stream);
+                       q_scale, k_int8, k_scale, v_fp8, v_scale, v_range, workspace, workspace_bytes, stream);
 }
 
 static int quant_v_entry(const void* v, const int64_t* v_strides, int dtype, int B, int H, int L, int D, uint8_t* v_fp8,
-                         float* v_scale, void* workspace, int64_t workspace_bytes, void* stream) {
+                         float* v_scale, float v_range, void* workspace, int64_t workspace_bytes, void* stream) {
   int rc = validate_sage(dtype, B, H, L, D, 128, 64);
+  if (rc) return rc;
+  rc = validate_v_range(v_range);
   if (rc) return rc;
   RowLayout lay;
   rc = make_layout(v_strides, B, H, L, D, 2, &lay);
@@ -641,22 +654,23 @@ static int quant_v_entry(const void* v, const int64_t* v_strides, int dtype, int
   hipStream_t st = (hipStream_t)stream;
   char* ws = (char*)workspace;
   if (dtype == SLA_BF16) {
-    if (D == 128) return quant_v_impl<bf16_tag, 128>(v, lay, BH, L, v_fp8, v_scale, ws, st);
-    return quant_v_impl<bf16_tag, 64>(v, lay, BH, L, v_fp8, v_scale, ws, st);
+    if (D == 128) return quant_v_impl<bf16_tag, 128>(v, lay, BH, L, v_fp8, v_scale, v_range, ws, st);
+    return quant_v_impl<bf16_tag, 64>(v, lay, BH, L, v_fp8, v_scale, v_range, ws, st);
   }
-  if (D == 128) return quant_v_impl<f16_tag, 128>(v, lay, BH, L, v_fp8, v_scale, ws, st);
-  return quant_v_impl<f16_tag, 64>(v, lay, BH, L, v_fp8, v_scale, ws, st);
+  if (D == 128) return quant_v_impl<f16_tag, 128>(v, lay, BH, L, v_fp8, v_scale, v_range, ws, st);
+  return quant_v_impl<f16_tag, 64>(v, lay, BH, L, v_fp8, v_scale, v_range, ws, st);
 }
 
 extern "C" int sage_quant_v(const void* v, int dtype, int B, int H, int L, int D, uint8_t* v_fp8, float* v_scale,
-                            void* workspace, int64_t workspace_bytes, void* stream) {
-  return quant_v_entry(v, nullptr, dtype, B, H, L, D, v_fp8, v_scale, workspace, workspace_bytes, stream);
+                            float v_range, void* workspace, int64_t workspace_bytes, void* stream) {
+  return quant_v_entry(v, nullptr, dtype, B, H, L, D, v_fp8, v_scale, v_range, workspace, workspace_bytes, stream);
 }
 
 extern "C" int sage_quant_v_strided(const void* v, const int64_t* v_strides, int dtype, int B, int H, int L, int D,
-                                    uint8_t* v_fp8, float* v_scale, void* workspace, int64_t workspace_bytes, void* stream) {
+                                    uint8_t* v_fp8, float* v_scale, float v_range, void* workspace,
+                                    int64_t workspace_bytes, void* stream) {
   SLA_REQUIRE(v_strides, SLA_ERR_BAD_ARG, "null strides");
-  return quant_v_entry(v, v_strides, dtype, B, H, L, D, v_fp8, v_scale, workspace, workspace_bytes, stream);
+  return quant_v_entry(v, v_strides, dtype, B, H, L, D, v_fp8, v_scale, v_range, workspace, workspace_bytes, stream);
 }
 
 extern "C" int sage_sparse_attn_fwd(const int8_t* q_int8, const float* q_scale, const int8_t* k_int8,

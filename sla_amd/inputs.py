@@ -97,6 +97,35 @@ def make_inputs(cfg: Config, seed: int = 0, H: int | None = None, with_do: bool 
     return out
 
 
+def make_inputs_on_device(cfg: Config, device, seed: int = 0, with_do: bool = False):
+    """The structured generator of :func:`make_inputs` run on the GPU (same field definition, the device's own random
+    streams, so not the same values): for the large configurations, where the CPU generator needs minutes.
+    Returns ``(q, k, v, do)`` on ``device``; ``do`` is None unless ``with_do``."""
+    assert cfg.grid is not None
+    g = torch.Generator(device=device).manual_seed(seed)
+    Fg, Y, X = cfg.grid
+    f = torch.arange(Fg, device=device, dtype=torch.float32).view(Fg, 1, 1) / Fg
+    y = torch.arange(Y, device=device, dtype=torch.float32).view(1, Y, 1) / Y
+    x = torch.arange(X, device=device, dtype=torch.float32).view(1, 1, X) / X
+    amp = 1.0 / math.sqrt(len(_FREQS) / 2.0)
+    shape = (cfg.B, cfg.H, cfg.L, cfg.D)
+    q = torch.empty(shape, device=device, dtype=cfg.dtype)
+    k = torch.empty(shape, device=device, dtype=cfg.dtype)
+    for b in range(cfg.B):
+        for h in range(cfg.H):
+            fld = torch.zeros(cfg.L, cfg.D, device=device)
+            for af, ay, ax in _FREQS:
+                arg = (2 * math.pi) * (af * f + ay * y + ax * x).reshape(cfg.L, 1)
+                fld += amp * torch.sin(arg + torch.rand(1, cfg.D, device=device, generator=g) * (2 * math.pi))
+            q[b, h] = 0.5 * torch.randn(cfg.L, cfg.D, device=device, generator=g) + fld
+            k[b, h] = 0.5 * torch.randn(cfg.L, cfg.D, device=device, generator=g) + fld
+            if cfg.k_bias_std > 0:
+                k[b, h] += cfg.k_bias_std * torch.randn(1, cfg.D, device=device, generator=g)
+    v = torch.randn(shape, device=device, generator=g).to(cfg.dtype)
+    do = torch.randn(shape, device=device, generator=g).to(cfg.dtype) if with_do else None
+    return q, k, v, do
+
+
 def make_proj(D: int, seed: int = 1):
     """Seeded non-zero proj_l parameters (weight (D,D), bias (D,)) in fp32.
 

@@ -15,6 +15,9 @@ from .linear import linear_out_fwd
 from .module import FEATURE_MAPS, _StateBuild
 
 SAGE_BLKQ, SAGE_BLKK = 128, 64
+# Range of the e4m3 values v is quantised to.  The reference's call passes 2.25 (SageSLA/core.py:129), which keeps the
+# fp16 accumulators of its PV product finite; the kernel here accumulates in fp32 and uses the whole e4m3 range.
+V_RANGE_E4M3, V_RANGE_REFERENCE = 448.0, 2.25
 
 
 def quant_qk(q, k):
@@ -35,9 +38,9 @@ def quant_qk(q, k):
     return q8, qs, k8, ks
 
 
-def quant_v(v):
+def quant_v(v, v_range=V_RANGE_E4M3):
     """Per-channel FP8 e4m3 v (contiguous or a row-contiguous view).  Returns (v_fp8 (B,H,L,D) float8_e4m3fn, contiguous,
-    v_scale (B,H,D) fp32)."""
+    v_scale (B,H,D) fp32 = max_L|v| / v_range).  ``v_range=2.25`` is the reference's constant (SageSLA/core.py:129)."""
     _lib.require_gpu(v)
     B, H, L, D = v.shape
     dt = _lib.dtype_code(v.dtype)
@@ -45,17 +48,17 @@ def quant_v(v):
     v8 = torch.empty((B, H, L, D), dtype=torch.float8_e4m3fn, device=v.device)
     vs = torch.empty((B, H, D), dtype=torch.float32, device=v.device)
     if v.is_contiguous():
-        rc = _lib.load().sage_quant_v(v.data_ptr(), dt, B, H, L, D, v8.data_ptr(), vs.data_ptr(), ws.data_ptr(), ws.numel(),
-                                      _lib.stream_ptr(v.device))
+        rc = _lib.load().sage_quant_v(v.data_ptr(), dt, B, H, L, D, v8.data_ptr(), vs.data_ptr(), float(v_range), ws.data_ptr(),
+                                      ws.numel(), _lib.stream_ptr(v.device))
     else:
         assert _lib.row_strided(v), "v must be contiguous or a row-contiguous view"
         rc = _lib.load().sage_quant_v_strided(v.data_ptr(), _lib.strides_arg(v), dt, B, H, L, D, v8.data_ptr(), vs.data_ptr(),
-                                              ws.data_ptr(), ws.numel(), _lib.stream_ptr(v.device))
+                                              float(v_range), ws.data_ptr(), ws.numel(), _lib.stream_ptr(v.device))
     _lib.check(rc)
     return v8, vs
 
 
-def sage_prepare(q, k, v, topk_ratio):
+def sage_prepare(q, k, v, topk_ratio, v_range=V_RANGE_E4M3):
     """Block map, INT8 q / k and FP8 v in one library call (q, k, v already in the compute dtype; contiguous, or
     row-contiguous views with common strides: the quantised tensors are contiguous (B, H, L, D) either way).
 
@@ -90,7 +93,7 @@ def sage_prepare(q, k, v, topk_ratio):
         vs = torch.empty((B, H, D), dtype=torch.float32, device=dev)
     tail = (dt, B, H, L, D, SAGE_BLKQ, SAGE_BLKK, T, sparse_map.data_ptr(), lut.data_ptr(), 8, q8.data_ptr(), qs.data_ptr(),
             k8.data_ptr(), ks.data_ptr(), None if v is None else v8.data_ptr(), None if v is None else vs.data_ptr(),
-            ws.data_ptr(), ws.numel(), _lib.stream_ptr(dev))
+            float(v_range), ws.data_ptr(), ws.numel(), _lib.stream_ptr(dev))
     vp = None if v is None else v.data_ptr()
     if contiguous:
         rc = _lib.load().sage_prepare(q.data_ptr(), k.data_ptr(), vp, *tail)

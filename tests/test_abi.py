@@ -102,8 +102,13 @@ def test_other_entry_points_validate():
                                    64, 1, 0.1, FAKE, 8, None) == _lib.ERR_WORKSPACE
     assert lib.sage_quant_qk(FAKE, FAKE, 1, 1, 1, 128, 128, 64, 64, FAKE, FAKE, FAKE, FAKE, FAKE, 1 << 30, None) == _lib.ERR_UNSUPPORTED
     assert "BLKQ=128" in _lib.last_error()
-    assert lib.sage_quant_v(FAKE, 1, 1, 1, 128, 32, FAKE, FAKE, FAKE, 1 << 30, None) == _lib.ERR_UNSUPPORTED
+    assert lib.sage_quant_v(FAKE, 1, 1, 1, 128, 32, FAKE, FAKE, 448.0, FAKE, 1 << 30, None) == _lib.ERR_UNSUPPORTED
     assert "headdim" in _lib.last_error()
+    # range of the e4m3 values: (0, 448]; 2.25 is the reference's constant (SageSLA/core.py:129)
+    for bad in (0.0, -1.0, 449.0, float("nan")):
+        assert lib.sage_quant_v(FAKE, 1, 1, 1, 128, 128, FAKE, FAKE, bad, FAKE, 1 << 30, None) == _lib.ERR_BAD_ARG
+        assert "v_range" in _lib.last_error()
+    assert lib.sage_quant_v(FAKE, 1, 1, 1, 128, 128, FAKE, FAKE, 2.25, FAKE, 8, None) == _lib.ERR_WORKSPACE
     assert lib.sage_sparse_attn_fwd(FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, 8, FAKE, 1, 1, 1, 128, 128, 128, 64, 9, 0.1,
                                     None) == _lib.ERR_BAD_ARG
     # strided variants: strides are {batch, head, row} in elements, checked before anything is launched
@@ -115,6 +120,10 @@ def test_other_entry_points_validate():
     assert bm(st(65536, 128, 100)) == _lib.ERR_BAD_ARG          # row stride below D
     assert bm(st(65536, 128, 260)) == _lib.ERR_BAD_ARG and "16-byte" in _lib.last_error()
     assert bm(st(1 << 40, 128, 1 << 30)) == _lib.ERR_UNSUPPORTED and "4 GiB" in _lib.last_error()
+    # heads whose rows alias each other: head stride D with row stride D puts row l of head 1 on row l + 1 of head 0
+    assert bm(st(65536, 128, 128)) == _lib.ERR_BAD_ARG and "overlap" in _lib.last_error()
+    assert bm(st(65536, 128, 136)) == _lib.ERR_BAD_ARG and "overlap" in _lib.last_error()     # interleaved, row too short
+    assert bm(st(65536, 256 * 128 - 8, 128)) == _lib.ERR_BAD_ARG and "overlap" in _lib.last_error()  # disjoint but 8 short
     assert lib.sla_linear_state_fwd_strided(FAKE, FAKE, st(65536, 128, 257), FAKE, 1, 0, 1, 2, 256, 128, FAKE, 1 << 30,
                                             None) == _lib.ERR_BAD_ARG
     assert lib.sla_sparse_attn_linear_fwd_strided(FAKE, FAKE, FAKE, st(65536, 128, 256), FAKE, 8, FAKE, 1 << 30, FAKE, None,
@@ -124,16 +133,16 @@ def test_other_entry_points_validate():
                                           FAKE, 1 << 30, None) == _lib.ERR_BAD_ARG
     assert lib.sla_linear_out_fwd_strided(FAKE, None, FAKE, None, FAKE, st(65536, 128, 256), 1, 0, 1, 2, 256, 128, FAKE, 1 << 30,
                                           None) == _lib.ERR_BAD_ARG and "strides" in _lib.last_error()
-    assert lib.sage_quant_v_strided(FAKE, st(65536, 128, 260), 1, 1, 2, 256, 128, FAKE, FAKE, FAKE, 1 << 30,
+    assert lib.sage_quant_v_strided(FAKE, st(65536, 128, 260), 1, 1, 2, 256, 128, FAKE, FAKE, 448.0, FAKE, 1 << 30,
                                     None) == _lib.ERR_BAD_ARG and "16-byte" in _lib.last_error()
     assert lib.sage_prepare_strided(FAKE, FAKE, None, st(65536, 128, 64), 1, 1, 2, 256, 128, 128, 64, 1, FAKE, FAKE, 8, FAKE, FAKE,
-                                    FAKE, FAKE, None, None, FAKE, 1 << 30, None) == _lib.ERR_BAD_ARG
+                                    FAKE, FAKE, None, None, 448.0, FAKE, 1 << 30, None) == _lib.ERR_BAD_ARG
     # one-call SageSLA preparation: block sizes, topk range and workspace are checked before any launch
     # (v and its two outputs may be left out together, not separately)
     assert lib.sage_prepare(FAKE, FAKE, None, 1, 1, 1, 256, 128, 128, 64, 2, FAKE, FAKE, 8, FAKE, FAKE, FAKE, FAKE, FAKE, None,
-                            FAKE, 1 << 30, None) == _lib.ERR_BAD_ARG
+                            448.0, FAKE, 1 << 30, None) == _lib.ERR_BAD_ARG
     prep = lambda BLKQ, topk, ws: lib.sage_prepare(FAKE, FAKE, FAKE, 1, 1, 1, 256, 128, BLKQ, 64, topk, FAKE, FAKE, 8, FAKE,  # noqa: E731
-                                                   FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, ws, None)
+                                                   FAKE, FAKE, FAKE, FAKE, FAKE, 448.0, FAKE, ws, None)
     assert prep(64, 1, 1 << 30) == _lib.ERR_UNSUPPORTED
     assert prep(128, 5, 1 << 30) == _lib.ERR_BAD_ARG and "topk" in _lib.last_error()
     assert prep(128, 2, 8) == _lib.ERR_WORKSPACE

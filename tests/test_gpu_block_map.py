@@ -98,3 +98,15 @@ def test_negative_scores_and_wide_rows(dev, dtype):
         q = (torch.rand(1, 1, L, 32, generator=g) + 0.5).to(dtype)
         k = -(torch.rand(1, 1, L, 32, generator=g) * torch.linspace(0.5, 2.0, L).view(1, 1, L, 1) + 0.5).to(dtype)
         _compare(q, k, ratio, 64, 64, dev)
+
+
+def test_widest_supported_row(dev):
+    # 4096 key blocks is the limit of the top-k kernel (the keys of four rows share 64 KB of LDS); 4097 is refused
+    g = torch.Generator().manual_seed(78)
+    L = 64 * 4096
+    q = (torch.rand(1, 1, L, 32, generator=g) - 0.3).to(torch.bfloat16)
+    k = (torch.rand(1, 1, L, 32, generator=g) * torch.linspace(0.5, 2.0, L).view(1, 1, L, 1) - 0.6).to(torch.bfloat16)
+    _compare(q, k, 0.01, 128, 64, dev)
+    with pytest.raises(AssertionError, match="4096"):
+        get_block_map(torch.zeros(1, 1, L + 1, 32, dtype=torch.bfloat16, device=dev),
+                      torch.zeros(1, 1, L + 1, 32, dtype=torch.bfloat16, device=dev), 0.01, 128, 64)

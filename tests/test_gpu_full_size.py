@@ -61,29 +61,8 @@ def test_rows_are_convex_combinations(dev, full):
 # whose offsets are the largest the kernels form.
 # ---------------------------------------------------------------------------------------------------------------
 def _device_inputs(cfg, dev, seed, with_do):
-    import math
-    g = torch.Generator(device=dev).manual_seed(seed)
-    Fg, Y, X = cfg.grid
-    f = torch.arange(Fg, device=dev, dtype=torch.float32).view(Fg, 1, 1) / Fg
-    y = torch.arange(Y, device=dev, dtype=torch.float32).view(1, Y, 1) / Y
-    x = torch.arange(X, device=dev, dtype=torch.float32).view(1, 1, X) / X
-    freqs = ((1, 0, 0), (0, 1, 0), (0, 0, 1), (1, 1, 0), (0, 1, 1), (2, 0, 1))
-    shape = (cfg.B, cfg.H, cfg.L, cfg.D)
-    q = torch.empty(shape, device=dev, dtype=cfg.dtype)
-    k = torch.empty(shape, device=dev, dtype=cfg.dtype)
-    for b in range(cfg.B):
-        for h in range(cfg.H):
-            fld = torch.zeros(cfg.L, cfg.D, device=dev)
-            for af, ay, ax in freqs:
-                arg = (2 * math.pi) * (af * f + ay * y + ax * x).reshape(cfg.L, 1)
-                fld += torch.sin(arg + torch.rand(1, cfg.D, device=dev, generator=g) * (2 * math.pi)) / math.sqrt(3.0)
-            q[b, h] = 0.5 * torch.randn(cfg.L, cfg.D, device=dev, generator=g) + fld
-            k[b, h] = 0.5 * torch.randn(cfg.L, cfg.D, device=dev, generator=g) + fld
-            if cfg.k_bias_std > 0:
-                k[b, h] += cfg.k_bias_std * torch.randn(1, cfg.D, device=dev, generator=g)
-    v = torch.randn(shape, device=dev, generator=g).to(cfg.dtype)
-    do = torch.randn(shape, device=dev, generator=g).to(cfg.dtype) if with_do else None
-    return q, k, v, do
+    from sla_amd.inputs import make_inputs_on_device
+    return make_inputs_on_device(cfg, dev, seed, with_do)
 
 
 def _check_map(m, lut, T, N):

@@ -110,3 +110,29 @@ def test_p_dtype_rounding_is_small_and_l_unrounded():
     o1, _ = O.sparse_attn_fwd_gather(q, k, v, lut, 64, 64)
     o2, _ = O.sparse_attn_fwd_gather(q, k, v, lut, 64, 64, p_dtype=torch.bfloat16)
     assert 0 < (o1 - o2).abs().max() < 5e-3
+
+
+def test_qk_scale_argument():
+    """``qk_scale`` (kernel.py:242, 251-252): the library attention with ``scale=`` when every block is selected;
+    and doubling the scale is the same as doubling q (exact in floating point), which fixes the forward, lse and
+    the factor of every gradient."""
+    g = torch.Generator().manual_seed(31)
+    q, k, v, do = (torch.randn(1, 2, 200, 32, generator=g) for _ in range(4))
+    full = torch.ones(1, 2, 4, 4, dtype=torch.int8)
+    o, lse = O.sparse_attn_fwd_dense(q, k, v, full, 64, 64, qk_scale=0.07)
+    sd = torch.nn.functional.scaled_dot_product_attention(q.double(), k.double(), v.double(), scale=0.07)
+    assert (o - sd).abs().max() < 1e-12
+    m, lut, T = O.get_block_map(q, k, 0.5, 64, 64)
+    s0 = 32 ** -0.5
+    a, lse_a = O.sparse_attn_fwd_dense(q, k, v, m, 64, 64, qk_scale=2 * s0)
+    b, lse_b = O.sparse_attn_fwd_dense(2 * q, k, v, m, 64, 64)
+    assert torch.equal(a, b) and torch.equal(lse_a, lse_b)
+    ag, _ = O.sparse_attn_fwd_gather(q, k, v, lut, 64, 64, qk_scale=2 * s0, dtype=torch.float64)
+    assert (ag - a).abs().max() < 1e-12
+    ga = O.sparse_attn_bwd_dense(q, k, v, a, do, lse_a, m, 64, 64, qk_scale=2 * s0)
+    gb = O.sparse_attn_bwd_dense(2 * q, k, v, b, do, lse_b, m, 64, 64)
+    assert (ga[0] - 2 * gb[0]).abs().max() < 1e-12       # d/dq f(2q) = 2 f'(2q)
+    assert (ga[1] - gb[1]).abs().max() < 1e-12 and (ga[2] - gb[2]).abs().max() < 1e-12
+    gg = O.sparse_attn_bwd_gather(q, k, v, a, do, lse_a, lut, 64, 64, qk_scale=2 * s0, dtype=torch.float64)
+    for x, y in zip(gg, ga):
+        assert (x - y).abs().max() < 1e-10
