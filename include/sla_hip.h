@@ -79,6 +79,18 @@ int sla_block_map_fwd(const void* q, const void* k, int dtype, int B, int H, int
                       int topk, void* workspace, int64_t workspace_bytes, int8_t* sparse_map, void* lut,
                       int lut_elem_bytes, void* stream);
 
+/* sla_block_map_fwd for callers that cannot allocate device memory and have no workspace to lend (code under HIP
+ * graph capture, serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same kernels
+ * and results as sla_block_map_fwd; the workspace is a fixed array of SLA_STATIC_SCRATCH_BYTES in device memory that
+ * every GPU the library runs on holds until the process ends.  Problems whose sla_workspace_bytes(SLA_WS_BLOCK_MAP,
+ * ...) exceeds that size are refused with SLA_ERR_WORKSPACE (B1 H12 L32760 D128 64/64 in bf16 needs 12.7 MB and fits).
+ * Calls no hipMalloc / hipFree.  The first call on a GPU looks up the array's device address (make it once outside a
+ * graph capture); the GPU that `stream` belongs to must be the current device.  All calls on one GPU share the array:
+ * calls that overlap in time on one GPU (different streams) race; nothing in it needs clearing between calls. */
+#define SLA_STATIC_SCRATCH_BYTES (16u << 20)
+int sla_block_map_fwd_static(const void* q, const void* k, int dtype, int B, int H, int L, int D, int BLKQ, int BLKK,
+                             int topk, int8_t* sparse_map, void* lut, int lut_elem_bytes, void* stream);
+
 /* Block-sparse FlashAttention forward over the look-up table.
  * o (B,H,L,D) in `dtype`, lse (B,H,L) fp32 = m + log2(l) in qk_scale*log2(e) units.
  * BLKQ in {64,128}, BLKK == 64, D in {64,128}, dtype bf16 or f16.

@@ -20,6 +20,7 @@ FMAP = {"elu": 0, "relu": 1, "softmax": 2}
 BWD_ACCUMULATE, BWD_STATES_READY = 1, 2
 
 ERR_BAD_ARG, ERR_UNSUPPORTED, ERR_LAUNCH, ERR_WORKSPACE = -1, -2, -3, -4
+STATIC_SCRATCH_BYTES = 16 << 20
 
 _c = ctypes
 _P, _I, _F, _I64 = _c.c_void_p, _c.c_int, _c.c_float, _c.c_int64
@@ -31,6 +32,7 @@ SIGNATURES = {
     "sla_workspace_bytes": (_I64, [_I] * 9),
     "sla_mean_pool": (_I, [_P, _P, _I, _I, _I, _I, _I, _P]),
     "sla_block_map_fwd": (_I, [_P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _I64, _P, _P, _I, _P]),
+    "sla_block_map_fwd_static": (_I, [_P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _I, _P]),
     "sla_block_map_fwd_strided": (_I, [_P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _I64, _P, _P, _I, _P]),
     "sla_linear_state_fwd_strided": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I64, _P]),
     "sla_sparse_attn_linear_fwd_strided": (_I, [_P, _P, _P, _P, _P, _I, _P, _I64, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I,

@@ -13,6 +13,8 @@
 // Selection is by (score descending, index ascending); -0.0 == +0.0.
 #include "common.h"
 
+#include <mutex>
+
 #pragma clang fp contract(off)
 
 namespace sla {
@@ -588,6 +590,57 @@ extern "C" int sla_block_map_fwd(const void* q, const void* k, int dtype, int B,
                                  int lut_elem_bytes, void* stream) {
   return block_map_entry(q, k, nullptr, dtype, B, H, L, D, BLKQ, BLKK, topk, workspace, workspace_bytes, sparse_map, lut,
                          lut_elem_bytes, stream);
+}
+
+// ---- the block-mask builder for callers that cannot allocate ---------------------------------------------------
+// Same kernels as sla_block_map_fwd; the workspace is a fixed array in device memory that every GPU the library runs
+// on holds from the moment the code object is loaded until the process ends.
+static __device__ __align__(256) unsigned char scratch[SLA_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int MAX_DEVICES = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[MAX_DEVICES];   // device address of `scratch` on each GPU, resolved on the first call there
+
+// The array's name is only a handle on the host: its address in the current GPU's memory is looked up once per GPU.
+int static_scratch(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  SLA_REQUIRE(e == hipSuccess && dev >= 0 && dev < MAX_DEVICES, SLA_ERR_LAUNCH, "hipGetDevice: %s (device %d)",
+              hipGetErrorString(e), dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    SLA_REQUIRE(e == hipSuccess && p, SLA_ERR_LAUNCH, "hipGetSymbolAddress(scratch) on device %d: %s", dev,
+                hipGetErrorString(e));
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return SLA_OK;
+}
+}  // namespace
+
+extern "C" int sla_block_map_fwd_static(const void* q, const void* k, int dtype, int B, int H, int L, int D, int BLKQ,
+                                        int BLKK, int topk, int8_t* sparse_map, void* lut, int lut_elem_bytes,
+                                        void* stream) {
+  // sizes first (testable without a GPU): the problem must fit the fixed array
+  SLA_REQUIRE(B > 0 && H > 0 && L > 0 && D > 0 && BLKQ > 0 && BLKK > 0 && (int64_t)B * H <= 65535, SLA_ERR_BAD_ARG,
+              "bad size (B=%d H=%d L=%d D=%d BLKQ=%d BLKK=%d)", B, H, L, D, BLKQ, BLKK);
+  SLA_REQUIRE(dtype == SLA_F32 || dtype == SLA_BF16 || dtype == SLA_F16, SLA_ERR_BAD_ARG, "unknown dtype %d", dtype);
+  const int64_t need = block_map_workspace_bytes(dtype, B * H, L, D, BLKQ, BLKK);
+  SLA_REQUIRE(need <= (int64_t)SLA_STATIC_SCRATCH_BYTES, SLA_ERR_WORKSPACE,
+              "this problem needs %lld bytes of scratch, the static buffer holds %lld: use sla_block_map_fwd with a "
+              "workspace of the caller's",
+              (long long)need, (long long)SLA_STATIC_SCRATCH_BYTES);
+  SLA_REQUIRE(q && k && sparse_map && (lut || topk == 0), SLA_ERR_BAD_ARG, "null pointer");
+  void* ws = nullptr;
+  int rc = static_scratch(&ws);
+  if (rc) return rc;
+  // every part of the scratch is written by one kernel of the sequence before a later one reads it: nothing
+  // has to be cleared between calls
+  return block_map_entry(q, k, nullptr, dtype, B, H, L, D, BLKQ, BLKK, topk, ws, (int64_t)SLA_STATIC_SCRATCH_BYTES,
+                         sparse_map, lut, lut_elem_bytes, stream);
 }
 
 extern "C" int sla_block_map_fwd_strided(const void* q, const void* k, const int64_t* qk_strides, int dtype, int B, int H,
