@@ -34,8 +34,8 @@ PEAK_I8F8_TOPS = 5000.0        # MI355X dense int8 / fp8 MFMA
 # profiler summaries, stamped with a fingerprint of the kernel's sources: when the kernel changes the stamp no
 # longer matches and `traffic` is reported as null until the counters have been read again (--record-traffic).
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "sparse_fwd_cfg3_hbm_traffic.json")
-KERNEL_SOURCES = ("sla_amd/csrc/sparse_fwd.hip", "sla_amd/csrc/common.h", "sla_amd/csrc/linear_state.h",
-                  "sla_amd/csrc/linear_common.h")
+KERNEL_SOURCES = ("sla_amd/csrc/sparse_fwd.hip", "sla_amd/csrc/sparse_fwd_pair.h", "sla_amd/csrc/common.h",
+                  "sla_amd/csrc/linear_state.h", "sla_amd/csrc/linear_common.h")
 
 
 def kernel_fingerprint() -> str:
@@ -64,7 +64,7 @@ def measured_traffic(workload: str):
 
 def record_traffic(values):
     fetch_kib, write_kib, fetch_factor, write_factor = values
-    t = {"workload": "cfg3", "kernel": "sparse_fwd_kernel<FUSED>", "fetch_size_kib": fetch_kib, "write_size_kib": write_kib,
+    t = {"workload": "cfg3", "kernel": "sparse_fwd_pair_kernel<FUSED>", "fetch_size_kib": fetch_kib, "write_size_kib": write_kib,
          "fetch_factor": fetch_factor, "write_factor": write_factor, "kernel_sources_sha256_16": kernel_fingerprint(),
          "kernel_sources": list(KERNEL_SOURCES)}
     with open(TRAFFIC_FILE, "w") as f:
@@ -279,7 +279,7 @@ def main():
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / PEAK_BF16_TFLOPS,
                      "traffic": traffic, "traffic_note": traffic_note,
-                     "traffic_unit": "HBM bytes per launch (fetch + write)", "kernel": "sparse_fwd_kernel<FUSED=true>",
+                     "traffic_unit": "HBM bytes per launch (fetch + write)", "kernel": "sparse_fwd_pair_kernel<FUSED=true>",
                      "flops_per_launch": sparse_flops, "ms_per_launch": ms_sparse},
     }
     extra = {"sla_fwd_ms": ms_fwd, "attention_fused_ms": ms_sparse}

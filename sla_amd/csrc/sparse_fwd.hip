@@ -410,6 +410,10 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(D == 6
   }
 }
 
+}  // namespace sla
+#include "sparse_fwd_pair.h"
+namespace sla {
+
 struct FusedLinear {        // state of the linear branch for the fused epilogue (all null / 0 when not fused)
   const uint16_t* kvwt;
   const uint16_t* zst;
@@ -427,6 +431,22 @@ static int launch_fwd(const void* q, const void* k, const void* v, const void* l
   const int total = (int)total64;
   const int grid = xcd_grid(total);
   const float c = qk_scale * 1.4426950408889634f;
+  // The common shape (head dim 128, 64-row query blocks) has a kernel of its own, which shares key blocks between
+  // neighbouring query blocks; it addresses a head with 32-bit byte offsets and indexes key blocks with 12 bits.
+  if (D == 128 && BLKQ == 64 && topk <= PAIR_MAX_T && cdiv(L, 64) <= 4096 && (uint64_t)lin.sl * 2u * (uint64_t)L < (1ull << 31)) {
+    const int total_p = BH * ((Mblk + 1) / 2);
+    const int grid_p = xcd_grid(total_p);
+    if (fl)
+      hipLaunchKernelGGL((sparse_fwd_pair_kernel<Tag, true>), dim3(grid_p), dim3(128), 0, st, (const uint16_t*)q,
+                         (const uint16_t*)k, (const uint16_t*)v, lut, lut64, (uint16_t*)o, lse, lin, lout, L, Mblk, topk, c,
+                         total_p, fl->kvwt, fl->zst, fl->bias, fl->fmap, fl->o_s);
+    else
+      hipLaunchKernelGGL((sparse_fwd_pair_kernel<Tag, false>), dim3(grid_p), dim3(128), 0, st, (const uint16_t*)q,
+                         (const uint16_t*)k, (const uint16_t*)v, lut, lut64, (uint16_t*)o, lse, lin, lout, L, Mblk, topk, c,
+                         total_p, (const uint16_t*)nullptr, (const uint16_t*)nullptr, (const float*)nullptr, 0,
+                         (uint16_t*)nullptr);
+    return check_launch("sparse_attn_fwd");
+  }
 #define SLA_FWD_CASE(DD, BQ)                                                                                          \
   if (D == DD && BLKQ == BQ) {                                                                                        \
     if (fl)                                                                                                           \

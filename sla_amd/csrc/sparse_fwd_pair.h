@@ -1,0 +1,671 @@
+// Block-sparse FlashAttention forward for 64-row query blocks at head dim 128: two adjacent query blocks per
+// workgroup, one wavefront per query block.
+//
+// Stands in for _attn_fwd of the reference (sparse_linear_attention/kernel.py:21-82) like sparse_fwd_kernel,
+// whose arithmetic it shares (S^T = K Q^T, thresholded reference maximum, P^T as B operand of O^T = V^T P^T).
+// What differs is who shares what:
+//   * a wave owns all 64 rows of its query block (two 32-row tiles), so every K fragment and every V^T fragment
+//     read from LDS feeds two MFMAs: half the LDS reads per MFMA of the 32-rows-per-wave kernel;
+//   * neighbouring query blocks select mostly the same key blocks.  The two look-up rows of a pair are split
+//     into the key blocks both selected ("shared", walked first, one copy of the tile in LDS for both waves)
+//     and the rest ("own": as many on either side, each wave walks its own, two tiles in LDS).  A pair that
+//     shares 19 of 25 key blocks moves 31 tiles instead of 50 from L2 into LDS;
+//   * a wave has the whole register file of its SIMD (one wave per SIMD): the next half-tiles of K and V wait
+//     in registers for a whole half-tile of arithmetic before they are needed, and the loop is rotated so that
+//     the exponentials of half-tile u run beside the score products of u+1 and the output products of u.
+// The unit of the loop is a half-tile of 32 keys.  K half-tiles live in a two-generation ring in LDS (u even /
+// odd), V half-tiles likewise; each generation has two slots (slot 0: shared tile or wave 0's own, slot 1: wave
+// 1's own).  Tiles go from global memory straight into LDS (buffer loads with the LDS bit: no staging registers, no
+// LDS store instructions - a single wave per SIMD is bound by the instructions it has to issue, and a 16-byte LDS
+// store costs as many issue cycles as five vector-ALU instructions).  Rows are unpadded in LDS; the 16-byte slots
+// of a row are XOR-swizzled with the row index (by choosing which global piece a lane fetches), so that both the
+// 128-bit row reads of K and the transposing reads of V are free of bank conflicts.  One workgroup barrier per unit.
+// Minus the reference maximum (in the units of q . k) is the C operand of the first score product of a chain: what
+// is left per score is one fp32 multiply by qk_scale * log2(e) before the exponential.  (Scaling Q instead, once, and
+// rounding it to 16 bit again would spare that multiply and shift the log-sum-exp by up to 0.02: too much for the
+// backward pass, which forms its probabilities from it.)
+#pragma once
+#include "linear_state.h"
+
+namespace sla {
+
+constexpr int PAIR_MAX_T = 1024;      // look-up rows longer than this, or more than 4096 key blocks, take sparse_fwd_kernel
+
+// Score products with their result in vector registers (the exponentials read it next) and the resident Q^T operand in
+// accumulation registers.  Written as instructions because the compiler gives every MFMA of a function that uses
+// accumulation registers an accumulation-register result and would copy the scores back one register at a time.
+// (Hazards: a score tile is read by the vector ALU an iteration after its last product, and the two chains alternate,
+// so consecutive dependent products are 64 cycles apart.)
+template <typename Tag>
+static __device__ __forceinline__ void mfma_scores_first(f32x16_t& d, const i16x8_t& a, const i16x8_t& b) {
+  if constexpr (__is_same(Tag, bf16_tag))
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "a"(b));
+  else
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "a"(b));
+}
+template <typename Tag>
+static __device__ __forceinline__ void mfma_scores_first(f32x16_t& d, const i16x8_t& a, const i16x8_t& b, const f32x16_t& c) {
+  if constexpr (__is_same(Tag, bf16_tag))
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %3" : "=&v"(d) : "v"(a), "a"(b), "v"(c));
+  else
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %3" : "=&v"(d) : "v"(a), "a"(b), "v"(c));
+}
+template <typename Tag>
+static __device__ __forceinline__ void mfma_scores(f32x16_t& d, const i16x8_t& a, const i16x8_t& b) {
+  if constexpr (__is_same(Tag, bf16_tag))
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "a"(b));
+  else
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "a"(b));
+}
+
+template <typename Tag, bool FUSED>
+__global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) void sparse_fwd_pair_kernel(
+    const uint16_t* __restrict__ q, const uint16_t* __restrict__ k, const uint16_t* __restrict__ v, const void* __restrict__ lut,
+    int lut64, uint16_t* __restrict__ o, float* __restrict__ lse, const RowLayout lin, const RowLayout lout, int L, int Mblk,
+    int topk, float scale_log2e, int total, const uint16_t* __restrict__ kvwt, const uint16_t* __restrict__ zst,
+    const float* __restrict__ bias, int fmap, uint16_t* __restrict__ o_s) {
+  using E = Elem<Tag>;
+  constexpr int D = 128, DC = D / 16, DT = D / 32;
+  constexpr int ROWB = D * 2;                         // bytes per row in LDS (unpadded)
+  constexpr int SLOT = 32 * ROWB;                     // one half-tile: 8 KB
+  constexpr int SSTR = TileRows<D>::SSTR;
+  constexpr float PLIM = 1024.0f;   // a lane's 16 probabilities of a sub-tile may sum to this before the reference moves
+  typedef __attribute__((address_space(3))) void lds_void;
+
+  // K ring: [generation][slot] at (2 gen + slot) * SLOT; V ring: the same, 4 * SLOT further on
+  __shared__ __attribute__((aligned(16))) uint8_t smem[8 * SLOT];
+  __shared__ uint32_t bitmap[2][128];
+  __shared__ uint16_t steps[2][PAIR_MAX_T];
+  __shared__ int repeated;
+  static_assert(2 * 32 * SSTR * 2 <= 4 * SLOT, "the staging tiles of the epilogue exceed the K ring");
+
+  const int logical = xcd_remap(blockIdx.x, gridDim.x, total);
+  if (logical < 0) return;
+  const int Mpair = (Mblk + 1) >> 1;
+  const int bh = logical / Mpair;
+  const int pj = logical - bh * Mpair;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int g = lane >> 5, r = lane & 31;
+  const bool pair_full = 2 * pj + 1 < Mblk;            // the last block of a head with an odd block count has no partner:
+  const int mb = (w == 1 && pair_full) ? 2 * pj + 1 : 2 * pj;   // wave 1 then repeats wave 0's block and stores nothing
+  const bool writes = w == 0 || pair_full;
+
+  const size_t head_off = lin.head(bh);
+  const uint32_t pitch = (uint32_t)lin.sl;
+  const uint32_t head_bytes = lin.head_range_bytes(L, D);
+  const __amdgpu_buffer_rsrc_t kh = make_rsrc(k + head_off, head_bytes);
+  const __amdgpu_buffer_rsrc_t vh = make_rsrc(v + head_off, head_bytes);
+
+  // This wave's 64 query rows are requested first, straight in B-operand order (lane = row, 16 bytes per 16-wide
+  // chunk of the head dim): they arrive while the look-up rows are merged.  (A lane-per-row access touches 32 memory
+  // lines per instruction; it happens once per workgroup and spares a trip through LDS and a barrier.)
+  const int qrow0 = mb * 64;
+  uint16_t* const stage = reinterpret_cast<uint16_t*>(smem) + w * 32 * SSTR;   // wave-private staging tile of the epilogue, 32 rows (overlaps the K ring)
+  i16x8_t qf[2][DC];
+  {
+    const __amdgpu_buffer_rsrc_t qh = make_rsrc(q + head_off, head_bytes);
+#pragma unroll
+    for (int qt = 0; qt < 2; ++qt)
+#pragma unroll
+      for (int c = 0; c < DC; ++c)
+        qf[qt][c] = buf_load_b128(qh, ((uint32_t)(qrow0 + 32 * qt + r) * pitch + 16 * c + 8 * g) * 2);   // rows past L: 0
+  }
+  // rows past L are never written into LDS; where V is concerned what LDS holds there meets a probability of exactly
+  // 0 and must not be a NaN pattern left behind by an earlier kernel: a ragged sequence starts from a zeroed V ring
+  if (L % 64 != 0) {
+#pragma unroll
+    for (int i = 0; i < 4 * SLOT / (128 * 16); ++i) reinterpret_cast<i32x4_t*>(smem + 4 * SLOT)[i * 128 + tid] = i32x4_t{0, 0, 0, 0};
+  }
+
+  // ---- the two look-up rows -> per-wave step lists: shared key blocks first (in the order of the first row), then own
+  const size_t rowA = ((size_t)bh * Mblk + 2 * pj) * topk;
+  const size_t rowB = pair_full ? rowA + topk : rowA;
+  auto lut_at = [&](size_t i) __attribute__((always_inline)) -> int {
+    return lut64 ? (int)reinterpret_cast<const long long*>(lut)[i] : reinterpret_cast<const int*>(lut)[i];
+  };
+  // (The split assumes what the mask builder guarantees: no key block twice in a row, every index below 4096.  A row
+  //  that names a block twice makes the pair walk both rows unshared, in the order given, each block as often as it
+  //  is named; an index is only ever used modulo 4096 here, and as it is where the rows of K and V are addressed,
+  //  where the buffer bounds apply.)
+  bitmap[0][tid] = 0;
+  bitmap[1][tid] = 0;
+  if (tid == 0) repeated = 0;
+  __syncthreads();
+  for (int t = tid; t < topk; t += 128) {
+    const int a = lut_at(rowA + t) & 4095, b = lut_at(rowB + t) & 4095;
+    const uint32_t seen_a = atomicOr(&bitmap[0][a >> 5], 1u << (a & 31));
+    const uint32_t seen_b = atomicOr(&bitmap[1][b >> 5], 1u << (b & 31));
+    if (((seen_a >> (a & 31)) | (seen_b >> (b & 31))) & 1u) repeated = 1;
+  }
+  __syncthreads();
+  int ns = 0;                                  // number of shared key blocks (the same in both waves)
+  if (repeated) {
+    const size_t rowW = w ? rowB : rowA;
+    for (int i = lane; i < topk; i += 64) steps[w][i] = (uint16_t)(lut_at(rowW + i) & 4095);
+  } else {
+    const unsigned long long lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+    int n = 0;
+    for (int c0 = 0; c0 < topk; c0 += 64) {
+      const int i = c0 + lane;
+      const int a = i < topk ? lut_at(rowA + i) & 4095 : 0;
+      const bool sel = i < topk && ((bitmap[1][a >> 5] >> (a & 31)) & 1u);
+      const unsigned long long bal = __ballot(sel);
+      if (sel) steps[w][n + __popcll(bal & lt_mask)] = (uint16_t)a;
+      n += __popcll(bal);
+    }
+    ns = n;
+    const size_t rowW = w ? rowB : rowA;
+    for (int c0 = 0; c0 < topk; c0 += 64) {
+      const int i = c0 + lane;
+      const int x = i < topk ? lut_at(rowW + i) & 4095 : 0;
+      const bool sel = i < topk && !((bitmap[1 - w][x >> 5] >> (x & 31)) & 1u);
+      const unsigned long long bal = __ballot(sel);
+      if (sel) steps[w][n + __popcll(bal & lt_mask)] = (uint16_t)x;
+      n += __popcll(bal);
+    }
+  }
+  ns = __builtin_amdgcn_readfirstlane(ns);
+
+  f32x16_t oacc[DT][2];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int qt = 0; qt < 2; ++qt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) oacc[dt][qt][i] = 0.f;
+  // Reference maximum of the online softmax, in the exponent's units; minus the reference in all sixteen registers of
+  // a tuple that is the C operand of the first score product of every chain.  The reference starts at 0 and the first
+  // unit always takes the path that moves it.
+  float m_used[2] = {0.f, 0.f};
+  float l_run[2] = {0.f, 0.f};
+  f32x16_t negm[2];
+#pragma unroll
+  for (int qt = 0; qt < 2; ++qt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) negm[qt][i] = 0.f;
+
+  // ---- addressing ----
+  // unit u = 2 * step + half.  Shared steps: one tile, slot 0, wave w fetches rows 16w..16w+15 of the half-tile
+  // (4 instructions of 1 KB for K, 4 for V).  Own steps: slot w, the wave fetches all 32 rows (8 + 8 instructions).
+  // Instruction i of a half-tile fills LDS rows 4i..4i+3: lane -> row 4i + lane / 16, 16-byte slot lane % 16, which
+  // receives piece (slot ^ swizzle(row)) of that row.  K: swizzle = row % 16; V: 2 * (row % 8).
+  // A single wave per SIMD pays issue time for every instruction, scalar ones included, so everything that does not
+  // change inside the loop is formed here: per instruction there is one vector add (lane part + scalar row base), one
+  // scalar add into M0 (LDS destination) and the load.
+  const int nunits = 2 * topk;
+  const int lrow = lane >> 4, lslot = lane & 15;
+  const uint32_t smem_addr = (uint32_t)(size_t)smem;      // LDS address of the rings
+  const uint32_t row_bytes = pitch * 2;                   // bytes between rows in memory
+  uint32_t koff[4], voff[4];          // lane part of the byte offset of instruction j (mod 4): row 4j + lane / 16, swizzled piece
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    koff[j] = (uint32_t)(4 * j + lrow) * row_bytes + ((lslot ^ ((4 * j + lrow) & 15)) * 16);
+    voff[j] = (uint32_t)(4 * j + lrow) * row_bytes + ((lslot ^ ((((4 * j + lrow) & 7) << 1) & 15)) * 16);
+  }
+  // What the requests of a step need, by kind of step: the byte offset of the first row this wave fetches and the LDS
+  // address (inside a slot pair) of its first instruction.
+  struct Step {
+    int tile;          // key block
+    int own;           // 0: shared step, 1: own step
+    uint32_t rb;       // byte offset in the head of the first row this wave fetches of half 0
+    uint32_t dst;      // LDS byte address, relative to a generation's slot pair, of this wave's first instruction
+  };
+  auto step_of = [&](int s_raw, int tile) __attribute__((always_inline)) -> Step {
+    const int own = s_raw < ns ? 0 : 1;
+    return Step{tile, own, (uint32_t)(tile * 64 + (own ? 0 : 16 * w)) * row_bytes,
+                smem_addr + (uint32_t)(own ? w * SLOT : 4 * w * 1024)};
+  };
+  auto step_lookup = [&](int s_raw) __attribute__((always_inline)) -> int {       // (per lane; made scalar where it is used)
+    return (int)steps[w][min(s_raw, topk - 1)];         // past the end: the last step again (fetched, never used)
+  };
+  const uint32_t half_bytes = 32 * row_bytes, quarter_bytes = 16 * row_bytes;
+  // one request: 4 rows, global -> LDS.  `ring` = byte offset of the slot pair (generation, K or V) plus the instruction's 1 KB
+  // (written as instructions: the compiler would make every later LDS read wait for a load it knows to target LDS;
+  //  the wait for these loads is the one before the barrier at the end of an iteration.  Rows past L lie outside the
+  //  buffer range: nothing is written for them and LDS keeps what it held, which is either the zeros it was filled
+  //  with at the start or rows of an earlier tile: finite values, whose scores are masked and whose probabilities are 0)
+#define SLA_PAIR_FETCH(RSRC, LANEOFF, ROWBASE, DST, RING)                                                              \
+  do {                                                                                                                 \
+    const uint32_t off_ = (LANEOFF) + (ROWBASE);                                                                       \
+    asm volatile("s_add_u32 m0, %0, %3\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(DST), "v"(off_), "s"(RSRC),  \
+                 "s"((uint32_t)(RING))                                                                                 \
+                 : "memory", "scc");                                                                                   \
+  } while (0)
+  // fragment addressing (bytes from the start of the rings; the slot of the current kind of step is added when the
+  // kind changes, once per kernel)
+  int kfo[DC];                      // K fragment c of this lane: row r, piece 2c + g
+#pragma unroll
+  for (int c = 0; c < DC; ++c) kfo[c] = r * ROWB + (((2 * c + g) ^ (r & 15)) * 16);
+  const int tr_row = (lane & 15) >> 2;
+  const int v_row = 4 * g + tr_row;                  // + 16 * group (+ 8 for the second read)
+  const int v_swz = ((v_row & 7) << 1) & 15;
+  int vfo[DT];                      // V^T fragment dt: 8 bytes at element 4 * (lane % 4) of the 16-column strip 2 dt + (lane / 16) % 2
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) {
+    const int piece = 4 * dt + 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);
+    vfo[dt] = 4 * SLOT + v_row * ROWB + ((piece ^ v_swz) * 16) + (lane & 1) * 8;
+  }
+  // The fragment offsets move to this wave's own slot once, when the walk passes from the shared steps to the own
+  // ones: for K in the odd iteration of step ns - 1 (K_{u+1} is then the first own half-tile), for V in the even
+  // iteration of step ns.  (No shared step: the prologue has moved them.  No own step: they never move.)
+  const int k_flip_step = (ns > 0 && ns < topk) ? ns - 1 : -1;
+  const int v_flip_step = (ns > 0 && ns < topk) ? ns : -1;
+  const int ragged_tile = (L & 63) ? (L >> 6) : -1;       // the only key block that can have missing rows
+
+  // ---- pieces of the arithmetic ----
+  auto row_max = [&](const f32x16_t& sv) __attribute__((always_inline)) {
+    float mx = sv[0];
+#pragma unroll
+    for (int i = 1; i < 16; ++i) mx = fmaxf(mx, sv[i]);
+    return mx;
+  };
+  auto mask_tail = [&](f32x16_t& sv, int valid) __attribute__((always_inline)) {          // rows of this half-tile at or past `valid` do not exist
+    const int lim = valid - 4 * g;                         // key index of register i is 8(i/4) + i%4 + 4g
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+      if (8 * (i >> 2) + (i & 3) >= lim) sv[i] = -INFINITY;
+  };
+  // Moves the reference of query tile qt up to the maximum of sub-tile sv (whose registers hold score - old reference);
+  // rescales what has been accumulated, re-bases sv and the already formed scores of the next unit (sn).
+  auto raise_reference = [&](f32x16_t& sv, f32x16_t& sn, int qt, bool first) __attribute__((always_inline)) {
+    float mx = row_max(sv);
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    const float up = first ? mx : fmaxf(mx, 0.f);          // new reference - old reference
+    const float f = first ? 0.f : fast_exp2(-up * scale_log2e);
+    m_used[qt] += up;
+    l_run[qt] *= f;
+    // The output accumulators live in the accumulation registers and, on the common path, are only ever touched by
+    // MFMAs.  They are scaled in place through one temporary, so that the register allocator has no reason to
+    // move the whole accumulator through the vector registers around the loop.
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");     // (the last products into these registers and into sn have landed)
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        float x = oacc[dt][qt][i], t;
+        asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 %0, %1"
+                     : "+a"(x), "=&v"(t)
+                     : "v"(f));
+        oacc[dt][qt][i] = x;
+      }
+    const float nm = -m_used[qt];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      sv[i] -= up;
+      // (in place: written as a plain subtraction the compiler keeps the re-based scores in other registers than the
+      //  scores, and pays for it with sixteen copies on the path that does not come here)
+      float x = sn[i];
+      asm volatile("v_sub_f32 %0, %0, %1" : "+v"(x) : "v"(up));
+      sn[i] = x;
+      float y = negm[qt][i];
+      asm volatile("v_mov_b32 %0, %1" : "+v"(y) : "v"(nm));
+      negm[qt][i] = y;
+    }
+  };
+  auto zero16 = [&](f32x16_t& x) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) x[i] = 0.f;
+  };
+  auto read_k = [&](int gen, i16x8_t (&kf)[DC]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int c = 0; c < DC; ++c) kf[c] = *reinterpret_cast<const i16x8_t*>(smem + gen * 2 * SLOT + kfo[c]);
+  };
+
+  // ---- prologue: K_0, V_0, K_1 into LDS; S_0 ----
+  f32x16_t s_a[2], s_b[2];        // scores of the current and of the next unit, swapping roles every iteration
+  i16x8_t kf[DC];
+  i16x8_t vf_a[2][DT], vf_b[2][DT];   // V^T fragments of the even / odd unit: [16-key group][32 output channels]
+  i32x4_t pbw[2][2];                  // packed probabilities: [query tile][16-key group]
+#pragma unroll
+  for (int c2 = 0; c2 < 2; ++c2) {
+    pbw[1][c2] = i32x4_t{0, 0, 0, 0};             // the first iteration's left-over products add nothing
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) vf_b[c2][dt] = i16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+  }
+  Step cur{0, 0, 0, 0}, nxt{0, 0, 0, 0};
+  if (nunits > 0) {
+    cur = step_of(0, __builtin_amdgcn_readfirstlane(step_lookup(0)));
+    nxt = step_of(min(1, topk - 1), __builtin_amdgcn_readfirstlane(step_lookup(1)));
+    // K_0, V_0 (generation 0) and K_1 (generation 1) of the first step
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      SLA_PAIR_FETCH(kh, koff[j], cur.rb, cur.dst, 0 * SLOT + j * 1024);
+      SLA_PAIR_FETCH(vh, voff[j], cur.rb, cur.dst, 4 * SLOT + j * 1024);
+      SLA_PAIR_FETCH(kh, koff[j], cur.rb + half_bytes, cur.dst, 2 * SLOT + j * 1024);
+    }
+    if (cur.own) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        SLA_PAIR_FETCH(kh, koff[j], cur.rb + quarter_bytes, cur.dst, 0 * SLOT + 4096 + j * 1024);
+        SLA_PAIR_FETCH(vh, voff[j], cur.rb + quarter_bytes, cur.dst, 4 * SLOT + 4096 + j * 1024);
+        SLA_PAIR_FETCH(kh, koff[j], cur.rb + half_bytes + quarter_bytes, cur.dst, 2 * SLOT + 4096 + j * 1024);
+      }
+#pragma unroll
+      for (int c = 0; c < DC; ++c) kfo[c] += w * SLOT;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) vfo[dt] += w * SLOT;
+    }
+  }
+  // Q is only ever an MFMA operand (unscaled: the scores stay in the units of q . k, the reference maximum too, and
+  // qk_scale * log2(e) multiplies the exponent's argument in fp32) and is parked in the accumulation registers: the
+  // vector registers are left for the score tiles, the fragments and the softmax arithmetic
+#pragma unroll
+  for (int qt = 0; qt < 2; ++qt)
+#pragma unroll
+    for (int c = 0; c < DC; ++c) asm volatile("" : "+a"(qf[qt][c]));
+  if (nunits > 0) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    read_k(0, kf);
+#pragma unroll
+    for (int c = 0; c < DC; ++c)
+#pragma unroll
+      for (int qt = 0; qt < 2; ++qt) {
+        if (c == 0) mfma_scores_first<Tag>(s_a[qt], kf[c], qf[qt][c]);
+        else mfma_scores<Tag>(s_a[qt], kf[c], qf[qt][c]);
+      }
+  }
+
+  // One iteration = unit u, 32 MFMAs, every one of them followed by its share of the other work (the order is pinned
+  // slot by slot: a single wave per SIMD has nobody else to fill its gaps):
+  //   slots  0.. 7  O^T(query tile 1) += V_{u-1}^T P_{u-1}^T   (left over from the previous unit; operands in registers)
+  //                 beside: exponentials of (u, query tile 0).  Before slot 4: wait for the requests of the previous
+  //                 iteration, one barrier (the four products already queued keep the matrix pipe busy meanwhile).
+  //                 From slot 4: K_{u+2} and V_{u+1} requested (memory -> LDS), fragments of K_{u+1}, then of V_u,
+  //                 fetched from LDS
+  //   slots  8..23  S_{u+1} = K_{u+1} Q^T (two chains)          beside: exponentials of (u, tile 0), then of (u, tile 1)
+  //   slots 24..31  O^T(query tile 0) += V_u^T P_u^T            beside: rest of the exponentials of (u, tile 1)
+  // After the barrier LDS holds K_{u+1} (generation (u+1)&1) and V_u (generation u&1); on entry s_cur = scores of u
+  // minus the reference.  Unit u is half HALF of step `cur`; the half after it belongs to `cur` (HALF 0) or to `nxt`
+  // (HALF 1).
+  int step_index = 0;
+  float e0 = 0.f, e1 = 0.f;           // one pair of exponentials on its way from the exponent to the packing
+  auto pair_exp = [&](const f32x16_t& sv, int j) __attribute__((always_inline)) {
+    e0 = fast_exp2(sv[2 * j] * scale_log2e);
+    e1 = fast_exp2(sv[2 * j + 1] * scale_log2e);
+    asm volatile("" : "+v"(e0), "+v"(e1));         // (stays in its slot: nothing moves this work towards its first use)
+  };
+  auto pair_pack = [&](int qt, int j, float& psum) __attribute__((always_inline)) {
+    uint32_t pw = E::pack2(e0, e1);
+    psum += e0 + e1;                               // (plain adds: a dot-product instruction beside the MFMAs stalls the matrix pipe)
+    asm volatile("" : "+v"(pw), "+v"(psum));
+    pbw[qt][j >> 2][j & 3] = (int)pw;
+  };
+  auto softmax_again = [&](const f32x16_t& sv, int qt) __attribute__((always_inline)) -> float {     // (rare path) all eight pairs of a sub-tile
+    float psum = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      pair_exp(sv, j);
+      pair_pack(qt, j, psum);
+    }
+    return psum;
+  };
+  float ps_seed = INFINITY;
+  auto iteration = [&](int HALF, f32x16_t (&s_cur)[2], f32x16_t (&s_nxt)[2], i16x8_t (&vf_prev)[2][DT],
+                       i16x8_t (&vf_cur)[2][DT]) __attribute__((always_inline)) {
+    const int gen = HALF;                          // generation of K_u / V_u; K_{u+1} lives in the other one
+    if (__builtin_expect(cur.tile == ragged_tile, 0)) {
+      const int valid = L - (cur.tile * 64 + 32 * HALF);   // rows of this half-tile that exist
+      mask_tail(s_cur[0], valid);
+      mask_tail(s_cur[1], valid);
+    }
+    // requests: K_{u+2} is half HALF of step nxt; V_{u+1} is half 1 of cur (HALF 0) or half 0 of nxt (HALF 1)
+    const Step& vs = HALF == 0 ? cur : nxt;
+    const uint32_t k_rb = nxt.rb + (HALF ? half_bytes : 0u);
+    const uint32_t v_rb = vs.rb + (HALF ? 0u : half_bytes);
+    // fragment reads: K_{u+1} is half 1 of cur (HALF 0) or half 0 of nxt (HALF 1); V_u is of cur.  Their slot changes
+    // once, when the walk passes from the shared steps to the own ones.
+    if (HALF == 1 && __builtin_expect(step_index == k_flip_step, 0)) {
+#pragma unroll
+      for (int c = 0; c < DC; ++c) kfo[c] += w * SLOT;
+    }
+    if (HALF == 0 && __builtin_expect(step_index == v_flip_step, 0)) {
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) vfo[dt] += w * SLOT;
+    }
+    // the key block of the step after next is looked up now and used at the end of the odd iteration
+    int tile2_lane = 0;
+    if (HALF) tile2_lane = step_lookup(step_index + 2);
+    // (the first unit's sums start from infinity: that sends it down the path that sets the reference)
+    float ps0 = HALF == 0 ? ps_seed : 0.f, ps1 = ps0;
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- block A: slots 0..23 ----
+#pragma unroll
+    for (int sl = 0; sl < 24; ++sl) {
+      if (sl == 4) {
+        // The requests of the previous iteration have had twenty slots to land; four products are queued in the
+        // matrix pipe while the two waves meet.  After the barrier: K_{u+1} and V_u are visible, and everyone has
+        // fetched its fragments of K_u and V_{u-1}, whose places this iteration's requests overwrite.
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if (sl < 8) {
+        const int c2 = sl >> 2, dt = sl & 3;
+        oacc[dt][1] = E::mfma32(vf_prev[c2][dt], __builtin_bit_cast(i16x8_t, pbw[1][c2]), oacc[dt][1]);
+      } else {
+        const int c = (sl - 8) >> 1, qt = (sl - 8) & 1;
+        if (c == 0) mfma_scores_first<Tag>(s_nxt[qt], kf[c], qf[qt][c], negm[qt]);
+        else mfma_scores<Tag>(s_nxt[qt], kf[c], qf[qt][c]);
+      }
+      // exponentials: query tile 0 in slots 0..15, query tile 1 (first half) in slots 16..23
+      if (sl < 16) {
+        if ((sl & 1) == 0) pair_exp(s_cur[0], sl >> 1);
+        else pair_pack(0, sl >> 1, ps0);
+      } else {
+        if ((sl & 1) == 0) pair_exp(s_cur[1], (sl - 16) >> 1);
+        else pair_pack(1, (sl - 16) >> 1, ps1);
+      }
+      // memory -> LDS: K_{u+2} (generation of u: K_u was used up an iteration ago) and V_{u+1} (the other generation:
+      // V_{u-1} was used up in the last iteration); 4 + 4 requests, 4 + 4 more on own steps
+      if (sl >= 4 && sl < 8) {
+        if (gen == 0) SLA_PAIR_FETCH(kh, koff[sl - 4], k_rb, nxt.dst, 0 * SLOT + (sl - 4) * 1024);
+        else SLA_PAIR_FETCH(kh, koff[sl - 4], k_rb, nxt.dst, 2 * SLOT + (sl - 4) * 1024);
+      } else if (sl >= 8 && sl < 12) {
+        if (gen == 0) SLA_PAIR_FETCH(vh, voff[sl - 8], v_rb, vs.dst, 6 * SLOT + (sl - 8) * 1024);
+        else SLA_PAIR_FETCH(vh, voff[sl - 8], v_rb, vs.dst, 4 * SLOT + (sl - 8) * 1024);
+      }
+      if (sl == 12 && nxt.own) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          if (gen == 0) SLA_PAIR_FETCH(kh, koff[j], k_rb + quarter_bytes, nxt.dst, 0 * SLOT + 4096 + j * 1024);
+          else SLA_PAIR_FETCH(kh, koff[j], k_rb + quarter_bytes, nxt.dst, 2 * SLOT + 4096 + j * 1024);
+        }
+      }
+      if (sl == 14 && vs.own) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          if (gen == 0) SLA_PAIR_FETCH(vh, voff[j], v_rb + quarter_bytes, vs.dst, 6 * SLOT + 4096 + j * 1024);
+          else SLA_PAIR_FETCH(vh, voff[j], v_rb + quarter_bytes, vs.dst, 4 * SLOT + 4096 + j * 1024);
+        }
+      }
+      // LDS reads: K_{u+1} fragments in slots 4..7 (used from slot 8 on), V_u fragments in slots 8..15
+      if (sl >= 4 && sl < 8) {
+        kf[2 * (sl - 4)] = *reinterpret_cast<const i16x8_t*>(smem + (gen ^ 1) * 2 * SLOT + kfo[2 * (sl - 4)]);
+        kf[2 * (sl - 4) + 1] = *reinterpret_cast<const i16x8_t*>(smem + (gen ^ 1) * 2 * SLOT + kfo[2 * (sl - 4) + 1]);
+      } else if (sl >= 8 && sl < 16) {
+        const int gi = (sl - 8) >> 2, dt = (sl - 8) & 3;
+        const uint8_t* p0 = smem + gen * 2 * SLOT + 16 * gi * ROWB + vfo[dt];
+        vf_cur[gi][dt] = concat4(lds_read_tr16(reinterpret_cast<const uint16_t*>(p0)),
+                                 lds_read_tr16(reinterpret_cast<const uint16_t*>(p0 + 8 * ROWB)));
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // rare path (one branch): the probabilities came out too large (or this is the first unit, whose reference is a
+    // placeholder): move the reference to this sub-tile's maximum and form them again
+    const bool first = HALF == 0 && step_index == 0;       // (looked at on the rare path only)
+    if (__builtin_expect(__any(!(ps0 <= PLIM)), 0)) {
+      raise_reference(s_cur[0], s_nxt[0], 0, first);
+      ps0 = softmax_again(s_cur[0], 0);
+    }
+    l_run[0] += ps0;
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- block B: slots 24..31 ----
+#pragma unroll
+    for (int sl = 0; sl < 8; ++sl) {
+      const int c2 = sl >> 2, dt = sl & 3;
+      oacc[dt][0] = E::mfma32(vf_cur[c2][dt], __builtin_bit_cast(i16x8_t, pbw[0][c2]), oacc[dt][0]);
+      if ((sl & 1) == 0) pair_exp(s_cur[1], 4 + (sl >> 1));
+      else pair_pack(1, 4 + (sl >> 1), ps1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (__builtin_expect(__any(!(ps1 <= PLIM)), 0)) {
+      raise_reference(s_cur[1], s_nxt[1], 1, first);
+      ps1 = softmax_again(s_cur[1], 1);
+    }
+    l_run[1] += ps1;
+    if (HALF == 0) ps_seed = 0.f;
+    if (HALF) {
+      cur = nxt;
+      nxt = step_of(min(step_index + 2, topk - 1), __builtin_amdgcn_readfirstlane(tile2_lane));
+    }
+  };
+
+  for (; step_index < topk; ++step_index) {
+    iteration(0, s_a, s_b, vf_b, vf_a);
+    iteration(1, s_b, s_a, vf_a, vf_b);
+  }
+  // the last unit's products for query tile 1 (nunits is even: its fragments are in vf_b)
+  if (nunits > 0) {
+#pragma unroll
+    for (int sl = 0; sl < 8; ++sl) {
+      const int c2 = sl >> 2, dt = sl & 3;
+      oacc[dt][1] = E::mfma32(vf_b[c2][dt], __builtin_bit_cast(i16x8_t, pbw[1][c2]), oacc[dt][1]);
+    }
+  }
+
+  // ---- epilogue ----
+  // every wave is done with the rings and no request is in flight: the staging tiles are free
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  const size_t out_off = lout.head(bh) + (size_t)qrow0 * (size_t)lout.sl;
+  // Fused linear branch: the per-head state KVW^T (D x D, 16 bit) goes into the V ring the way K half-tiles do (four
+  // slots of 32 rows, swizzled pieces, each wave requests half), the unscaled q rows come again in B-operand order.
+  // z and the bias come up front as well: at one wave per SIMD nothing hides a load issued where it is used.
+  i16x8_t qraw[2][DC], zreg[DC];
+  f32x4_t breg[DT][4];
+  if (FUSED) {
+    const __amdgpu_buffer_rsrc_t sth = make_rsrc(kvwt + (size_t)bh * D * D, D * D * 2);
+    const __amdgpu_buffer_rsrc_t qh = make_rsrc(q + head_off, head_bytes);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      // instruction i of this wave: rows 64w + 4i .. +3 of the state -> slot 4 + 2w + i / 8, rows 4 (i % 8) ..
+      const int j = i & 3;
+      const uint32_t soff = (uint32_t)(4 * j + lrow) * ROWB + ((lslot ^ ((4 * j + lrow) & 15)) * 16);
+      SLA_PAIR_FETCH(sth, soff, (uint32_t)((64 * w + 4 * (i - j)) * ROWB), smem_addr, (4 + 2 * w + (i >> 3)) * SLOT + (i & 7) * 1024);
+    }
+#pragma unroll
+    for (int qt = 0; qt < 2; ++qt)
+#pragma unroll
+      for (int c = 0; c < DC; ++c)
+        qraw[qt][c] = buf_load_b128(qh, ((uint32_t)(qrow0 + 32 * qt + r) * pitch + 16 * c + 8 * g) * 2);
+    const uint16_t* z_h = zst + (size_t)bh * D;
+#pragma unroll
+    for (int c = 0; c < DC; ++c) zreg[c] = *reinterpret_cast<const i16x8_t*>(z_h + 16 * c + 8 * g);
+#pragma unroll
+    for (int et = 0; et < DT; ++et)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; ++i4) {
+        const f32x4_t b4 = *reinterpret_cast<const f32x4_t*>(bias + 32 * et + 8 * i4 + 4 * g);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) breg[et][i4][j] = round16<Tag>(b4[j]);
+      }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+  }
+#pragma unroll
+  for (int qt = 0; qt < 2; ++qt) {
+    uint16_t* const stage_q = stage;
+    const int rows_valid = writes ? min(32, L - qrow0 - 32 * qt) : 0;
+    const float l_tot = l_run[qt] + __shfl_xor(l_run[qt], 32);
+    const float inv = 1.0f / l_tot;
+    const int qrow = qrow0 + 32 * qt + r;
+    if (qrow < L && g == 0 && writes) lse[(size_t)bh * L + qrow] = m_used[qt] * scale_log2e + fast_log2(l_tot);
+    auto park_attention = [&]() __attribute__((always_inline)) {
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int i4 = 0; i4 < 4; ++i4) {
+          i32x2_t wv;
+          wv[0] = (int)E::pack2(oacc[dt][qt][4 * i4 + 0] * inv, oacc[dt][qt][4 * i4 + 1] * inv);
+          wv[1] = (int)E::pack2(oacc[dt][qt][4 * i4 + 2] * inv, oacc[dt][qt][4 * i4 + 3] * inv);
+          *reinterpret_cast<i32x2_t*>(&stage_q[r * SSTR + 32 * dt + 8 * i4 + 4 * g]) = wv;
+        }
+      wave_lds_fence();
+    };
+    auto flush_rows = [&](uint16_t* dst_tile, size_t dst_pitch) __attribute__((always_inline)) {
+      TileRows<D> t;
+      t.unpark(stage_q, lane);
+      t.store(dst_tile, rows_valid, lane, dst_pitch);
+      wave_lds_fence();
+    };
+    if (!FUSED) {
+      park_attention();
+      flush_rows(o + out_off + (size_t)(32 * qt) * (size_t)lout.sl, (size_t)lout.sl);
+    } else {
+      // ---- linear branch of the same rows (see sparse_fwd_kernel) ----
+      // (the resident fragments hold q scaled for the attention: these are the unscaled rows)
+      float f[DC][8];
+#pragma unroll
+      for (int c = 0; c < DC; ++c)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) f[c][j] = E::to_float((uint16_t)qraw[qt][c][j]);
+      float row_mx, row_inv;
+      phi_row_pair<Tag, DC>(fmap, f, row_mx, row_inv);
+      float den = 0.f;
+      i16x8_t fq[DC];
+#pragma unroll
+      for (int c = 0; c < DC; ++c) {
+        const i16x8_t zc = zreg[c];
+        i32x4_t pw;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) den += round16<Tag>(f[c][j] * E::to_float((uint16_t)zc[j]));
+#pragma unroll
+        for (int j = 0; j < 4; ++j) pw[j] = (int)E::pack2(f[c][2 * j], f[c][2 * j + 1]);
+        fq[c] = __builtin_bit_cast(i16x8_t, pw);
+      }
+      den += __shfl_xor(den, 32);
+      den = round16<Tag>(1e-5f + round16<Tag>(den));
+      const float inv_den = 1.0f / den;
+#pragma unroll
+      for (int et = 0; et < DT; ++et) {
+        i16x8_t a[DC];
+#pragma unroll
+        for (int c = 0; c < DC; ++c)
+          a[c] = *reinterpret_cast<const i16x8_t*>(smem + (4 + et) * SLOT + r * ROWB + (((2 * c + g) ^ (r & 15)) * 16));
+        f32x16_t acc;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+#pragma unroll
+        for (int c = 0; c < DC; ++c) acc = E::mfma32(a[c], fq[c], acc);
+#pragma unroll
+        for (int i4 = 0; i4 < 4; ++i4) {
+          const int e0 = 32 * et + 8 * i4 + 4 * g;
+          const f32x4_t b4 = breg[et][i4];
+          i32x2_t ws, wo;
+          ws[0] = (int)E::pack2(oacc[et][qt][4 * i4 + 0] * inv, oacc[et][qt][4 * i4 + 1] * inv);
+          ws[1] = (int)E::pack2(oacc[et][qt][4 * i4 + 2] * inv, oacc[et][qt][4 * i4 + 3] * inv);
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            const uint32_t x = (uint32_t)ws[h];
+            const float l0 = round16<Tag>(pin_f32(__builtin_fmaf(acc[4 * i4 + 2 * h], inv_den, b4[2 * h])));
+            const float l1 = round16<Tag>(pin_f32(__builtin_fmaf(acc[4 * i4 + 2 * h + 1], inv_den, b4[2 * h + 1])));
+            wo[h] = (int)E::pack2(E::to_float((uint16_t)(x & 0xffff)) + l0, E::to_float((uint16_t)(x >> 16)) + l1);
+          }
+          *reinterpret_cast<i32x2_t*>(&stage_q[r * SSTR + e0]) = wo;
+        }
+      }
+      wave_lds_fence();
+      flush_rows(o + out_off + (size_t)(32 * qt) * (size_t)lout.sl, (size_t)lout.sl);
+      if (o_s) {
+        park_attention();
+        flush_rows(o_s + ((size_t)bh * L + qrow0 + 32 * qt) * D, D);
+      }
+    }
+  }
+}
+
+#undef SLA_PAIR_FETCH
+
+}  // namespace sla
