@@ -433,8 +433,11 @@ static int launch_fwd(const void* q, const void* k, const void* v, const void* l
   const float c = qk_scale * 1.4426950408889634f;
   // The common shape (head dim 128, 64-row query blocks) has a kernel of its own, which shares key blocks between
   // neighbouring query blocks; it addresses a head with 32-bit byte offsets and indexes key blocks with 12 bits.
-  if (D == 128 && BLKQ == 64 && topk <= PAIR_MAX_T && cdiv(L, 64) <= 4096 && (uint64_t)lin.sl * 2u * (uint64_t)L < (1ull << 31)) {
-    const int total_p = BH * ((Mblk + 1) / 2);
+  // (Two query blocks per workgroup halve the number of workgroups: a launch too small to give every compute unit
+  // its two workgroups keeps one query block per workgroup.)
+  const int total_p = BH * ((Mblk + 1) / 2);
+  if (D == 128 && BLKQ == 64 && topk <= PAIR_MAX_T && cdiv(L, 64) <= 4096 && (uint64_t)lin.sl * 2u * (uint64_t)L < (1ull << 31) &&
+      total_p >= 512) {
     const int grid_p = xcd_grid(total_p);
     if (fl)
       hipLaunchKernelGGL((sparse_fwd_pair_kernel<Tag, true>), dim3(grid_p), dim3(128), 0, st, (const uint16_t*)q,
