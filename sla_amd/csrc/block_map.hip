@@ -287,10 +287,112 @@ __global__ __launch_bounds__(256) void score_kernel(const typename IO::raw* __re
   }
 }
 
+// The same scores from the matrix cores, for 16-bit dtypes.  v_mfma_f32_32x32x2_f32 adds its two products to the
+// accumulator one after the other, each with a single rounding: k = 0 first, then k = 1.  A chain of them over
+// d = 0, 2, 4, ... therefore is the d-ascending chain of fp32 fused multiply-adds of score_kernel, bit for bit (the
+// product of two 16-bit values is exact in fp32, so fused or not makes no difference; values whose products fall
+// into the fp32 subnormal range aside), at twice the rate of the vector ALU.
+// 64 x 64NW scores per workgroup, one wave per 32 x 32NW part (NW independent accumulation chains).  The 64 pooled rows of either operand go through LDS
+// (coalesced 16-byte loads; rows padded by 16 bytes, so that the row-per-lane reads are free of bank conflicts);
+// lanes l and l + 32 read the same rows and feed the even and the odd d.  The rounded scores go back through LDS
+// and leave in 256-byte runs.
+template <typename IO, int D, int NW>
+__global__ __launch_bounds__(256) void score_mfma_kernel(const typename IO::raw* __restrict__ pq,
+                                                         const typename IO::raw* __restrict__ pk,
+                                                         typename IO::raw* __restrict__ score, int M, int N) {
+  static_assert(sizeof(typename IO::raw) == 2 && D % 32 == 0, "16-bit dtypes, 256 threads fetch whole rows");
+  constexpr int NC = D / 8;              // 16-byte pieces per row
+  constexpr int RS = D * 2 + 16;         // bytes between rows in LDS
+  constexpr int OS = 64 * NW * 2 + 4;         // bytes between rows of the staged scores
+  constexpr int TN = 64 * NW;            // scores per row of the workgroup's tile
+  __shared__ __attribute__((aligned(16))) uint8_t sm[(64 + TN) * RS];
+  static_assert(64 * OS <= (64 + TN) * RS, "the staged scores reuse the operand tiles");
+  const int bh = blockIdx.z, tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 31, h = lane >> 5;
+  const int m0 = blockIdx.y * 64, n0 = blockIdx.x * (64 * NW);
+  const __amdgpu_buffer_rsrc_t qh = make_rsrc(pq + (size_t)bh * M * D, (uint32_t)M * D * 2);    // rows past the end read as zero
+  const __amdgpu_buffer_rsrc_t kh = make_rsrc(pk + (size_t)bh * N * D, (uint32_t)N * D * 2);
+#pragma unroll
+  for (int i = 0; i < 64 * NC / 256; ++i) {
+    const int p = tid + 256 * i, row = p / NC, pc = p % NC;
+    const i16x8_t a = buf_load_b128(qh, ((uint32_t)(m0 + row) * D + 8 * pc) * 2);
+    i16x8_t b[NW];
+#pragma unroll
+    for (int t = 0; t < NW; ++t) b[t] = buf_load_b128(kh, ((uint32_t)(n0 + 64 * t + row) * D + 8 * pc) * 2);
+    *reinterpret_cast<i16x8_t*>(sm + row * RS + pc * 16) = a;
+#pragma unroll
+    for (int t = 0; t < NW; ++t) *reinterpret_cast<i16x8_t*>(sm + (64 + 64 * t + row) * RS + pc * 16) = b[t];
+  }
+  __syncthreads();
+  const int wm = wave >> 1, wn = wave & 1;
+  const uint8_t* arow = sm + (wm * 32 + r) * RS;
+  const uint8_t* brow = sm + (64 + wn * 32 * NW + r) * RS;      // this wave's NW tiles of 32 columns lie side by side
+  f32x16_t acc[NW];
+#pragma unroll
+  for (int t = 0; t < NW; ++t)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[t][i] = 0.f;
+  const int sh = 16 * h;
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    const i32x4_t aw = *reinterpret_cast<const i32x4_t*>(arow + c * 16);
+    i32x4_t bw[NW];
+#pragma unroll
+    for (int t = 0; t < NW; ++t) bw[t] = *reinterpret_cast<const i32x4_t*>(brow + 32 * t * RS + c * 16);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float av = IO::ld((typename IO::raw)((uint32_t)aw[j] >> sh));
+#pragma unroll
+      for (int t = 0; t < NW; ++t) {
+        const float bv = IO::ld((typename IO::raw)((uint32_t)bw[t][j] >> sh));
+        acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[t], 0, 0, 0);
+      }
+    }
+  }
+  __syncthreads();                       // every wave has read its operands: the tiles make room for the scores
+#pragma unroll
+  for (int t = 0; t < NW; ++t)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int m = wm * 32 + 8 * (i >> 2) + (i & 3) + 4 * h;
+      *reinterpret_cast<typename IO::raw*>(sm + m * OS + (wn * 32 * NW + 32 * t + r) * 2) = IO::st(acc[t][i]);
+    }
+  __syncthreads();
+  typename IO::raw* out = score + (size_t)bh * M * N;
+  constexpr int TPR = 32 * NW;           // threads per row of staged scores, two scores each
+  const int orow = tid / TPR, ocol = (tid % TPR) * 2;
+#pragma unroll
+  for (int pass = 0; pass < 64 * TPR / 256; ++pass) {
+    const int ml = pass * (256 / TPR) + orow, m = m0 + ml, n = n0 + ocol;
+    if (m >= M || n >= N) continue;
+    const uint32_t two = *reinterpret_cast<const uint32_t*>(sm + ml * OS + ocol * 2);
+    typename IO::raw* dst = out + (size_t)m * N + n;
+    if (!(N & 1) && n + 1 < N) {
+      *reinterpret_cast<uint32_t*>(dst) = two;          // (N even: every pair starts 4-byte aligned)
+    } else {
+      dst[0] = (typename IO::raw)(two & 0xffffu);
+      if (n + 1 < N) dst[1] = (typename IO::raw)(two >> 16);
+    }
+  }
+}
+
 template <typename IO>
 static void launch_score(const typename IO::raw* pq, const typename IO::raw* pk, typename IO::raw* score, int BH, int M, int N,
                          int D, hipStream_t st) {
   const dim3 grid(cdiv(N, 64), cdiv(M, 64), BH);
+  if constexpr (sizeof(typename IO::raw) == 2) {
+    const bool fits = (int64_t)M * D * 2 < (1ll << 32) && (int64_t)N * D * 2 < (1ll << 32);
+    // (NW = 2, two column tiles per wave, is no faster: 159 against 153 us for 40 heads of 1182 x 1182 scores)
+    if (D == 128 && fits) {
+      hipLaunchKernelGGL((score_mfma_kernel<IO, 128, 1>), grid, dim3(256), 0, st, pq, pk, score, M, N);
+      return;
+    }
+    if (D == 64 && fits) {
+      hipLaunchKernelGGL((score_mfma_kernel<IO, 64, 1>), grid, dim3(256), 0, st, pq, pk, score, M, N);
+      return;
+    }
+  }
   if (D % 32 == 0)
     hipLaunchKernelGGL((score_kernel<IO, true>), grid, dim3(256), 0, st, pq, pk, score, M, N, D);
   else
@@ -308,9 +410,28 @@ static __device__ __forceinline__ uint32_t order_key(float f) {
   return u & ~((1u << LOW_BIT) - 1u);
 }
 
-// One wavefront per (bh, m) row (four rows per workgroup): radix-select the T-th largest key bit
-// by bit with ballot counts, then emit winners in ascending index order (ties at the threshold
-// value go to the lowest indices).  Writes the int8 map row and the look-up-table row.
+// Inclusive prefix sum over the 64 lanes of a wave (data-parallel-primitive moves inside rows of 16 lanes, then the
+// row totals are handed on).
+static __device__ __forceinline__ int wave_inclusive_sum(int x, int lane) {
+  const int rl = lane & 15;
+  int t;
+  t = __builtin_amdgcn_update_dpp(0, x, 0x111, 0xf, 0xf, false);      // row_shr:1
+  if (rl >= 1) x += t;
+  t = __builtin_amdgcn_update_dpp(0, x, 0x112, 0xf, 0xf, false);      // row_shr:2
+  if (rl >= 2) x += t;
+  t = __builtin_amdgcn_update_dpp(0, x, 0x114, 0xf, 0xf, false);      // row_shr:4
+  if (rl >= 4) x += t;
+  t = __builtin_amdgcn_update_dpp(0, x, 0x118, 0xf, 0xf, false);      // row_shr:8
+  if (rl >= 8) x += t;
+  t = __builtin_amdgcn_update_dpp(0, x, 0x142, 0xa, 0xf, false);      // row_bcast:15 (last lane of a row -> the next row)
+  if ((lane & 31) >= 16) x += t;
+  t = __builtin_amdgcn_update_dpp(0, x, 0x143, 0xc, 0xf, false);      // row_bcast:31 (lane 31 -> the upper half)
+  if (lane >= 32) x += t;
+  return x;
+}
+
+// One wavefront per (bh, m) row (four rows per workgroup): radix-select the T-th largest key, then emit
+// winners in ascending index order (ties at the threshold value go to the lowest indices).  Writes the int8 map row and the look-up-table row.
 // EPL > 0: the row's keys live in EPL registers per lane (N <= 64*EPL); EPL == 0: keys in LDS.
 // LOW_BIT: lowest key bit that can differ (16 for 16-bit score dtypes, whose low bits are zero).
 template <typename IO, int EPL, int LOW_BIT>
@@ -318,6 +439,7 @@ __global__ __launch_bounds__(256) void topk_kernel(const typename IO::raw* __res
                                                    int8_t* __restrict__ sparse_map, void* __restrict__ lut, int lut64, int N,
                                                    int T, size_t nrows) {
   extern __shared__ uint32_t lds_keys[];
+  __shared__ __attribute__((aligned(16))) uint32_t hist_all[4][256];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const size_t row = (size_t)blockIdx.x * 4 + wave;
   if (row >= nrows) return;
@@ -342,26 +464,61 @@ __global__ __launch_bounds__(256) void topk_kernel(const typename IO::raw* __res
     const int i = e * 64 + lane;
     return i < N ? keys[i] : 0u;
   };
-  uint32_t thr = 0;
-  for (int bit = 31; bit >= LOW_BIT; --bit) {
-    const uint32_t cand = thr | (1u << bit);
-    int cnt = 0;
+  // Radix select, eight key bits per pass (two passes for bf16 scores): the keys that agree with the digits found
+  // so far are counted per value of the next digit in a 256-bin histogram (LDS atomics of this wave on its own
+  // bins); lane l then owns the four highest undecided digits 255 - 4l .. 252 - 4l, a prefix sum over the lanes
+  // gives the number of keys above them, and the one lane whose digits straddle the wanted rank names the digit.
+  if (T <= 0) {              // nothing to select (a ratio that rounds to no block at all): an all-zero map row, no table row
+    int8_t* zrow = sparse_map + row * N;
+    for (int i = lane; i < N; i += 64) zrow[i] = 0;
+    return;
+  }
+  uint32_t thr = 0;          // digits decided so far
+  int need = T;              // rank of the threshold among the keys that agree with them
+  uint32_t* hist = hist_all[wave];
+#pragma unroll
+  for (int hi = 32; hi > LOW_BIT;) {
+    const int w = (hi - LOW_BIT) < 8 ? (hi - LOW_BIT) : 8;
+    const int shift = hi - w;
+    *reinterpret_cast<i32x4_t*>(&hist[4 * lane]) = i32x4_t{0, 0, 0, 0};
+    wave_lds_fence();
+    auto count_key = [&](int e, uint32_t kv) {
+      const bool in = e * 64 + lane < N;
+      const bool agrees = hi == 32 || ((kv ^ thr) >> (hi & 31)) == 0;
+      if (in && agrees) atomicAdd(&hist[(kv >> shift) & ((1u << w) - 1u)], 1u);
+    };
     if (EPL > 0) {
 #pragma unroll
-      for (int e = 0; e < NR; ++e) cnt += __popcll(__ballot((e * 64 + lane < N) && kreg[e] >= cand));
+      for (int e = 0; e < NR; ++e) count_key(e, kreg[e]);
     } else {
-      for (int e = 0; e < nit; ++e) cnt += __popcll(__ballot((e * 64 + lane < N) && key_at(e) >= cand));
+      for (int e = 0; e < nit; ++e) count_key(e, key_at(e));
     }
-    if (cnt >= T) thr = cand;
-  }
-  int n_gt = 0;
-  if (EPL > 0) {
+    wave_lds_fence();
+    const i32x4_t c4 = *reinterpret_cast<const i32x4_t*>(&hist[252 - 4 * lane]);    // digits 252 - 4l .. 255 - 4l
+    const int c[4] = {c4[3], c4[2], c4[1], c4[0]};                                   // in descending order of the digit
+    const int mine = c[0] + c[1] + c[2] + c[3];
+    const int incl = wave_inclusive_sum(mine, lane);
+    const int above = incl - mine;               // keys (among those that agree) whose digit is above all of this lane's
+    const bool here = above < need && need <= incl;
+    int digit = 0, rest = 0;
 #pragma unroll
-    for (int e = 0; e < NR; ++e) n_gt += __popcll(__ballot((e * 64 + lane < N) && kreg[e] > thr));
-  } else {
-    for (int e = 0; e < nit; ++e) n_gt += __popcll(__ballot((e * 64 + lane < N) && key_at(e) > thr));
+    for (int jj = 0; jj < 4; ++jj) {             // (at most one of the four digits straddles the rank)
+      int before = above;
+#pragma unroll
+      for (int t = 0; t < jj; ++t) before += c[t];
+      if (before < need && need <= before + c[jj]) {
+        digit = 255 - 4 * lane - jj;
+        rest = need - before;
+      }
+    }
+    const unsigned long long who = __ballot(here);
+    const int src = who ? (int)__builtin_ctzll(who) : 0;
+    digit = __builtin_amdgcn_readlane(digit, src);
+    need = __builtin_amdgcn_readlane(rest, src);
+    thr |= (uint32_t)digit << shift;
+    hi = shift;
   }
-  const int need_eq = T - n_gt;
+  const int need_eq = need;
   int run_eq = 0, run_sel = 0;
   const unsigned long long lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
   int8_t* mrow = sparse_map + row * N;
@@ -376,7 +533,7 @@ __global__ __launch_bounds__(256) void topk_kernel(const typename IO::raw* __res
     const unsigned long long bsel = __ballot(sel);
     const int pos = run_sel + __popcll(bsel & lt_mask);
     if (in) mrow[i] = sel ? 1 : 0;
-    if (sel) {
+    if (sel && pos < T) {              // (pos < T always holds; the test keeps a wrong count from ever leaving the row)
       if (lut64)
         reinterpret_cast<long long*>(lut)[row * T + pos] = i;
       else

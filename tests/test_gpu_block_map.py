@@ -28,6 +28,16 @@ def test_random_inputs(dev, dtype, L, BLKQ, BLKK, ratio):
     _compare(q, k, ratio, BLKQ, BLKK, dev)
 
 
+@pytest.mark.parametrize("D,dtype", [(128, torch.bfloat16), (64, torch.float16)])
+def test_many_rows_of_small_blocks(dev, D, dtype):
+    """256 heads of 255 x 255 blocks of 8 rows: many rows, ragged at both edges of the score tiles, both head dims
+    of the matrix-core score kernel."""
+    g = torch.Generator().manual_seed(D)
+    q = torch.randn(2, 128, 2036, D, generator=g).to(dtype)
+    k = (torch.randn(2, 128, 2036, D, generator=g) + 0.3).to(dtype)
+    _compare(q, k, 0.1, 8, 8, dev)
+
+
 def test_integer_inputs_with_ties(dev):
     # every sum is exact in fp32, many exact score ties: only the tie rule decides
     q, k = integer_inputs(1, 2, 2048, 128, seed=3, lo=-1, hi=1)
