@@ -230,6 +230,33 @@ static __device__ __forceinline__ float pin_f32(float x) {
   return x;
 }
 
+// Matrix products with their result in vector registers (the vector ALU reads it next) and the resident B operand in
+// accumulation registers.  Written as instructions because the compiler gives every MFMA of a function that uses
+// accumulation registers an accumulation-register result and would copy the scores back one register at a time.
+// (The compiler sees no MFMA here and inserts no wait states: callers keep the vector ALU away from a result for the
+// length of the product, and alternate two chains so that consecutive dependent products are 64 cycles apart.)
+template <typename Tag>
+static __device__ __forceinline__ void mfma_scores_first(f32x16_t& d, const i16x8_t& a, const i16x8_t& b) {
+  if constexpr (__is_same(Tag, bf16_tag))
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "a"(b));
+  else
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "a"(b));
+}
+template <typename Tag>
+static __device__ __forceinline__ void mfma_scores_first(f32x16_t& d, const i16x8_t& a, const i16x8_t& b, const f32x16_t& c) {
+  if constexpr (__is_same(Tag, bf16_tag))
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %3" : "=&v"(d) : "v"(a), "a"(b), "v"(c));
+  else
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %3" : "=&v"(d) : "v"(a), "a"(b), "v"(c));
+}
+template <typename Tag>
+static __device__ __forceinline__ void mfma_scores(f32x16_t& d, const i16x8_t& a, const i16x8_t& b) {
+  if constexpr (__is_same(Tag, bf16_tag))
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "a"(b));
+  else
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "a"(b));
+}
+
 static __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 static __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 

@@ -667,6 +667,10 @@ void launch_col_lists(const int8_t* sparse_map, int* list, int* count, int BH, i
                      vec_ok);
 }
 
+}  // namespace sla
+#include "sparse_bwd_stream.h"
+namespace sla {
+
 struct BwdWs {
   int seg;                  // longest stretch of a key block's list one workgroup walks
   int64_t max_items, max_slots;
@@ -681,6 +685,7 @@ static BwdWs bwd_ws(int BH, int L, int D, int BLKQ, int BLKK, int topk) {
   const int64_t entries = (int64_t)BH * M * topk;
   int64_t seg = (entries + 2047) / 2048;     // 512 resident workgroups, a quarter of the average each
   if (seg < 64) seg = 64;
+  if (seg > DKDV_STREAM_MAX_SEG) seg = DKDV_STREAM_MAX_SEG;      // (a work item's entries have to fit its LDS copy)
   w.seg = (int)seg;
   w.max_items = (int64_t)BH * N + entries / seg;
   w.max_slots = 2 * entries / seg;
@@ -724,13 +729,21 @@ static int bwd_impl(const void* q, const void* k, const void* v, const void* o, 
                      (int)w.max_items, (int)w.max_slots);
   const int total_q = BH * Mblk;
   const bool contig = lin.sl == D && ldo.sl == D;
+  // head dim 128 with 64-row query blocks has a dK/dV kernel of its own (32-bit byte offsets inside a head)
+  const bool stream_dkdv = D == 128 && BLKQ == 64 && (uint64_t)lin.sl * 2u * (uint64_t)L < (1ull << 31) &&
+                           (uint64_t)ldo.sl * 2u * (uint64_t)L < (1ull << 31);
 #define SLA_BWD_LAUNCH(CONTIG)                                                                                              \
   hipLaunchKernelGGL((bwd_dq_kernel<Tag, D, BLKQ, CONTIG>), dim3(xcd_grid(total_q)), dim3(BLKQ * 2), 0, st,                 \
                      (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse, delta, lut,     \
                      lut64, (uint16_t*)dq, lin, ldo, L, Mblk, topk, qk_scale, total_q);                                    \
-  hipLaunchKernelGGL((bwd_dkdv_kernel<Tag, D, BLKQ, CONTIG>), dim3(xcd_grid(w.max_items)), dim3(256), 0, st,               \
-                     (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse, delta, list,    \
-                     count, items, totals, part, w.seg, (uint16_t*)dk, (uint16_t*)dv, lin, ldo, L, Mblk, Nblk, qk_scale);
+  if (stream_dkdv)                                                                                                          \
+    hipLaunchKernelGGL((bwd_dkdv_stream_kernel<Tag>), dim3(xcd_grid(w.max_items)), dim3(128), 0, st, (const uint16_t*)q,    \
+                       (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse, delta, list, count, items,       \
+                       totals, part, w.seg, (uint16_t*)dk, (uint16_t*)dv, lin, ldo, L, Mblk, Nblk, qk_scale);             \
+  else                                                                                                                      \
+    hipLaunchKernelGGL((bwd_dkdv_kernel<Tag, D, BLKQ, CONTIG>), dim3(xcd_grid(w.max_items)), dim3(256), 0, st,             \
+                       (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse, delta, list,  \
+                       count, items, totals, part, w.seg, (uint16_t*)dk, (uint16_t*)dv, lin, ldo, L, Mblk, Nblk, qk_scale);
   if (contig) {
     SLA_BWD_LAUNCH(true)
   } else {

@@ -1,0 +1,355 @@
+// dK / dV of the block-sparse attention backward for 64-row query blocks at head dim 128: one workgroup of two
+// waves per key block (or per segment of a key block's list), one wave per SIMD.
+//
+// Stands in for _attn_bwd_dkdv of the reference (sparse_linear_attention/kernel.py:160-237) like bwd_dkdv_kernel,
+// whose work items, lists and arithmetic it shares.  What differs:
+//   * a wave owns 32 keys and the whole head dimension: K^T and V^T fragments (B operands of S = Q K^T and
+//     dP = dO V^T) and the dK^T / dV^T accumulators (128 d x 32 keys each) stay in its registers, P and dS leave
+//     the accumulators in the B-operand layout of dV^T += dO^T P and dK^T += Q^T dS.  Nothing is handed from wave
+//     to wave, and there is one barrier per 32 query rows;
+//   * Q and dO rows go from memory straight into LDS (buffer loads with the LDS bit), 32 rows at a time, into a
+//     ring of four generations; the rows of unit u + 3 are requested while unit u is worked on.  Rows are unpadded;
+//     the 16-byte pieces of a row are XOR-swizzled with the row index so that both the row-wise reads (A operands
+//     of S and dP) and the transposing reads (A operands of the second products) are free of bank conflicts;
+//   * the loop is rotated: the exponentials and the rest of the vector arithmetic of unit u run beside the first
+//     products of unit u + 1, then come the second products of unit u.
+#pragma once
+#include "common.h"
+
+namespace sla {
+
+// 16 bytes per lane, memory -> LDS: lane l's piece lands at lds_base + lds_off + 16 l
+static __device__ __forceinline__ void lds_dma_b128(__amdgpu_buffer_rsrc_t rsrc, uint32_t byte_off, uint32_t lds_base,
+                                                    uint32_t lds_off) {
+  asm volatile("s_add_u32 m0, %0, %3\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(lds_base), "v"(byte_off), "s"(rsrc),
+               "s"(lds_off)
+               : "memory", "scc");
+}
+// 4 bytes per lane: lane l's word lands at lds_base + lds_off + 4 l
+static __device__ __forceinline__ void lds_dma_b32(__amdgpu_buffer_rsrc_t rsrc, uint32_t byte_off, uint32_t lds_base,
+                                                   uint32_t lds_off) {
+  asm volatile("s_add_u32 m0, %0, %3\n\tbuffer_load_dword %1, %2, 0 offen lds" ::"s"(lds_base), "v"(byte_off), "s"(rsrc),
+               "s"(lds_off)
+               : "memory", "scc");
+}
+
+constexpr int DKDV_STREAM_MAX_SEG = 1024;      // list entries one work item may have (they are copied into LDS)
+
+template <typename Tag>
+__global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) void bwd_dkdv_stream_kernel(
+    const uint16_t* __restrict__ q, const uint16_t* __restrict__ k, const uint16_t* __restrict__ v,
+    const uint16_t* __restrict__ d_o, const float* __restrict__ lse, const float* __restrict__ delta,
+    const int* __restrict__ list, const int* __restrict__ count, const i32x4_t* __restrict__ items,
+    const int* __restrict__ totals, float* __restrict__ part, int seg, uint16_t* __restrict__ dk, uint16_t* __restrict__ dv,
+    const RowLayout lin, const RowLayout ldo, int L, int Mblk, int Nblk, float qk_scale) {
+  using E = Elem<Tag>;
+  constexpr int D = 128, DC = D / 16, DT = D / 32;
+  constexpr int ROWB = D * 2;               // bytes per row in LDS (unpadded)
+  constexpr int TILE = 32 * ROWB;           // 32 rows of Q or of dO
+  constexpr int GEN = 2 * TILE + 256;       // one generation: Q rows, dO rows, 32 log-sum-exps, 32 deltas
+  constexpr int NG = 4;
+  constexpr int NREQ = 9;                   // requests per wave and unit: 4 x Q, 4 x dO (its 16 rows), 1 x lse or delta
+  __shared__ __attribute__((aligned(16))) uint8_t smem[NG * GEN];
+  // This work item's list entries.  (Read from memory inside the loop they would be vector loads - the inline assembly
+  // keeps the compiler from using the scalar path - and waiting for a vector load means waiting for every memory ->
+  // LDS request issued before it.)
+  __shared__ int entries[DKDV_STREAM_MAX_SEG];
+
+  // work item (see bwd_dkdv_kernel)
+  const int total = totals[0];
+  const int per_xcd = (total + 7) >> 3;
+  if ((int)(blockIdx.x >> 3) >= per_xcd) return;
+  const int logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  if (logical >= total) return;
+  const i32x4_t item = items[logical];
+  const int bh = __builtin_amdgcn_readfirstlane(item[0]), nb = __builtin_amdgcn_readfirstlane(item[1]);
+  const int sg = __builtin_amdgcn_readfirstlane(item[2]), slot = __builtin_amdgcn_readfirstlane(item[3]);
+  if (slot < -1) return;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);         // keys 32w .. 32w+31 of the block
+  const int g = lane >> 5, r = lane & 31;
+  const float c_log2e = qk_scale * 1.4426950408889634f;
+
+  const size_t head_off = lin.head(bh);
+  const uint32_t pitch = (uint32_t)lin.sl, pitch_do = (uint32_t)ldo.sl;
+  const __amdgpu_buffer_rsrc_t qh = make_rsrc(q + head_off, lin.head_range_bytes(L, D));
+  const __amdgpu_buffer_rsrc_t doh = make_rsrc(d_o + ldo.head(bh), ldo.head_range_bytes(L, D));
+  const __amdgpu_buffer_rsrc_t kb = make_rsrc(k + head_off, lin.head_range_bytes(L, D));
+  const __amdgpu_buffer_rsrc_t vb = make_rsrc(v + head_off, lin.head_range_bytes(L, D));
+  // wave 0 fetches the log-sum-exps of a unit, wave 1 its deltas
+  const __amdgpu_buffer_rsrc_t ldh = make_rsrc((w ? delta : lse) + (size_t)bh * L, (uint32_t)L * 4);
+
+  // K^T and V^T fragments (B operands): this lane's key column, 8 adjacent d per chunk; parked in accumulation registers
+  const int krow = nb * 64 + w * 32 + r;
+  const bool kok = krow < L;
+  i16x8_t kf[DC], vf[DC];
+#pragma unroll
+  for (int c = 0; c < DC; ++c) {
+    kf[c] = buf_load_b128(kb, ((uint32_t)krow * pitch + 16 * c + 8 * g) * 2);     // rows past L read as zero
+    vf[c] = buf_load_b128(vb, ((uint32_t)krow * pitch + 16 * c + 8 * g) * 2);
+  }
+  // Rows past L are never written into LDS (they lie outside the buffers), and what LDS holds in their place must
+  // be finite: their probabilities are exactly 0 (log-sum-exp +inf), and 0 times a finite number adds nothing.
+#pragma unroll
+  for (int i = 0; i < (NG * GEN / 16 + 127) / 128; ++i)
+    if (i * 128 + tid < NG * GEN / 16) reinterpret_cast<i32x4_t*>(smem)[i * 128 + tid] = i32x4_t{0, 0, 0, 0};
+
+  f32x16_t dkacc[DT], dvacc[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      dkacc[dt][i] = 0.f;
+      dvacc[dt][i] = 0.f;
+    }
+
+  // this work item's part of the list, in units of 32 query rows (two per listed query block)
+  const int* mylist = list + ((size_t)bh * Nblk + nb) * Mblk;
+  const int e0 = sg * seg;
+  const int e1 = min(__builtin_amdgcn_readfirstlane(count[(size_t)bh * Nblk + nb]), (sg + 1) * seg);
+  const int nunits = 2 * (e1 - e0);
+  auto entry_row0 = [&](int e) __attribute__((always_inline)) -> int {          // past the end: the last entry again (fetched, never used)
+    return __builtin_amdgcn_readfirstlane(entries[min(e, e1 - e0 - 1)]) * 64;
+  };
+
+  for (int i = tid; i < e1 - e0; i += 128) entries[i] = mylist[e0 + i];
+
+  // ---- addressing ----
+  // A request moves 4 rows (64 lanes x 16 bytes): lane -> row 4j + lane / 16 of this wave's 16 rows, 16-byte slot
+  // lane % 16, which receives piece (slot ^ swz(row)) of that row.  swz(row) = 4 (row % 4) + (row / 4) % 4: for one
+  // piece the 16 rows of a row-wise read hit 16 different slots, and the 4 rows x 4 pieces of a transposing read too.
+  auto swz = [](int row) __attribute__((always_inline)) { return ((row & 3) << 2) | ((row >> 2) & 3); };
+  const uint32_t smem_addr = (uint32_t)(size_t)smem;
+  const int lrow = lane >> 4, lslot = lane & 15;
+  uint32_t qoff[4], dooff[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int row = 16 * w + 4 * j + lrow;                     // row of the unit (16 w: a multiple of 16, no part in swz)
+    const uint32_t piece = (uint32_t)(lslot ^ swz(row & 15)) * 16;
+    qoff[j] = (uint32_t)row * pitch * 2 + piece;
+    dooff[j] = (uint32_t)row * pitch_do * 2 + piece;
+  }
+  // LDS addresses of this wave's 16 rows inside a tile and of its 32 words (log-sum-exps or deltas) behind the tiles
+  const uint32_t rows_base = __builtin_amdgcn_readfirstlane(smem_addr + (uint32_t)(16 * w) * ROWB);
+  const uint32_t ld_base = __builtin_amdgcn_readfirstlane(smem_addr + (uint32_t)w * 128);
+  auto request = [&](int row0, int gen) __attribute__((always_inline)) {
+    const uint32_t base = (uint32_t)gen * GEN;
+    const uint32_t rq = (uint32_t)row0 * pitch * 2, rdo = (uint32_t)row0 * pitch_do * 2;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      lds_dma_b128(qh, qoff[j] + rq, rows_base, base + j * 1024);
+      lds_dma_b128(doh, dooff[j] + rdo, rows_base, base + TILE + j * 1024);
+    }
+    if (lane < 32) lds_dma_b32(ldh, (uint32_t)(row0 + lane) * 4, ld_base, base + 2 * TILE);
+  };
+  // row-wise fragment c of this lane: row r, piece 2c + g
+  int rfo[DC];
+#pragma unroll
+  for (int c = 0; c < DC; ++c) rfo[c] = r * ROWB + (((2 * c + g) ^ swz(r & 15)) * 16);
+  // transposed fragment (16 query rows x 32 d): rows 16 c2 + 4 g + (lane % 16) / 4 and 8 further on, 8 bytes at element
+  // 4 (lane % 4) of the 16-column strip 2 dt + (lane / 16) % 2
+  const int tr_row = 4 * g + ((lane & 15) >> 2);
+  int tfo[2][DT];                    // [which of the two rows][dt], without the 16 c2 rows
+#pragma unroll
+  for (int h = 0; h < 2; ++h)
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      const int row = tr_row + 8 * h;
+      const int piece = 4 * dt + 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);
+      tfo[h][dt] = row * ROWB + ((piece ^ swz(row & 15)) * 16) + (lane & 1) * 8;
+    }
+
+  // ---- prologue: units 0, 1, 2 requested; S and dP of unit 0 ----
+  f32x16_t s_a, dp_a, s_b, dp_b;
+#pragma unroll
+  for (int c = 0; c < DC; ++c) asm volatile("" : "+a"(kf[c]), "+a"(vf[c]));
+  __syncthreads();                                             // the zeros are in place before anything is requested
+  // first query rows of the listed blocks: E0 = of the entry of units u and u + 1, E1 = of the next one, E2 = of the one after
+  int E0 = 0, E1 = 0, E2 = 0;
+  if (nunits > 0) {
+    E0 = entry_row0(0);
+    E1 = entry_row0(1);
+    E2 = entry_row0(2);
+    request(E0, 0);
+    request(E0 + 32, 1);
+    request(E1, 2);
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NREQ) : "memory");
+    __syncthreads();
+#pragma unroll
+    for (int c = 0; c < DC; ++c) {
+      const i16x8_t a = *reinterpret_cast<const i16x8_t*>(smem + rfo[c]);
+      const i16x8_t b = *reinterpret_cast<const i16x8_t*>(smem + TILE + rfo[c]);
+      if (c == 0) {
+        mfma_scores_first<Tag>(s_a, a, kf[c]);
+        mfma_scores_first<Tag>(dp_a, b, vf[c]);
+      } else {
+        mfma_scores<Tag>(s_a, a, kf[c]);
+        mfma_scores<Tag>(dp_a, b, vf[c]);
+      }
+    }
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");         // (the vector ALU reads these results next)
+  }
+
+  // What one iteration fetches from LDS for the next one (the data landed long before): the log-sum-exps and deltas of
+  // its 32 query rows (accumulator register 4 i4 + j of S / dP is query row 8 i4 + 4 g + j of the unit; this lane's
+  // column is its key) and the transposed fragments of its first two groups of second products.
+  f32x4_t l4[4], d4[4];
+  i16x8_t trd[4], trq[4];            // transposed dO / Q fragments of group grp in slot grp % 4, fetched two groups ahead
+  auto row_scalars = [&](const uint8_t* gen, int i4) __attribute__((always_inline)) {
+    l4[i4] = *reinterpret_cast<const f32x4_t*>(gen + 2 * TILE + (8 * i4 + 4 * g) * 4);
+    d4[i4] = *reinterpret_cast<const f32x4_t*>(gen + 2 * TILE + 128 + (8 * i4 + 4 * g) * 4);
+  };
+  auto tr_frags = [&](const uint8_t* gen, int grp) __attribute__((always_inline)) {
+    const int c2 = grp >> 2, dt = grp & 3;
+    const uint8_t* t0 = gen + 16 * c2 * ROWB;
+    trd[grp & 3] = concat4(lds_read_tr16(reinterpret_cast<const uint16_t*>(t0 + TILE + tfo[0][dt])),
+                           lds_read_tr16(reinterpret_cast<const uint16_t*>(t0 + TILE + tfo[1][dt])));
+    trq[grp & 3] = concat4(lds_read_tr16(reinterpret_cast<const uint16_t*>(t0 + tfo[0][dt])),
+                           lds_read_tr16(reinterpret_cast<const uint16_t*>(t0 + tfo[1][dt])));
+  };
+  if (nunits > 0) {
+#pragma unroll
+    for (int i4 = 0; i4 < 4; ++i4) row_scalars(smem, i4);
+    tr_frags(smem, 0);
+    tr_frags(smem, 1);
+  }
+
+  // One iteration = unit u, 32 MFMAs:
+  //   slots  0..15  S and dP of unit u + 1 (two chains)      beside: P and dS of unit u
+  //   slots 16..31  dV^T += dO^T P, dK^T += Q^T dS of unit u  beside: the requests for unit u + 3, and what the next
+  //                                                            iteration wants from LDS first (see above)
+  // On entry: s_cur, dp_cur = Q K^T and dO V^T of unit u.  Before anything else: this wave's part of unit u + 1 has
+  // landed (all but the latest nine requests), one barrier (the partner's part too; everyone is done with unit u - 1,
+  // whose generation the requests for u + 3 overwrite).  A single wave per SIMD has nobody to hide its LDS latency:
+  // every fragment is fetched three products (row-wise) or two groups (transposed) before it is used, and the first
+  // four elements of the vector arithmetic run while the first row-wise fragments are on their way.
+  // GU = u % 4: the generation of unit u.  (Unrolling four iterations to make it a constant costs more registers
+  // than the kernel has: the compiler then spills the resident fragments.)
+  auto iteration = [&](int GU, f32x16_t& s_cur, f32x16_t& dp_cur, f32x16_t& s_nxt, f32x16_t& dp_nxt, int row0_u,
+                       int row0_req) __attribute__((always_inline)) {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NREQ) : "memory");
+    __syncthreads();
+    const uint8_t* gu = smem + GU * GEN;                       // unit u: transposed reads
+    const uint8_t* gn = smem + ((GU + 1) & 3) * GEN;           // unit u + 1: row-wise reads, scalars, first transposed reads
+    i16x8_t af[4], bf[4];
+#pragma unroll
+    for (int c = 0; c < 3; ++c) {
+      af[c] = *reinterpret_cast<const i16x8_t*>(gn + rfo[c]);
+      bf[c] = *reinterpret_cast<const i16x8_t*>(gn + TILE + rfo[c]);
+    }
+    if (__builtin_expect(row0_u + 32 > L, 0)) {                // rows past L: +inf makes every probability exactly 0
+#pragma unroll
+      for (int i4 = 0; i4 < 4; ++i4)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (row0_u + 8 * i4 + 4 * g + j >= L) {
+            l4[i4][j] = INFINITY;
+            d4[i4][j] = 0.f;
+          }
+    }
+    i32x4_t pw[2], dw[2];
+    // element i of unit u: P = exp2(S c - lse), dS = P (dP - delta); packed in pairs
+    auto element = [&](int i) __attribute__((always_inline)) {
+      float p = fast_exp2(__builtin_fmaf(s_cur[i], c_log2e, -l4[i >> 2][i & 3]));
+      float ds = p * (dp_cur[i] - d4[i >> 2][i & 3]);
+      asm volatile("" : "+v"(p), "+v"(ds));
+      s_cur[i] = p;
+      dp_cur[i] = ds;
+      if (i & 1) {
+        uint32_t a = E::pack2(s_cur[i - 1], s_cur[i]), b = E::pack2(dp_cur[i - 1], dp_cur[i]);
+        asm volatile("" : "+v"(a), "+v"(b));
+        pw[i >> 3][(i >> 1) & 3] = (int)a;
+        dw[i >> 3][(i >> 1) & 3] = (int)b;
+      }
+    };
+#pragma unroll
+    for (int i = 0; i < 4; ++i) element(i);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int c = 0; c < DC; ++c) {
+      if (c + 3 < DC) {
+        af[(c + 3) & 3] = *reinterpret_cast<const i16x8_t*>(gn + rfo[c + 3]);
+        bf[(c + 3) & 3] = *reinterpret_cast<const i16x8_t*>(gn + TILE + rfo[c + 3]);
+      }
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        if (half == 0) {
+          if (c == 0) mfma_scores_first<Tag>(s_nxt, af[c & 3], kf[c]);
+          else mfma_scores<Tag>(s_nxt, af[c & 3], kf[c]);
+        } else {
+          if (c == 0) mfma_scores_first<Tag>(dp_nxt, bf[c & 3], vf[c]);
+          else mfma_scores<Tag>(dp_nxt, bf[c & 3], vf[c]);
+        }
+        const int sl = 2 * c + half;                           // twelve elements left for sixteen slots
+        if (sl < 12) element(4 + sl);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    // (a key row past L only ever feeds its own, never stored, column of dK^T / dV^T: no masking needed)
+    const uint32_t req_base = (uint32_t)((GU + 3) & 3) * GEN;
+    const uint32_t rq = (uint32_t)row0_req * pitch * 2, rdo = (uint32_t)row0_req * pitch_do * 2;
+    // eight groups (c2, dt) of two products
+#pragma unroll
+    for (int grp = 0; grp < 8; ++grp) {
+      const int c2 = grp >> 2, dt = grp & 3;
+      if (grp + 2 < 8) tr_frags(gu, grp + 2);
+      else tr_frags(gn, grp + 2 - 8);                          // the next unit's first two groups
+      if (grp >= 4) row_scalars(gn, grp - 4);                  // and its scalars
+      dvacc[dt] = E::mfma32(trd[grp & 3], __builtin_bit_cast(i16x8_t, pw[c2]), dvacc[dt]);
+      dkacc[dt] = E::mfma32(trq[grp & 3], __builtin_bit_cast(i16x8_t, dw[c2]), dkacc[dt]);
+      if (grp < 4) {
+        lds_dma_b128(qh, qoff[grp] + rq, rows_base, req_base + grp * 1024);
+        lds_dma_b128(doh, dooff[grp] + rdo, rows_base, req_base + TILE + grp * 1024);
+      } else if (grp == 4) {
+        if (lane < 32) lds_dma_b32(ldh, (uint32_t)(row0_req + lane) * 4, ld_base, req_base + 2 * TILE);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  for (int u = 0; u < nunits; u += 2) {
+    const int E3 = entry_row0((u >> 1) + 3);                        // (looked up now, used two units from now)
+    iteration(u & 3, s_a, dp_a, s_b, dp_b, E0, E1 + 32);            // unit u; requests unit u + 3
+    iteration((u + 1) & 3, s_b, dp_b, s_a, dp_a, E0 + 32, E2);      // unit u + 1; requests u + 4
+    E0 = E1;
+    E1 = E2;
+    E2 = E3;
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");    // (nothing of this workgroup is in flight when it ends)
+
+  if (slot >= 0) {
+    // one segment of a long list: fp32 partial [dk | dv][64][D], added up by bwd_dkdv_reduce_kernel
+    float* pk = part + (size_t)slot * (2 * 64 * D) + (size_t)(w * 32 + r) * D;
+    float* pv = pk + 64 * D;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; ++i4) {
+        const int d0 = 32 * dt + 8 * i4 + 4 * g;
+        *reinterpret_cast<f32x4_t*>(pk + d0) = f32x4_t{dkacc[dt][4 * i4 + 0] * qk_scale, dkacc[dt][4 * i4 + 1] * qk_scale,
+                                                       dkacc[dt][4 * i4 + 2] * qk_scale, dkacc[dt][4 * i4 + 3] * qk_scale};
+        *reinterpret_cast<f32x4_t*>(pv + d0) =
+            f32x4_t{dvacc[dt][4 * i4 + 0], dvacc[dt][4 * i4 + 1], dvacc[dt][4 * i4 + 2], dvacc[dt][4 * i4 + 3]};
+      }
+    return;
+  }
+  if (kok) {
+    uint16_t* dkrow = dk + head_off + (size_t)krow * pitch;
+    uint16_t* dvrow = dv + head_off + (size_t)krow * pitch;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; ++i4) {
+        const int d0 = 32 * dt + 8 * i4 + 4 * g;
+        i32x2_t wv;
+        wv[0] = (int)E::pack2(dkacc[dt][4 * i4 + 0] * qk_scale, dkacc[dt][4 * i4 + 1] * qk_scale);
+        wv[1] = (int)E::pack2(dkacc[dt][4 * i4 + 2] * qk_scale, dkacc[dt][4 * i4 + 3] * qk_scale);
+        *reinterpret_cast<i32x2_t*>(dkrow + d0) = wv;
+        wv[0] = (int)E::pack2(dvacc[dt][4 * i4 + 0], dvacc[dt][4 * i4 + 1]);
+        wv[1] = (int)E::pack2(dvacc[dt][4 * i4 + 2], dvacc[dt][4 * i4 + 3]);
+        *reinterpret_cast<i32x2_t*>(dvrow + d0) = wv;
+      }
+  }
+}
+
+}  // namespace sla

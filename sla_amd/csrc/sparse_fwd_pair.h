@@ -31,33 +31,6 @@ namespace sla {
 
 constexpr int PAIR_MAX_T = 1024;      // look-up rows longer than this, or more than 4096 key blocks, take sparse_fwd_kernel
 
-// Score products with their result in vector registers (the exponentials read it next) and the resident Q^T operand in
-// accumulation registers.  Written as instructions because the compiler gives every MFMA of a function that uses
-// accumulation registers an accumulation-register result and would copy the scores back one register at a time.
-// (Hazards: a score tile is read by the vector ALU an iteration after its last product, and the two chains alternate,
-// so consecutive dependent products are 64 cycles apart.)
-template <typename Tag>
-static __device__ __forceinline__ void mfma_scores_first(f32x16_t& d, const i16x8_t& a, const i16x8_t& b) {
-  if constexpr (__is_same(Tag, bf16_tag))
-    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "a"(b));
-  else
-    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "a"(b));
-}
-template <typename Tag>
-static __device__ __forceinline__ void mfma_scores_first(f32x16_t& d, const i16x8_t& a, const i16x8_t& b, const f32x16_t& c) {
-  if constexpr (__is_same(Tag, bf16_tag))
-    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %3" : "=&v"(d) : "v"(a), "a"(b), "v"(c));
-  else
-    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %3" : "=&v"(d) : "v"(a), "a"(b), "v"(c));
-}
-template <typename Tag>
-static __device__ __forceinline__ void mfma_scores(f32x16_t& d, const i16x8_t& a, const i16x8_t& b) {
-  if constexpr (__is_same(Tag, bf16_tag))
-    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "a"(b));
-  else
-    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "a"(b));
-}
-
 template <typename Tag, bool FUSED>
 __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) void sparse_fwd_pair_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ k, const uint16_t* __restrict__ v, const void* __restrict__ lut,
