@@ -298,16 +298,23 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
   const int tr_key = 8 * (slot >> 2) + 4 * g + (slot & 3);
   const int tr_col = 16 * ((lane >> 4) & 1) + 8 * (li & 1);
 
-  // S^T of one tile: raw int32 products of both 32-key halves
+  // The integer products start from the bit pattern of the float 1.5 * 2^23 instead of from zero: the integer
+  // MAGIC + s, read as a float, IS the float 12582912 + s (|s| <= 128 * 127^2 < 2^22 stays inside the binade whose
+  // unit in the last place is 1), so the scores reach the exponent's multiply-add without an int -> float
+  // conversion per element; 12582912 * sc joins the constant that multiply-add subtracts.
+  constexpr int MAGIC = 0x4B400000;
+  constexpr float MAGIC_F = 12582912.0f;
+  i32x16_t magic;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) magic[i] = MAGIC;
+  // S^T of one tile: MAGIC + raw int32 products of both 32-key halves
   auto scores = [&](int kslot, i32x16_t (&acc)[2]) {
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
 #pragma unroll
-      for (int i = 0; i < 16; ++i) acc[t][i] = 0;
-#pragma unroll
       for (int c = 0; c < QC; ++c) {
         const i32x4_t a = *reinterpret_cast<const i32x4_t*>(&sK[kslot][(32 * t + r) * STR + 32 * c + 16 * g]);
-        acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, qf[c], acc[t], 0, 0, 0);
+        acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, qf[c], c == 0 ? magic : acc[t], 0, 0, 0);
       }
     }
   };
@@ -318,7 +325,7 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) s[t][i] = (float)acc[t][i];
+      for (int i = 0; i < 16; ++i) s[t][i] = __int_as_float(acc[t][i]);         // = 12582912 + score
     if (kv_valid < BLKK) {                 // ragged last key block: missing rows take no part
       const int lim = kv_valid - 4 * g;    // key index of register i is 32t + 8(i/4) + i%4 + 4g
 #pragma unroll
@@ -333,6 +340,7 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[t][i]);
+    mx -= MAGIC_F;                         // (exact: both are integers below 2^24)
     if (__any(mx * sc > m_used + TAU)) {   // rare: move the reference and rescale what is accumulated
       float m_new = fmaxf(mx, __shfl_xor(mx, 32)) * sc;
       m_new = fmaxf(m_used, m_new);
@@ -346,7 +354,7 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
         for (int i = 0; i < 16; ++i) oacc[dt][i] *= f;
     }
     // 112 p = exp2(s*sc - (m_used - log2 112)); -inf scores give exactly 0
-    const float m_off = m_used - LOG2_P_SCALE;
+    const float m_off = __builtin_fmaf(MAGIC_F, sc, m_used - LOG2_P_SCALE);
     i32x8_t pb;
 #pragma unroll
     for (int t = 0; t < 2; ++t)
