@@ -162,7 +162,8 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   // unit u = 2 * step + half.  Shared steps: one tile, slot 0, wave w fetches rows 16w..16w+15 of the half-tile
   // (4 instructions of 1 KB for K, 4 for V).  Own steps: slot w, the wave fetches all 32 rows (8 + 8 instructions).
   // Instruction i of a half-tile fills LDS rows 4i..4i+3: lane -> row 4i + lane / 16, 16-byte slot lane % 16, which
-  // receives piece (slot ^ swizzle(row)) of that row.  K: swizzle = row % 16; V: 2 * (row % 8).
+  // receives piece (slot ^ swizzle(row)) of that row.  K: swizzle = row % 16 (the 16 rows of a row-wise read hit 16 different
+  // slots); V: 4 (row % 4) + (row / 4) % 2 (so do the 4 rows x 4 pieces of a transposing read).
   // A single wave per SIMD pays issue time for every instruction, scalar ones included, so everything that does not
   // change inside the loop is formed here: per instruction there is one vector add (lane part + scalar row base), one
   // scalar add into M0 (LDS destination) and the load.
@@ -174,7 +175,7 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     koff[j] = (uint32_t)(4 * j + lrow) * row_bytes + ((lslot ^ ((4 * j + lrow) & 15)) * 16);
-    voff[j] = (uint32_t)(4 * j + lrow) * row_bytes + ((lslot ^ ((((4 * j + lrow) & 7) << 1) & 15)) * 16);
+    voff[j] = (uint32_t)(4 * j + lrow) * row_bytes + ((lslot ^ ((((4 * j + lrow) & 3) << 2) | (((4 * j + lrow) >> 2) & 1))) * 16);
   }
   // What the requests of a step need, by kind of step: the byte offset of the first row this wave fetches and the LDS
   // address (inside a slot pair) of its first instruction.
@@ -212,7 +213,7 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   for (int c = 0; c < DC; ++c) kfo[c] = r * ROWB + (((2 * c + g) ^ (r & 15)) * 16);
   const int tr_row = (lane & 15) >> 2;
   const int v_row = 4 * g + tr_row;                  // + 16 * group (+ 8 for the second read)
-  const int v_swz = ((v_row & 7) << 1) & 15;
+  const int v_swz = ((v_row & 3) << 2) | ((v_row >> 2) & 1);      // (the same for row + 8)
   int vfo[DT];                      // V^T fragment dt: 8 bytes at element 4 * (lane % 4) of the 16-column strip 2 dt + (lane / 16) % 2
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) {
