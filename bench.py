@@ -210,6 +210,8 @@ def main():
     ap.add_argument("--workload", default="cfg3")
     ap.add_argument("--cpu-heads", type=int, default=12, help="heads of the workload timed on the CPU oracle (0 = skip)")
     ap.add_argument("--no-extras", action="store_true", help="skip the per-kernel, backward and SageSLA timings")
+    ap.add_argument("--one-config", action="store_true",
+                    help="keep the extras of the workload itself, skip the other configurations (for profiler runs)")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run one plain 1 GiB read + 1 GiB write elementwise kernel, the known-size reference for "
                          "scaling the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
@@ -334,7 +336,7 @@ def main():
         except (AssertionError, RuntimeError, NotImplementedError) as e:
             extra["sla_fwd_complement_mode_ms"] = None
             extra["complement_note"] = str(e)[:200]
-    if not args.no_extras and cfg.name == "cfg3":
+    if not args.no_extras and not args.one_config and cfg.name == "cfg3":
         extra.update(other_configs(torch, dev, max(args.steps // 10, 3)))
     if args.pmc_calibration:
         x = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()

@@ -7,9 +7,9 @@
 //   * a wave owns all 64 rows of its query block (two 32-row tiles), so every K fragment and every V^T fragment
 //     read from LDS feeds two MFMAs: half the LDS reads per MFMA of the 32-rows-per-wave kernel;
 //   * neighbouring query blocks select mostly the same key blocks.  The two look-up rows of a pair are split
-//     into the key blocks both selected ("shared", walked first, one copy of the tile in LDS for both waves)
-//     and the rest ("own": as many on either side, each wave walks its own, two tiles in LDS).  A pair that
-//     shares 19 of 25 key blocks moves 31 tiles instead of 50 from L2 into LDS;
+//     into the key blocks both selected ("shared": one copy of the tile in LDS for both waves) and the rest
+//     ("own": as many on either side, each wave walks its own, two tiles in LDS), interleaved in the order of
+//     the first row.  A pair that shares 19 of 25 key blocks moves 31 tiles instead of 50 from L2 into LDS;
 //   * a wave has the whole register file of its SIMD (one wave per SIMD): the next half-tiles of K and V wait
 //     in registers for a whole half-tile of arithmetic before they are needed, and the loop is rotated so that
 //     the exponentials of half-tile u run beside the score products of u+1 and the output products of u.
@@ -49,6 +49,7 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   __shared__ __attribute__((aligned(16))) uint8_t smem[8 * SLOT];
   __shared__ uint32_t bitmap[2][128];
   __shared__ uint16_t steps[2][PAIR_MAX_T];
+  __shared__ uint16_t own_b[PAIR_MAX_T];        // the key blocks only the second row names (wave 1's scratch)
   __shared__ int repeated;
   static_assert(2 * 32 * SSTR * 2 <= 4 * SLOT, "the staging tiles of the epilogue exceed the K ring");
 
@@ -91,7 +92,7 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     for (int i = 0; i < 4 * SLOT / (128 * 16); ++i) reinterpret_cast<i32x4_t*>(smem + 4 * SLOT)[i * 128 + tid] = i32x4_t{0, 0, 0, 0};
   }
 
-  // ---- the two look-up rows -> per-wave step lists: shared key blocks first (in the order of the first row), then own
+  // ---- the two look-up rows -> per-wave step lists
   const size_t rowA = ((size_t)bh * Mblk + 2 * pj) * topk;
   const size_t rowB = pair_full ? rowA + topk : rowA;
   auto lut_at = [&](size_t i) __attribute__((always_inline)) -> int {
@@ -112,33 +113,42 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     if (((seen_a >> (a & 31)) | (seen_b >> (b & 31))) & 1u) repeated = 1;
   }
   __syncthreads();
-  int ns = 0;                                  // number of shared key blocks (the same in both waves)
+  // Step p of the pair follows entry p of the first row: a key block the second row names as well is a shared step;
+  // otherwise it is an own step, on which wave 0 takes that block and wave 1 the next block (in the order of its row)
+  // that only the second row names: both rows have as many of those.  Key blocks so come in the order of the look-up
+  // rows, ascending as the mask builder writes them, and the pairs that are resident on an XCD sweep K and V together.
+  // Bit 15 of a step marks an own step.
   if (repeated) {
     const size_t rowW = w ? rowB : rowA;
-    for (int i = lane; i < topk; i += 64) steps[w][i] = (uint16_t)(lut_at(rowW + i) & 4095);
+    for (int i = lane; i < topk; i += 64) steps[w][i] = (uint16_t)((lut_at(rowW + i) & 4095) | 0x8000);
   } else {
     const unsigned long long lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
-    int n = 0;
+    if (w == 1) {                                // the second row's own blocks, in its order
+      int n = 0;
+      for (int c0 = 0; c0 < topk; c0 += 64) {
+        const int i = c0 + lane;
+        const int x = i < topk ? lut_at(rowB + i) & 4095 : 0;
+        const bool sel = i < topk && !((bitmap[0][x >> 5] >> (x & 31)) & 1u);
+        const unsigned long long bal = __ballot(sel);
+        if (sel) own_b[n + __popcll(bal & lt_mask)] = (uint16_t)x;
+        n += __popcll(bal);
+      }
+      wave_lds_fence();
+    }
+    int n = 0;                                   // own steps before this chunk
     for (int c0 = 0; c0 < topk; c0 += 64) {
       const int i = c0 + lane;
       const int a = i < topk ? lut_at(rowA + i) & 4095 : 0;
-      const bool sel = i < topk && ((bitmap[1][a >> 5] >> (a & 31)) & 1u);
-      const unsigned long long bal = __ballot(sel);
-      if (sel) steps[w][n + __popcll(bal & lt_mask)] = (uint16_t)a;
-      n += __popcll(bal);
-    }
-    ns = n;
-    const size_t rowW = w ? rowB : rowA;
-    for (int c0 = 0; c0 < topk; c0 += 64) {
-      const int i = c0 + lane;
-      const int x = i < topk ? lut_at(rowW + i) & 4095 : 0;
-      const bool sel = i < topk && !((bitmap[1 - w][x >> 5] >> (x & 31)) & 1u);
-      const unsigned long long bal = __ballot(sel);
-      if (sel) steps[w][n + __popcll(bal & lt_mask)] = (uint16_t)x;
+      const bool own = i < topk && !((bitmap[1][a >> 5] >> (a & 31)) & 1u);
+      const unsigned long long bal = __ballot(own);
+      if (i < topk) {
+        int tile = a;
+        if (own && w == 1) tile = own_b[n + __popcll(bal & lt_mask)];
+        steps[w][i] = (uint16_t)(tile | (own ? 0x8000 : 0));
+      }
       n += __popcll(bal);
     }
   }
-  ns = __builtin_amdgcn_readfirstlane(ns);
 
   f32x16_t oacc[DT][2];
 #pragma unroll
@@ -185,8 +195,8 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     uint32_t rb;       // byte offset in the head of the first row this wave fetches of half 0
     uint32_t dst;      // LDS byte address, relative to a generation's slot pair, of this wave's first instruction
   };
-  auto step_of = [&](int s_raw, int tile) __attribute__((always_inline)) -> Step {
-    const int own = s_raw < ns ? 0 : 1;
+  auto step_of = [&](int entry) __attribute__((always_inline)) -> Step {
+    const int own = entry >> 15, tile = entry & 4095;
     return Step{tile, own, (uint32_t)(tile * 64 + (own ? 0 : 16 * w)) * row_bytes,
                 smem_addr + (uint32_t)(own ? w * SLOT : 4 * w * 1024)};
   };
@@ -220,11 +230,9 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     const int piece = 4 * dt + 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);
     vfo[dt] = 4 * SLOT + v_row * ROWB + ((piece ^ v_swz) * 16) + (lane & 1) * 8;
   }
-  // The fragment offsets move to this wave's own slot once, when the walk passes from the shared steps to the own
-  // ones: for K in the odd iteration of step ns - 1 (K_{u+1} is then the first own half-tile), for V in the even
-  // iteration of step ns.  (No shared step: the prologue has moved them.  No own step: they never move.)
-  const int k_flip_step = (ns > 0 && ns < topk) ? ns - 1 : -1;
-  const int v_flip_step = (ns > 0 && ns < topk) ? ns : -1;
+  // The fragment offsets point at the shared slot or at this wave's own slot; they move whenever the kind of the step
+  // they read from changes (k_own / v_own: where they point now).
+  int k_own = 0, v_own = 0;
   const int ragged_tile = (L & 63) ? (L >> 6) : -1;       // the only key block that can have missing rows
 
   // ---- pieces of the arithmetic ----
@@ -299,8 +307,8 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   }
   Step cur{0, 0, 0, 0}, nxt{0, 0, 0, 0};
   if (nunits > 0) {
-    cur = step_of(0, __builtin_amdgcn_readfirstlane(step_lookup(0)));
-    nxt = step_of(min(1, topk - 1), __builtin_amdgcn_readfirstlane(step_lookup(1)));
+    cur = step_of(__builtin_amdgcn_readfirstlane(step_lookup(0)));
+    nxt = step_of(__builtin_amdgcn_readfirstlane(step_lookup(1)));
     // K_0, V_0 (generation 0) and K_1 (generation 1) of the first step
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -319,6 +327,7 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
       for (int c = 0; c < DC; ++c) kfo[c] += w * SLOT;
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) vfo[dt] += w * SLOT;
+      k_own = v_own = 1;
     }
   }
   // Q is only ever an MFMA operand (unscaled: the scores stay in the units of q . k, the reference maximum too, and
@@ -389,14 +398,19 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     const uint32_t k_rb = nxt.rb + (HALF ? half_bytes : 0u);
     const uint32_t v_rb = vs.rb + (HALF ? 0u : half_bytes);
     // fragment reads: K_{u+1} is half 1 of cur (HALF 0) or half 0 of nxt (HALF 1); V_u is of cur.  Their slot changes
-    // once, when the walk passes from the shared steps to the own ones.
-    if (HALF == 1 && __builtin_expect(step_index == k_flip_step, 0)) {
+    // when the kind of step does.
+    const int k_need = HALF ? nxt.own : cur.own;
+    if (__builtin_expect(k_need != k_own, 0)) {
+      const int d = k_need ? w * SLOT : -w * SLOT;
 #pragma unroll
-      for (int c = 0; c < DC; ++c) kfo[c] += w * SLOT;
+      for (int c = 0; c < DC; ++c) kfo[c] += d;
+      k_own = k_need;
     }
-    if (HALF == 0 && __builtin_expect(step_index == v_flip_step, 0)) {
+    if (__builtin_expect(cur.own != v_own, 0)) {
+      const int d = cur.own ? w * SLOT : -w * SLOT;
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) vfo[dt] += w * SLOT;
+      for (int dt = 0; dt < DT; ++dt) vfo[dt] += d;
+      v_own = cur.own;
     }
     // the key block of the step after next is looked up now and used at the end of the odd iteration
     int tile2_lane = 0;
@@ -492,7 +506,7 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     if (HALF == 0) ps_seed = 0.f;
     if (HALF) {
       cur = nxt;
-      nxt = step_of(min(step_index + 2, topk - 1), __builtin_amdgcn_readfirstlane(tile2_lane));
+      nxt = step_of(__builtin_amdgcn_readfirstlane(tile2_lane));
     }
   };
 
