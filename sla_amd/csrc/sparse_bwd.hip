@@ -732,10 +732,16 @@ static int bwd_impl(const void* q, const void* k, const void* v, const void* o, 
   // head dim 128 with 64-row query blocks has a dK/dV kernel of its own (32-bit byte offsets inside a head)
   const bool stream_dkdv = D == 128 && BLKQ == 64 && (uint64_t)lin.sl * 2u * (uint64_t)L < (1ull << 31) &&
                            (uint64_t)ldo.sl * 2u * (uint64_t)L < (1ull << 31);
+  const bool stream_dq = stream_dkdv && topk <= DQ_STREAM_MAX_T && total_q >= 1024;      // (enough query blocks for a wave on every SIMD)
 #define SLA_BWD_LAUNCH(CONTIG)                                                                                              \
-  hipLaunchKernelGGL((bwd_dq_kernel<Tag, D, BLKQ, CONTIG>), dim3(xcd_grid(total_q)), dim3(BLKQ * 2), 0, st,                 \
-                     (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse, delta, lut,     \
-                     lut64, (uint16_t*)dq, lin, ldo, L, Mblk, topk, qk_scale, total_q);                                    \
+  if (stream_dq)                                                                                                            \
+    hipLaunchKernelGGL((bwd_dq_stream_kernel<Tag>), dim3(xcd_grid(total_q)), dim3(64), 0, st, (const uint16_t*)q,           \
+                       (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse, delta, lut, lut64, (uint16_t*)dq, \
+                       lin, ldo, L, Mblk, topk, qk_scale, total_q);                                                        \
+  else                                                                                                                      \
+    hipLaunchKernelGGL((bwd_dq_kernel<Tag, D, BLKQ, CONTIG>), dim3(xcd_grid(total_q)), dim3(BLKQ * 2), 0, st,               \
+                       (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse, delta, lut,   \
+                       lut64, (uint16_t*)dq, lin, ldo, L, Mblk, topk, qk_scale, total_q);                                  \
   if (stream_dkdv)                                                                                                          \
     hipLaunchKernelGGL((bwd_dkdv_stream_kernel<Tag>), dim3(xcd_grid(w.max_items)), dim3(128), 0, st, (const uint16_t*)q,    \
                        (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse, delta, list, count, items,       \

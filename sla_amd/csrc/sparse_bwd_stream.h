@@ -352,4 +352,262 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   }
 }
 
+
+// ---- dQ ------------------------------------------------------------------------------------------------------------
+// dQ of the block-sparse attention backward for 64-row query blocks at head dim 128: one wave per query block, one wave
+// per SIMD, no barriers.
+//
+// Stands in for _attn_bwd_dq of the reference (sparse_linear_attention/kernel.py:95-157) like bwd_dq_kernel, whose
+// arithmetic it shares (S^T = K Q^T and dP^T = V dO^T, so that the log-sum-exp and delta of a query are per-lane
+// scalars and dS^T leaves the accumulator as the B operand of dQ^T += K^T dS^T).  What differs:
+//   * the wave owns all 64 query rows (two tiles of 32): Q^T and dO^T fragments and the dQ^T accumulators fill the
+//     accumulation registers, and every transposed K fragment read from LDS feeds two products;
+//   * K and V go from memory straight into LDS, 32 keys at a time, two generations each, swizzled like the Q / dO
+//     rows of bwd_dkdv_stream_kernel; the 32 keys after next are requested as soon as the current ones are used up
+//     (the transposed K fragments wait in registers), a unit and a half before they are wanted;
+//   * inside a unit of 32 keys the two query tiles are staggered: S, dP of tile 0 | S, dP of tile 1 beside the
+//     vector arithmetic of tile 0 | dQ of tile 0 beside the vector arithmetic of tile 1 | dQ of tile 1.
+constexpr int DQ_STREAM_MAX_T = 2048;          // look-up rows longer than this take bwd_dq_kernel
+
+template <typename Tag>
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 1))) void bwd_dq_stream_kernel(
+    const uint16_t* __restrict__ q, const uint16_t* __restrict__ k, const uint16_t* __restrict__ v,
+    const uint16_t* __restrict__ d_o, const float* __restrict__ lse, const float* __restrict__ delta,
+    const void* __restrict__ lut, int lut64, uint16_t* __restrict__ dq, const RowLayout lin, const RowLayout ldo, int L,
+    int Mblk, int topk, float qk_scale, int total) {
+  using E = Elem<Tag>;
+  constexpr int D = 128, DC = D / 16, DT = D / 32;
+  constexpr int ROWB = D * 2;
+  constexpr int TILE = 32 * ROWB;                 // 32 rows of K or V
+  __shared__ __attribute__((aligned(16))) uint8_t smem[4 * TILE];      // K generation 0, 1; V generation 0, 1
+  __shared__ uint16_t entries[DQ_STREAM_MAX_T];                        // this block's look-up row
+
+  const int logical = xcd_remap(blockIdx.x, gridDim.x, total);
+  if (logical < 0) return;
+  const int bh = logical / Mblk;
+  const int mb = logical - bh * Mblk;
+  const int lane = threadIdx.x;
+  const int g = lane >> 5, r = lane & 31;
+  const float c_log2e = qk_scale * 1.4426950408889634f;
+
+  const size_t head_off = lin.head(bh);
+  const uint32_t pitch = (uint32_t)lin.sl, pitch_do = (uint32_t)ldo.sl;
+  const uint32_t row_bytes = pitch * 2;
+  const __amdgpu_buffer_rsrc_t qh = make_rsrc(q + head_off, lin.head_range_bytes(L, D));
+  const __amdgpu_buffer_rsrc_t doh = make_rsrc(d_o + ldo.head(bh), ldo.head_range_bytes(L, D));
+  const __amdgpu_buffer_rsrc_t kh = make_rsrc(k + head_off, lin.head_range_bytes(L, D));
+  const __amdgpu_buffer_rsrc_t vh = make_rsrc(v + head_off, lin.head_range_bytes(L, D));
+  const int qrow0 = mb * 64;
+
+  // Q^T and dO^T fragments (B operands; rows past L read as zero), per-lane scalars of the two query tiles
+  i16x8_t qf[2][DC], dof[2][DC];
+  float lse_q[2], delta_q[2];
+#pragma unroll
+  for (int qt = 0; qt < 2; ++qt) {
+    const int qrow = qrow0 + 32 * qt + r;
+#pragma unroll
+    for (int c = 0; c < DC; ++c) {
+      qf[qt][c] = buf_load_b128(qh, ((uint32_t)qrow * pitch + 16 * c + 8 * g) * 2);
+      dof[qt][c] = buf_load_b128(doh, ((uint32_t)qrow * pitch_do + 16 * c + 8 * g) * 2);
+    }
+    // rows past L: lse = +inf makes every probability exactly 0 (the reference loads `other=inf`)
+    lse_q[qt] = qrow < L ? lse[(size_t)bh * L + qrow] : INFINITY;
+    delta_q[qt] = qrow < L ? delta[(size_t)bh * L + qrow] : 0.f;
+  }
+  const size_t lut_row = ((size_t)bh * Mblk + mb) * topk;
+  for (int i = lane; i < topk; i += 64)
+    entries[i] = (uint16_t)(lut64 ? (int)reinterpret_cast<const long long*>(lut)[lut_row + i]
+                                  : reinterpret_cast<const int*>(lut)[lut_row + i]);
+  // key rows past L are never written into LDS: what LDS holds in their place has to be finite (their probabilities
+  // are masked to exactly 0 below)
+#pragma unroll
+  for (int i = 0; i < 4 * TILE / 16 / 64; ++i) reinterpret_cast<i32x4_t*>(smem)[i * 64 + lane] = i32x4_t{0, 0, 0, 0};
+  wave_lds_fence();
+
+  f32x16_t dqacc[DT][2];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int qt = 0; qt < 2; ++qt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) dqacc[dt][qt][i] = 0.f;
+
+  // ---- addressing (see bwd_dkdv_stream_kernel) ----
+  auto swz = [](int row) __attribute__((always_inline)) { return ((row & 3) << 2) | ((row >> 2) & 3); };
+  const uint32_t smem_addr = __builtin_amdgcn_readfirstlane((uint32_t)(size_t)smem);
+  const int lrow = lane >> 4, lslot = lane & 15;
+  uint32_t koff[4];                  // request j covers rows 4 j + lane / 16 of the 32: j % 4 here, 16 rows more for j >= 4
+#pragma unroll
+  for (int j = 0; j < 4; ++j) koff[j] = (uint32_t)(4 * j + lrow) * row_bytes + (uint32_t)(lslot ^ swz(4 * j + lrow)) * 16;
+  const int nunits = 2 * topk;
+  auto unit_rows = [&](int u) __attribute__((always_inline)) -> int {           // first key row of unit u; past the end: the last unit again
+    const int uc = min(u, nunits - 1);
+    return __builtin_amdgcn_readfirstlane((int)entries[uc >> 1]) * 64 + 32 * (uc & 1);
+  };
+  auto request = [&](int key0, int GEN) __attribute__((always_inline)) {
+    const uint32_t rb = (uint32_t)key0 * row_bytes;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const uint32_t off = koff[j & 3] + rb + (uint32_t)(j >> 2) * 16 * row_bytes;
+      lds_dma_b128(kh, off, smem_addr, GEN * TILE + j * 1024);
+      lds_dma_b128(vh, off, smem_addr, (2 + GEN) * TILE + j * 1024);
+    }
+  };
+  int rfo[DC];
+#pragma unroll
+  for (int c = 0; c < DC; ++c) rfo[c] = r * ROWB + (((2 * c + g) ^ swz(r & 15)) * 16);
+  const int tr_row = 4 * g + ((lane & 15) >> 2);
+  int tfo[2][DT];
+#pragma unroll
+  for (int h = 0; h < 2; ++h)
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      const int row = tr_row + 8 * h;
+      const int piece = 4 * dt + 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);
+      tfo[h][dt] = row * ROWB + ((piece ^ swz(row & 15)) * 16) + (lane & 1) * 8;
+    }
+#pragma unroll
+  for (int qt = 0; qt < 2; ++qt)
+#pragma unroll
+    for (int c = 0; c < DC; ++c) asm volatile("" : "+a"(qf[qt][c]), "+a"(dof[qt][c]));
+
+  // One unit = 32 keys, 48 MFMAs.  GEN = u % 2.
+  f32x16_t s0, dp0, s1, dp1;
+  auto unit = [&](int GEN, int key0, int key0_next2) __attribute__((always_inline)) {
+    asm volatile("s_waitcnt vmcnt(16)" ::: "memory");          // this unit's rows have landed (the next unit's 16 requests may be out)
+    const uint8_t* kg = smem + GEN * TILE;
+    const uint8_t* vg = smem + (2 + GEN) * TILE;
+    const int valid = L - key0;                                // key rows of this unit that exist
+    i16x8_t af[4], bf[4];                                      // row-wise fragments, three products ahead
+    auto first_products = [&](f32x16_t& s, f32x16_t& dp, const i16x8_t (&qq)[DC], const i16x8_t (&dd)[DC], auto&& beside)
+        __attribute__((always_inline)) {
+#pragma unroll
+      for (int c = 0; c < 3; ++c) {
+        af[c] = *reinterpret_cast<const i16x8_t*>(kg + rfo[c]);
+        bf[c] = *reinterpret_cast<const i16x8_t*>(vg + rfo[c]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int c = 0; c < DC; ++c) {
+        if (c + 3 < DC) {
+          af[(c + 3) & 3] = *reinterpret_cast<const i16x8_t*>(kg + rfo[c + 3]);
+          bf[(c + 3) & 3] = *reinterpret_cast<const i16x8_t*>(vg + rfo[c + 3]);
+        }
+        if (c == 0) mfma_scores_first<Tag>(s, af[0], qq[0]);
+        else mfma_scores<Tag>(s, af[c & 3], qq[c]);
+        beside(2 * c);
+        __builtin_amdgcn_sched_barrier(0);
+        if (c == 0) mfma_scores_first<Tag>(dp, bf[0], dd[0]);
+        else mfma_scores<Tag>(dp, bf[c & 3], dd[c]);
+        beside(2 * c + 1);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+    // element i of a tile: dS^T = P^T (dP^T - delta), P = exp2(S c - lse); packed in pairs into the B operand
+    auto element = [&](f32x16_t& s, f32x16_t& dp, int qt, i32x4_t (&dsw)[2], int i) __attribute__((always_inline)) {
+      float p = fast_exp2(__builtin_fmaf(s[i], c_log2e, -lse_q[qt]));
+      float ds = p * (dp[i] - delta_q[qt]);
+      asm volatile("" : "+v"(ds));
+      s[i] = ds;
+      if (i & 1) {
+        uint32_t a = E::pack2(s[i - 1], s[i]);
+        asm volatile("" : "+v"(a));
+        dsw[i >> 3][(i >> 1) & 3] = (int)a;
+      }
+    };
+    auto mask_tail = [&](f32x16_t& s) __attribute__((always_inline)) {       // key index of register i is 8 (i / 4) + i % 4 + 4 g
+      const int lim = valid - 4 * g;
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        if (8 * (i >> 2) + (i & 3) >= lim) s[i] = -INFINITY;
+    };
+    i32x4_t dsw0[2], dsw1[2];
+    first_products(s0, dp0, qf[0], dof[0], [](int) __attribute__((always_inline)) {});
+    // (the vector ALU keeps off a product's result for two products' time: the elements start in slot 2)
+    first_products(s1, dp1, qf[1], dof[1], [&](int sl) __attribute__((always_inline)) {
+      if (sl == 2 && __builtin_expect(valid < 32, 0)) mask_tail(s0);
+      if (sl >= 2) element(s0, dp0, 0, dsw0, sl - 2);
+      if (sl >= 14) element(s0, dp0, 0, dsw0, sl);             // sixteen elements in fourteen slots
+    });
+    // second products: transposed K fragments, fetched once and used by both query tiles
+    i16x8_t trk[2][DT];
+#pragma unroll
+    for (int c2 = 0; c2 < 2; ++c2)
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        const uint8_t* t0 = kg + 16 * c2 * ROWB;
+        trk[c2][dt] = concat4(lds_read_tr16(reinterpret_cast<const uint16_t*>(t0 + tfo[0][dt])),
+                              lds_read_tr16(reinterpret_cast<const uint16_t*>(t0 + tfo[1][dt])));
+      }
+    __builtin_amdgcn_sched_barrier(0);
+    if (__builtin_expect(valid < 32, 0)) {
+      asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+      mask_tail(s1);
+    }
+#pragma unroll
+    for (int sl = 0; sl < 8; ++sl) {
+      const int c2 = sl >> 2, dt = sl & 3;
+      dqacc[dt][0] = E::mfma32(trk[c2][dt], __builtin_bit_cast(i16x8_t, dsw0[c2]), dqacc[dt][0]);
+      // This unit's V has been used up, its K is in registers (or on its way there): their generation takes the unit
+      // after next, a unit and a half before it is wanted.  One request per product: requests that follow each other
+      // closely wait for the compute unit's one vector-memory path, and a single wave waits with them.  V first.
+      {
+        const uint32_t off = koff[sl & 3] + (uint32_t)key0_next2 * row_bytes + (uint32_t)(sl >> 2) * 16 * row_bytes;
+        lds_dma_b128(vh, off, smem_addr, (2 + GEN) * TILE + sl * 1024);
+      }
+      if (sl >= 2) {
+        element(s1, dp1, 1, dsw1, 2 * (sl - 2));
+        element(s1, dp1, 1, dsw1, 2 * (sl - 2) + 1);
+      }
+      if (sl >= 6) {
+        element(s1, dp1, 1, dsw1, 12 + 2 * (sl - 6));
+        element(s1, dp1, 1, dsw1, 13 + 2 * (sl - 6));
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int sl = 0; sl < 8; ++sl) {
+      const int c2 = sl >> 2, dt = sl & 3;
+      dqacc[dt][1] = E::mfma32(trk[c2][dt], __builtin_bit_cast(i16x8_t, dsw1[c2]), dqacc[dt][1]);
+      if (sl == 0) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");        // (every read of K has long returned)
+      const uint32_t off = koff[sl & 3] + (uint32_t)key0_next2 * row_bytes + (uint32_t)(sl >> 2) * 16 * row_bytes;
+      lds_dma_b128(kh, off, smem_addr, GEN * TILE + sl * 1024);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  int key_cur = 0, key_n1 = 0;
+  if (nunits > 0) {
+    key_cur = unit_rows(0);
+    key_n1 = unit_rows(1);
+    request(key_cur, 0);
+    request(key_n1, 1);
+  }
+  for (int u = 0; u < nunits; u += 2) {
+    const int key_n2 = unit_rows(u + 2), key_n3 = unit_rows(u + 3);
+    unit(0, key_cur, key_n2);
+    unit(1, key_n1, key_n3);
+    key_cur = key_n2;
+    key_n1 = key_n3;
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // (nothing of this workgroup is in flight when it ends)
+
+#pragma unroll
+  for (int qt = 0; qt < 2; ++qt) {
+    const int qrow = qrow0 + 32 * qt + r;
+    if (qrow < L) {
+      uint16_t* orow = dq + head_off + (size_t)qrow * pitch;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int i4 = 0; i4 < 4; ++i4) {
+          i32x2_t wv;
+          wv[0] = (int)E::pack2(dqacc[dt][qt][4 * i4 + 0] * qk_scale, dqacc[dt][qt][4 * i4 + 1] * qk_scale);
+          wv[1] = (int)E::pack2(dqacc[dt][qt][4 * i4 + 2] * qk_scale, dqacc[dt][qt][4 * i4 + 3] * qk_scale);
+          *reinterpret_cast<i32x2_t*>(orow + 32 * dt + 8 * i4 + 4 * g) = wv;
+        }
+    }
+  }
+}
+
 }  // namespace sla

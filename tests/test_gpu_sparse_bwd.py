@@ -37,6 +37,24 @@ def test_against_dense_oracle(dev, dtype, L, D, BLKQ, ratio):
         assert cos_sim(a, b) >= TOL_COS, name
 
 
+@pytest.mark.parametrize("H,L,dtype,ratio", [(64, 1024, torch.bfloat16, 0.25), (70, 970, torch.float16, 0.3),
+                                              (65, 1000, torch.bfloat16, 0.2)])
+def test_many_query_blocks(dev, H, L, dtype, ratio):
+    """At least 1024 query blocks of 64 rows at head dim 128: the launch size from which dQ comes from the kernel that
+    gives a whole query block to one wave (and dK / dV from its counterpart); ragged last key blocks with fewer and
+    with more than 32 rows."""
+    g = torch.Generator().manual_seed(H + L)
+    q, k, v, do = (torch.randn(1, H, L, 128, generator=g).to(dtype) for _ in range(4))
+    m, lut, T = O.get_block_map(q, k, ratio, 64, 64)
+    o_ref, lse_ref = O.sparse_attn_fwd_dense(q, k, v, m, 64, 64)
+    refs = O.sparse_attn_bwd_dense(q, k, v, o_ref, do, lse_ref, m, 64, 64)
+    o, dq, dk, dv = _grads(q, k, v, do, m, lut, T, 64, dev)
+    for name, a, b in zip(("dq", "dk", "dv"), (dq, dk, dv), refs):
+        assert torch.isfinite(a.float()).all(), name
+        assert max_abs(a, b) <= TOL_ABS, name
+        assert cos_sim(a, b) >= TOL_COS, name
+
+
 def test_full_selection_equals_sdpa_autograd(dev):
     g = torch.Generator().manual_seed(21)
     q, k, v, do = (torch.randn(2, 2, 300, 128, generator=g).to(torch.bfloat16) for _ in range(4))
