@@ -106,13 +106,29 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   bitmap[1][tid] = 0;
   if (tid == 0) repeated = 0;
   __syncthreads();
-  for (int t = tid; t < topk; t += 128) {
-    const int a = lut_at(rowA + t) & 4095, b = lut_at(rowB + t) & 4095;
-    const uint32_t seen_a = atomicOr(&bitmap[0][a >> 5], 1u << (a & 31));
-    const uint32_t seen_b = atomicOr(&bitmap[1][b >> 5], 1u << (b & 31));
-    if (((seen_a >> (a & 31)) | (seen_b >> (b & 31))) & 1u) repeated = 1;
+  // Every wave reads both rows (the first 64 entries of either stay in registers: the passes below would otherwise each
+  // wait for memory again) and marks its own row's blocks.
+  int a_first = 0, b_first = 0;
+  for (int c0 = 0; c0 < topk; c0 += 64) {
+    const int i = c0 + lane;
+    if (i < topk) {
+      const int a = lut_at(rowA + i) & 4095, b = lut_at(rowB + i) & 4095;
+      if (c0 == 0) {
+        a_first = a;
+        b_first = b;
+      }
+      const int x = w ? b : a;
+      const uint32_t seen = atomicOr(&bitmap[w][x >> 5], 1u << (x & 31));
+      if ((seen >> (x & 31)) & 1u) repeated = 1;
+    }
   }
   __syncthreads();
+  auto row_a = [&](int c0, int i) __attribute__((always_inline)) -> int {
+    return c0 == 0 ? a_first : (i < topk ? lut_at(rowA + i) & 4095 : 0);
+  };
+  auto row_b = [&](int c0, int i) __attribute__((always_inline)) -> int {
+    return c0 == 0 ? b_first : (i < topk ? lut_at(rowB + i) & 4095 : 0);
+  };
   // Step p of the pair follows entry p of the first row: a key block the second row names as well is a shared step;
   // otherwise it is an own step, on which wave 0 takes that block and wave 1 the next block (in the order of its row)
   // that only the second row names: both rows have as many of those.  Key blocks so come in the order of the look-up
@@ -127,7 +143,7 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
       int n = 0;
       for (int c0 = 0; c0 < topk; c0 += 64) {
         const int i = c0 + lane;
-        const int x = i < topk ? lut_at(rowB + i) & 4095 : 0;
+        const int x = row_b(c0, i);
         const bool sel = i < topk && !((bitmap[0][x >> 5] >> (x & 31)) & 1u);
         const unsigned long long bal = __ballot(sel);
         if (sel) own_b[n + __popcll(bal & lt_mask)] = (uint16_t)x;
@@ -138,7 +154,7 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     int n = 0;                                   // own steps before this chunk
     for (int c0 = 0; c0 < topk; c0 += 64) {
       const int i = c0 + lane;
-      const int a = i < topk ? lut_at(rowA + i) & 4095 : 0;
+      const int a = row_a(c0, i);
       const bool own = i < topk && !((bitmap[1][a >> 5] >> (a & 31)) & 1u);
       const unsigned long long bal = __ballot(own);
       if (i < topk) {
