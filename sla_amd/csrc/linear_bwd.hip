@@ -16,7 +16,7 @@
 //   reduce : fixed-order sums of the partials -> dS (16 bit, both orientations), dz, per-head dW, db;
 //            a second small kernel adds the heads
 //   kv     : per 32 keys on one wave: dc^T = dS v^T + dz, dv^T = dS^T c^T, dk = phi'(k) dc
-#include "linear_state.h"
+#include "linear_bwd_stream.h"
 
 namespace sla {
 
@@ -580,19 +580,22 @@ __global__ __launch_bounds__(64 * NW) void linear_bwd_kv_kernel(const uint16_t* 
 struct LinBwdWs {
   LinWs fwd;
   LinSplit st;   // slices of the states kernel (two workgroups per compute unit)
+  LinSplit ss;   // slices of the stream kernel (one workgroup per compute unit, 128 rows per step): never more than st's
   size_t dn, y, dden, ds_part, dw_part, dz_part, db_part, ds, dst, dz, dw_head, db_head, total;
 };
 static LinBwdWs lin_bwd_ws(int BH, int L, int D) {
   LinBwdWs w;
   w.fwd = lin_ws(BH, L, D);
   w.st = lin_split(BH, L, 512);
+  w.ss = lin_split(BH, L, 256, LBS_TR);
   const int64_t np = (int64_t)BH * w.st.nsplit;
   size_t off = w.fwd.total;
   w.dn = off;      off += align_up((int64_t)BH * L * D * 2, 256);
   w.y = off;       off += align_up((int64_t)BH * L * D * 2, 256);
   w.dden = off;    off += align_up((int64_t)BH * L * 4, 256);
   w.ds_part = off; off += align_up(np * D * D * 4, 256);
-  w.dw_part = off; off += align_up(np * D * D * 4, 256);
+  // (the stream path keeps M of every head there in both orientations: two matrices per head at least)
+  w.dw_part = off; off += align_up((np > 2 * BH ? np : 2 * (int64_t)BH) * D * D * 4, 256);
   w.dz_part = off; off += align_up(np * D * 4, 256);
   w.db_part = off; off += align_up(np * D * 4, 256);
   w.ds = off;      off += align_up((int64_t)BH * D * D * 2, 256);
@@ -611,15 +614,45 @@ static int linear_bwd_impl(const void* q, const void* k, const void* v, const fl
                            int fmap, int BH, int L, int flags, char* ws, hipStream_t st) {
   const LinBwdWs w = lin_bwd_ws(BH, L, D);
   const int accumulate = flags & SLA_BWD_ACCUMULATE;
-  if (!(flags & SLA_BWD_STATES_READY)) launch_state_build<Tag, D>(k, v, lin, weight, fmap, BH, L, ws, w.fwd, st);
+  if (!(flags & SLA_BWD_STATES_READY)) {
+    // everything the forward's state build leaves: transposed state, z, and (fold) the folded state + 16-bit weight
+    launch_state_build<Tag, D>(k, v, lin, weight, fmap, BH, L, ws, w.fwd, st, false);
+    hipLaunchKernelGGL((linear_fold_kernel<Tag>), dim3(cdiv(D * D, 256), BH), dim3(256), 0, st,
+                       (const uint16_t*)(ws + w.fwd.kvt), weight, (uint16_t*)(ws + w.fwd.kvwt), (uint16_t*)(ws + w.fwd.wt), D);
+  }
   uint16_t* kvt = (uint16_t*)(ws + w.fwd.kvt);
   uint16_t* z = (uint16_t*)(ws + w.fwd.z);
+  constexpr int NW_ROWS = 4, NW_KV = 8;   // one workgroup per compute unit either way (LDS)
+  const int tiles_kv = balanced_tiles(cdiv(L, 32 * NW_KV), BH, 1);
+  // (the stream kernel addresses a head's rows through 32-bit buffer offsets)
+  const auto fits32 = [&](const RowLayout& lay) { return ((int64_t)(L - 1) * lay.sl + D) * 2 < ((int64_t)1 << 32); };
+  bool streamed = false;
+  if constexpr (D == 128) streamed = fits32(lin) && fits32(ldo);
+  if constexpr (D == 128) if (streamed) {
+    // q and G once: dq, and the partial sums M^T, dz, db of every slice (the slices' partials and the per-head M^T
+    // take the places of the two-matrix partials of the general path: ds_part, dw_part)
+    float* m_part = (float*)(ws + w.ds_part);
+    float* mt_head = (float*)(ws + w.dw_part);
+    float* m_head = mt_head + (size_t)BH * D * D;
+#define SLA_LBS_LAUNCH(FM)                                                                                                  \
+  hipLaunchKernelGGL((linear_bwd_stream_kernel<Tag, FM>), dim3(w.ss.nsplit, BH), dim3(512), 0, st, (const uint16_t*)q,        \
+                     (const uint16_t*)d_out, (const uint16_t*)(ws + w.fwd.kvwt), z, (uint16_t*)dq, lin, ldo, m_part,          \
+                     (float*)(ws + w.dz_part), (float*)(ws + w.db_part), L, w.ss.rows_per_split, accumulate)
+    if (fmap == SLA_FMAP_ELU) SLA_LBS_LAUNCH(SLA_FMAP_ELU);
+    else if (fmap == SLA_FMAP_RELU) SLA_LBS_LAUNCH(SLA_FMAP_RELU);
+    else SLA_LBS_LAUNCH(SLA_FMAP_SOFTMAX);
+#undef SLA_LBS_LAUNCH
+    hipLaunchKernelGGL(linear_bwd_sum_kernel, dim3(cdiv(D * D, 256), BH), dim3(256), 0, st, (const float*)m_part,
+                       (const float*)(ws + w.dz_part), (const float*)(ws + w.db_part), mt_head, m_head, (float*)(ws + w.dz),
+                       (float*)(ws + w.db_head), w.ss.nsplit, D);
+    hipLaunchKernelGGL((linear_bwd_products_kernel<Tag>), dim3(D * D / 256, BH, 2), dim3(256), 0, st, (const float*)mt_head,
+                       (const float*)m_head, weight, kvt, (uint16_t*)(ws + w.ds), (uint16_t*)(ws + w.dst), (float*)(ws + w.dw_head), D);
+  }
+  if (!streamed) {
   uint16_t* dn = (uint16_t*)(ws + w.dn);
   uint16_t* y = (uint16_t*)(ws + w.y);
   float* dden = (float*)(ws + w.dden);
-  constexpr int NW_ROWS = 4, NW_KV = 8;   // one workgroup per compute unit either way (LDS)
   const int tiles_rows = balanced_tiles(cdiv(L, 32 * NW_ROWS), BH, 1);
-  const int tiles_kv = balanced_tiles(cdiv(L, 32 * NW_KV), BH, 1);
   hipLaunchKernelGGL((linear_bwd_rows_kernel<Tag, D, NW_ROWS>), dim3(cdiv(L, 32 * NW_ROWS * tiles_rows), BH), dim3(64 * NW_ROWS), 0, st, (const uint16_t*)q,
                      (const uint16_t*)d_out, kvt, (const uint16_t*)(ws + w.fwd.kvp), z, (const uint16_t*)(ws + w.fwd.wt), (uint16_t*)dq, lin, ldo, dn, y,
                      dden, L, fmap, tiles_rows, accumulate);
@@ -630,6 +663,7 @@ static int linear_bwd_impl(const void* q, const void* k, const void* v, const fl
                      (const float*)(ws + w.ds_part), (const float*)(ws + w.dw_part), (const float*)(ws + w.dz_part),
                      (const float*)(ws + w.db_part), (uint16_t*)(ws + w.ds), (uint16_t*)(ws + w.dst), (float*)(ws + w.dz),
                      (float*)(ws + w.dw_head), (float*)(ws + w.db_head), w.st.nsplit, D);
+  }
   hipLaunchKernelGGL(linear_bwd_reduce_heads_kernel, dim3(cdiv(D * D, 256)), dim3(256), 0, st,
                      (const float*)(ws + w.dw_head), (const float*)(ws + w.db_head), d_weight, d_bias, BH, D);
   if (lin.sl == D)

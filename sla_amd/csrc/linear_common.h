@@ -92,13 +92,14 @@ struct LinSplit {
 };
 // Slices of the sequence for the kernels that reduce over L: as many (head, slice) workgroups as fit the chip at
 // once (`slots` = 256 compute units x workgroups per unit), never more, so there is no second, part-filled round.
-static inline LinSplit lin_split(int BH, int L, int slots = 768) {
+// Slices are multiples of `gran` rows (the rows a kernel takes per step).
+static inline LinSplit lin_split(int BH, int L, int slots = 768, int gran = 64) {
   int nsplit = slots / BH;
-  const int max_split = cdiv(L, 64);
+  const int max_split = cdiv(L, gran);
   if (nsplit > max_split) nsplit = max_split;
   if (nsplit < 1) nsplit = 1;
   LinSplit s;
-  s.rows_per_split = cdiv(cdiv(L, nsplit), 64) * 64;
+  s.rows_per_split = cdiv(cdiv(L, nsplit), gran) * gran;
   s.nsplit = cdiv(L, s.rows_per_split);
   return s;
 }

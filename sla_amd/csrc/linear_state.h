@@ -214,6 +214,29 @@ __global__ void linear_prep_weight_kernel(const float* __restrict__ weight, uint
   wt[d * D + e] = h;
 }
 
+// ---- kernel 3 (forward, and a backward that has to rebuild the states): fold the projection into the state -------------------------------------------------
+// kvwt[bh][e][d1] = round16( sum_d2 round16(W[e][d2]) * KVT[d2][d1] ), fp32 accumulation in ascending d2.
+// (phi(Q) KV / den) W^T = (phi(Q) (KV W^T)) / den, so the output kernel needs one product per query tile.
+// grid (D*D/256, BH): thread (e, d1); the 256 threads of a workgroup share at most two rows e.
+// The workgroups of head 0 also leave the 16-bit transposed weight wt[d][e] that a backward reads (what
+// linear_prep_weight_kernel writes), which saves the forward one launch in its chain of small kernels.
+template <typename Tag>
+__global__ __launch_bounds__(256) void linear_fold_kernel(const uint16_t* __restrict__ kvt, const float* __restrict__ weight,
+                                                          uint16_t* __restrict__ kvwt, uint16_t* __restrict__ wt, int D) {
+  using E = Elem<Tag>;
+  const int bh = blockIdx.y;
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= D * D) return;
+  const int e = i / D, d1 = i % D;
+  if (bh == 0) wt[d1 * D + e] = E::from_float(weight[i]);
+  const uint16_t* s = kvt + (size_t)bh * D * D + d1;
+  const float* w = weight + (size_t)e * D;
+  float acc = 0.f;
+#pragma unroll 8
+  for (int d2 = 0; d2 < D; ++d2) acc += round16<Tag>(w[d2]) * E::to_float(s[(size_t)d2 * D]);
+  kvwt[(size_t)bh * D * D + i] = E::from_float(acc);
+}
+
 // ---- workspace layout of the state build -----------------------------------------------------
 // The finished states (kvt .. wt) come first: `states_end` bytes that a caller may copy aside after the
 // forward and put back at the start of the backward's workspace instead of having them rebuilt.

@@ -83,6 +83,40 @@ def test_linear_branch_backward_vs_autograd_oracle(dev, fmap, L, D):
         assert cos_sim(a, r) >= TOL_COS, (name, cos_sim(a, r))
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("fmap", ["elu", "relu", "softmax"])
+@pytest.mark.parametrize("B,H,L", [(1, 2, 50), (1, 3, 4099), (1, 1, 129), (2, 1, 2048)])
+def test_backward_head_dim_128_slices_and_tails(dev, dtype, fmap, B, H, L):
+    """The one-pass query-side kernel of head dim 128: a length below one 128-row step, lengths that end a slice in the
+    middle of a step, many slices per head, both 16-bit types (inputs scaled down so that float16 stays finite)."""
+    gen = torch.Generator().manual_seed(L + H)
+    q, k, v, g = (torch.randn(B, H, L, 128, generator=gen).mul(0.5).to(dtype) for _ in range(4))
+    w, b = make_proj(128)
+    refs = _oracle_linear_grads(q, k, v, w, b, g, fmap)
+    out = linear_bwd(q.to(dev), k.to(dev), v.to(dev), w.to(dev), b.to(dev), g.to(dev), fmap)
+    torch.cuda.synchronize()
+    for name, a, r in zip(("dq", "dk", "dv", "dW", "db"), out, refs):
+        a = a.cpu()
+        assert torch.isfinite(a.float()).all(), name
+        scale = max(1.0, float(r.abs().max()))
+        assert max_abs(a, r) <= TOL_ABS * scale, (name, max_abs(a, r), scale)
+        assert cos_sim(a, r) >= TOL_COS, (name, cos_sim(a, r))
+
+
+@pytest.mark.parametrize("D", [128, 64])
+def test_backward_accumulates_like_a_16_bit_addition(dev, D):
+    """accumulate_into: the gradient is rounded to 16 bit, then added to what the tensor held, rounded once more."""
+    gen = torch.Generator().manual_seed(5)
+    q, k, v, g = (torch.randn(1, 2, 700, D, generator=gen).to(torch.bfloat16).to(dev) for _ in range(4))
+    w, b = (t.to(dev) for t in make_proj(D))
+    fresh = linear_bwd(q, k, v, w, b, g, "elu")
+    base = [torch.randn_like(q) for _ in range(3)]
+    acc = linear_bwd(q, k, v, w, b, g, "elu", accumulate_into=tuple(t.clone() for t in base))
+    for a, f, b0 in zip(acc[:3], fresh[:3], base):
+        assert torch.equal(a, (b0.float() + f.float()).to(torch.bfloat16))
+    assert torch.equal(acc[3], fresh[3]) and torch.equal(acc[4], fresh[4])
+
+
 def test_split_entry_points_equal_the_fused_one(dev):
     """state half on a side stream + output half on the main one == sla_linear_fwd, bit for bit."""
     g = torch.Generator().manual_seed(7)
