@@ -176,6 +176,25 @@ int sla_sparse_attn_linear_fwd_strided(const void* q, const void* k, const void*
                                        const int64_t* out_strides, float* lse, int dtype, int fmap, int B, int H, int L,
                                        int D, int BLKQ, int BLKK, int topk, float qk_scale, void* stream);
 
+/* Backward of the whole module in one call: the kernels of sla_sparse_attn_bwd(_strided) followed by those of
+ * sla_linear_bwd(_strided) with SLA_BWD_ACCUMULATE (the linear branch adds into dq, dk, dv), results equal to those two
+ * calls bit for bit.  The only flag is SLA_BWD_STATES_READY.  qkv_strides / do_strides: both NULL for contiguous
+ * (B, H, L, D) tensors, else as in the strided calls.  o_s is the attention output the forward saved.  The two workspaces
+ * are those of the two calls (SLA_WS_SPARSE_BWD, SLA_WS_LINEAR_BWD).
+ * side_stream (may be NULL or equal to stream: then everything runs on `stream`) takes the short kernels - the
+ * per-key-block lists of the map, and the per-head reductions and small products of the linear branch - so that they run
+ * beside the long dQ and dK/dV kernels instead of between them; `stream` waits for all of it before the call's last
+ * kernel, so later work needs ordering against `stream` only.  The streams must belong to the current device and have the
+ * same (default) priority.
+ * Replaces autograd through SparseLinearAttention.forward, sparse_linear_attention/core.py:88-100 with
+ * kernel.py:277-320. */
+int sla_module_bwd(const void* q, const void* k, const void* v, const int64_t* qkv_strides, const void* o_s,
+                   const void* d_out, const int64_t* do_strides, const float* lse, const int8_t* sparse_map, const void* lut,
+                   int lut_elem_bytes, const float* weight, const float* bias, void* dq, void* dk, void* dv, float* d_weight,
+                   float* d_bias, int dtype, int fmap, int B, int H, int L, int D, int BLKQ, int BLKK, int topk,
+                   float qk_scale, int flags, void* sparse_workspace, int64_t sparse_workspace_bytes, void* linear_workspace,
+                   int64_t linear_workspace_bytes, void* stream, void* side_stream);
+
 /* Linear branch in "complement" mode (opt-in): query block i attends linearly only to the key
  * blocks (of 64 rows) that its look-up row did NOT select; projection, bias and residual as in
  * sla_linear_fwd.  out = residual + proj(o_l).  lut as produced by sla_block_map_fwd; BLKK must be 64.

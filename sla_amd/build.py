@@ -17,7 +17,7 @@ LIBDIR = os.path.join(HERE, "lib")
 LIBPATH = os.path.join(LIBDIR, "libsla_hip.so")
 
 SOURCES = ["capi.hip", "block_map.hip", "sparse_fwd.hip", "linear.hip", "linear_bwd.hip", "sparse_bwd.hip", "sage.hip",
-           "linear_complement.hip"]
+           "linear_complement.hip", "module_bwd.hip"]
 
 COMMON_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",

@@ -16,6 +16,7 @@
 //   reduce : fixed-order sums of the partials -> dS (16 bit, both orientations), dz, per-head dW, db;
 //            a second small kernel adds the heads
 //   kv     : per 32 keys on one wave: dc^T = dS v^T + dz, dv^T = dS^T c^T, dk = phi'(k) dc
+#include "bwd_steps.h"
 #include "linear_bwd_stream.h"
 
 namespace sla {
@@ -611,10 +612,10 @@ int64_t linear_bwd_workspace_bytes(int BH, int L, int D) { return (int64_t)lin_b
 template <typename Tag, int D>
 static int linear_bwd_impl(const void* q, const void* k, const void* v, const float* weight, const void* d_out, void* dq,
                            void* dk, void* dv, const RowLayout& lin, const RowLayout& ldo, float* d_weight, float* d_bias,
-                           int fmap, int BH, int L, int flags, char* ws, hipStream_t st) {
+                           int fmap, int BH, int L, int flags, char* ws, hipStream_t st, int steps) {
   const LinBwdWs w = lin_bwd_ws(BH, L, D);
   const int accumulate = flags & SLA_BWD_ACCUMULATE;
-  if (!(flags & SLA_BWD_STATES_READY)) {
+  if ((steps & LB_STATES) && !(flags & SLA_BWD_STATES_READY)) {
     // everything the forward's state build leaves: transposed state, z, and (fold) the folded state + 16-bit weight
     launch_state_build<Tag, D>(k, v, lin, weight, fmap, BH, L, ws, w.fwd, st, false);
     hipLaunchKernelGGL((linear_fold_kernel<Tag>), dim3(cdiv(D * D, 256), BH), dim3(256), 0, st,
@@ -634,6 +635,7 @@ static int linear_bwd_impl(const void* q, const void* k, const void* v, const fl
     float* m_part = (float*)(ws + w.ds_part);
     float* mt_head = (float*)(ws + w.dw_part);
     float* m_head = mt_head + (size_t)BH * D * D;
+    if (steps & LB_QUERY) {
 #define SLA_LBS_LAUNCH(FM)                                                                                                  \
   hipLaunchKernelGGL((linear_bwd_stream_kernel<Tag, FM>), dim3(w.ss.nsplit, BH), dim3(512), 0, st, (const uint16_t*)q,        \
                      (const uint16_t*)d_out, (const uint16_t*)(ws + w.fwd.kvwt), z, (uint16_t*)dq, lin, ldo, m_part,          \
@@ -642,30 +644,38 @@ static int linear_bwd_impl(const void* q, const void* k, const void* v, const fl
     else if (fmap == SLA_FMAP_RELU) SLA_LBS_LAUNCH(SLA_FMAP_RELU);
     else SLA_LBS_LAUNCH(SLA_FMAP_SOFTMAX);
 #undef SLA_LBS_LAUNCH
+    }
+    if (steps & LB_REDUCE) {
     hipLaunchKernelGGL(linear_bwd_sum_kernel, dim3(cdiv(D * D, 256), BH), dim3(256), 0, st, (const float*)m_part,
                        (const float*)(ws + w.dz_part), (const float*)(ws + w.db_part), mt_head, m_head, (float*)(ws + w.dz),
                        (float*)(ws + w.db_head), w.ss.nsplit, D);
     hipLaunchKernelGGL((linear_bwd_products_kernel<Tag>), dim3(D * D / 256, BH, 2), dim3(256), 0, st, (const float*)mt_head,
                        (const float*)m_head, weight, kvt, (uint16_t*)(ws + w.ds), (uint16_t*)(ws + w.dst), (float*)(ws + w.dw_head), D);
+    }
   }
   if (!streamed) {
   uint16_t* dn = (uint16_t*)(ws + w.dn);
   uint16_t* y = (uint16_t*)(ws + w.y);
   float* dden = (float*)(ws + w.dden);
   const int tiles_rows = balanced_tiles(cdiv(L, 32 * NW_ROWS), BH, 1);
+  if (steps & LB_QUERY) {
   hipLaunchKernelGGL((linear_bwd_rows_kernel<Tag, D, NW_ROWS>), dim3(cdiv(L, 32 * NW_ROWS * tiles_rows), BH), dim3(64 * NW_ROWS), 0, st, (const uint16_t*)q,
                      (const uint16_t*)d_out, kvt, (const uint16_t*)(ws + w.fwd.kvp), z, (const uint16_t*)(ws + w.fwd.wt), (uint16_t*)dq, lin, ldo, dn, y,
                      dden, L, fmap, tiles_rows, accumulate);
   hipLaunchKernelGGL((linear_bwd_states_kernel<Tag, D>), dim3(w.st.nsplit, BH), dim3(256), 0, st, (const uint16_t*)q, dn,
                      (const uint16_t*)d_out, y, dden, lin, ldo, (float*)(ws + w.ds_part), (float*)(ws + w.dw_part),
                      (float*)(ws + w.dz_part), (float*)(ws + w.db_part), L, w.st.rows_per_split, fmap);
+  }
+  if (steps & LB_REDUCE)
   hipLaunchKernelGGL((linear_bwd_reduce_kernel<Tag>), dim3(cdiv(D * D, 256), BH), dim3(256), 0, st,
                      (const float*)(ws + w.ds_part), (const float*)(ws + w.dw_part), (const float*)(ws + w.dz_part),
                      (const float*)(ws + w.db_part), (uint16_t*)(ws + w.ds), (uint16_t*)(ws + w.dst), (float*)(ws + w.dz),
                      (float*)(ws + w.dw_head), (float*)(ws + w.db_head), w.st.nsplit, D);
   }
-  hipLaunchKernelGGL(linear_bwd_reduce_heads_kernel, dim3(cdiv(D * D, 256)), dim3(256), 0, st,
-                     (const float*)(ws + w.dw_head), (const float*)(ws + w.db_head), d_weight, d_bias, BH, D);
+  if (steps & LB_REDUCE)
+    hipLaunchKernelGGL(linear_bwd_reduce_heads_kernel, dim3(cdiv(D * D, 256)), dim3(256), 0, st,
+                       (const float*)(ws + w.dw_head), (const float*)(ws + w.db_head), d_weight, d_bias, BH, D);
+  if (!(steps & LB_KEYS)) return check_launch("linear_bwd");
   if (lin.sl == D)
     hipLaunchKernelGGL((linear_bwd_kv_kernel<Tag, D, NW_KV, true>), dim3(cdiv(L, 32 * NW_KV * tiles_kv), BH), dim3(64 * NW_KV),
                        0, st, (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)(ws + w.ds),
@@ -731,14 +741,10 @@ void launch_weight_grads(int dtype, int D, const void* q, const void* dn, const 
   }
 }
 
-}  // namespace sla
-
-using namespace sla;
-
-static int linear_bwd_entry(const void* q, const void* k, const void* v, const int64_t* qkv_strides, const float* weight,
-                            const float* bias, const void* d_out, const int64_t* do_strides, void* dq, void* dk, void* dv,
-                            float* d_weight, float* d_bias, int dtype, int fmap, int B, int H, int L, int D, int flags,
-                            void* workspace, int64_t workspace_bytes, void* stream) {
+int linear_bwd_steps(const void* q, const void* k, const void* v, const int64_t* qkv_strides, const float* weight,
+                     const float* bias, const void* d_out, const int64_t* do_strides, void* dq, void* dk, void* dv,
+                     float* d_weight, float* d_bias, int dtype, int fmap, int B, int H, int L, int D, int flags,
+                     void* workspace, int64_t workspace_bytes, void* stream, int steps) {
   int rc = validate_linear(dtype, fmap, B, H, L, D);
   if (rc) return rc;
   SLA_REQUIRE((flags & ~(SLA_BWD_ACCUMULATE | SLA_BWD_STATES_READY)) == 0, SLA_ERR_BAD_ARG, "unknown flag bits in %d", flags);
@@ -760,7 +766,8 @@ static int linear_bwd_entry(const void* q, const void* k, const void* v, const i
   hipStream_t st = (hipStream_t)stream;
   char* ws = (char*)workspace;
 #define SLA_LINB_CASE(TAG, DD) \
-  return linear_bwd_impl<TAG, DD>(q, k, v, weight, d_out, dq, dk, dv, lin, ldo, d_weight, d_bias, fmap, BH, L, flags, ws, st)
+  return linear_bwd_impl<TAG, DD>(q, k, v, weight, d_out, dq, dk, dv, lin, ldo, d_weight, d_bias, fmap, BH, L, flags, ws, st, \
+                                  steps)
   if (dtype == SLA_BF16) {
     if (D == 128) SLA_LINB_CASE(bf16_tag, 128);
     SLA_LINB_CASE(bf16_tag, 64);
@@ -770,12 +777,16 @@ static int linear_bwd_entry(const void* q, const void* k, const void* v, const i
 #undef SLA_LINB_CASE
 }
 
+}  // namespace sla
+
+using namespace sla;
+
 extern "C" int sla_linear_bwd(const void* q, const void* k, const void* v, const float* weight, const float* bias,
                               const void* d_out, void* dq, void* dk, void* dv, float* d_weight, float* d_bias, int dtype,
                               int fmap, int B, int H, int L, int D, int flags, void* workspace,
                               int64_t workspace_bytes, void* stream) {
-  return linear_bwd_entry(q, k, v, nullptr, weight, bias, d_out, nullptr, dq, dk, dv, d_weight, d_bias, dtype, fmap, B, H, L,
-                          D, flags, workspace, workspace_bytes, stream);
+  return linear_bwd_steps(q, k, v, nullptr, weight, bias, d_out, nullptr, dq, dk, dv, d_weight, d_bias, dtype, fmap, B, H, L,
+                          D, flags, workspace, workspace_bytes, stream, LB_ALL);
 }
 
 extern "C" int sla_linear_bwd_strided(const void* q, const void* k, const void* v, const int64_t* qkv_strides,
@@ -784,6 +795,6 @@ extern "C" int sla_linear_bwd_strided(const void* q, const void* k, const void* 
                                       int B, int H, int L, int D, int flags, void* workspace, int64_t workspace_bytes,
                                       void* stream) {
   SLA_REQUIRE(qkv_strides && do_strides, SLA_ERR_BAD_ARG, "null strides");
-  return linear_bwd_entry(q, k, v, qkv_strides, weight, bias, d_out, do_strides, dq, dk, dv, d_weight, d_bias, dtype, fmap, B,
-                          H, L, D, flags, workspace, workspace_bytes, stream);
+  return linear_bwd_steps(q, k, v, qkv_strides, weight, bias, d_out, do_strides, dq, dk, dv, d_weight, d_bias, dtype, fmap, B,
+                          H, L, D, flags, workspace, workspace_bytes, stream, LB_ALL);
 }

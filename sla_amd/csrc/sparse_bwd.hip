@@ -19,7 +19,7 @@
 //                in registers as B operands; P and dS leave the accumulators in B-operand layout
 //                for dV^T += dO^T P and dK^T += Q^T dS (Q^T, dO^T via transposing LDS reads).
 //                Four waves: two key halves x two halves of the head dimension.
-#include "common.h"
+#include "bwd_steps.h"
 
 namespace sla {
 
@@ -709,7 +709,7 @@ template <typename Tag, int D, int BLKQ>
 static int bwd_impl(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
                     const int8_t* sparse_map, const void* lut, int lut64, void* dq, void* dk, void* dv,
                     const RowLayout& lin, const RowLayout& ldo, int BH, int L, int topk, float qk_scale, char* ws,
-                    hipStream_t st) {
+                    hipStream_t st, int steps) {
   const BwdWs w = bwd_ws(BH, L, D, BLKQ, 64, topk);
   const int Mblk = cdiv(L, BLKQ), Nblk = cdiv(L, 64);
   float* delta = (float*)(ws + w.delta);
@@ -717,16 +717,18 @@ static int bwd_impl(const void* q, const void* k, const void* v, const void* o, 
   int* list = (int*)(ws + w.list);
   const size_t rows = (size_t)BH * L;
   constexpr int RPB = 256 / (D / 8);
-  hipLaunchKernelGGL((bwd_delta_kernel<Tag, D>), dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, st,
-                     (const uint16_t*)o, (const uint16_t*)d_o, ldo, delta, rows, L);
-  launch_col_lists(sparse_map, list, count, BH, Mblk, Nblk, st);
+  if (steps & SB_DQ)
+    hipLaunchKernelGGL((bwd_delta_kernel<Tag, D>), dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, st,
+                       (const uint16_t*)o, (const uint16_t*)d_o, ldo, delta, rows, L);
+  if (steps & SB_LISTS) launch_col_lists(sparse_map, list, count, BH, Mblk, Nblk, st);
   int* nseg = (int*)(ws + w.nseg);
   int* slot0 = (int*)(ws + w.slot0);
   i32x4_t* items = (i32x4_t*)(ws + w.items);
   int* totals = (int*)(ws + w.totals);
   float* part = (float*)(ws + w.part);
-  hipLaunchKernelGGL(bwd_segments_kernel, dim3(1), dim3(1024), 0, st, count, nseg, slot0, items, totals, BH * Nblk, Nblk, w.seg,
-                     (int)w.max_items, (int)w.max_slots);
+  if (steps & SB_LISTS)
+    hipLaunchKernelGGL(bwd_segments_kernel, dim3(1), dim3(1024), 0, st, count, nseg, slot0, items, totals, BH * Nblk, Nblk,
+                       w.seg, (int)w.max_items, (int)w.max_slots);
   const int total_q = BH * Mblk;
   const bool contig = lin.sl == D && ldo.sl == D;
   // head dim 128 with 64-row query blocks has a dK/dV kernel of its own (32-bit byte offsets inside a head)
@@ -734,7 +736,8 @@ static int bwd_impl(const void* q, const void* k, const void* v, const void* o, 
                            (uint64_t)ldo.sl * 2u * (uint64_t)L < (1ull << 31);
   const bool stream_dq = stream_dkdv && topk <= DQ_STREAM_MAX_T && total_q >= 1024;      // (enough query blocks for a wave on every SIMD)
 #define SLA_BWD_LAUNCH(CONTIG)                                                                                              \
-  if (stream_dq)                                                                                                            \
+  if (!(steps & SB_DQ)) {                                                                                                   \
+  } else if (stream_dq)                                                                                                     \
     hipLaunchKernelGGL((bwd_dq_stream_kernel<Tag>), dim3(xcd_grid(total_q)), dim3(64), 0, st, (const uint16_t*)q,           \
                        (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse, delta, lut, lut64, (uint16_t*)dq, \
                        lin, ldo, L, Mblk, topk, qk_scale, total_q);                                                        \
@@ -742,7 +745,8 @@ static int bwd_impl(const void* q, const void* k, const void* v, const void* o, 
     hipLaunchKernelGGL((bwd_dq_kernel<Tag, D, BLKQ, CONTIG>), dim3(xcd_grid(total_q)), dim3(BLKQ * 2), 0, st,               \
                        (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse, delta, lut,   \
                        lut64, (uint16_t*)dq, lin, ldo, L, Mblk, topk, qk_scale, total_q);                                  \
-  if (stream_dkdv)                                                                                                          \
+  if (!(steps & SB_DKDV)) {                                                                                                 \
+  } else if (stream_dkdv)                                                                                                   \
     hipLaunchKernelGGL((bwd_dkdv_stream_kernel<Tag>), dim3(xcd_grid(w.max_items)), dim3(128), 0, st, (const uint16_t*)q,    \
                        (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse, delta, list, count, items,       \
                        totals, part, w.seg, (uint16_t*)dk, (uint16_t*)dv, lin, ldo, L, Mblk, Nblk, qk_scale);             \
@@ -756,20 +760,16 @@ static int bwd_impl(const void* q, const void* k, const void* v, const void* o, 
     SLA_BWD_LAUNCH(false)
   }
 #undef SLA_BWD_LAUNCH
-  hipLaunchKernelGGL((bwd_dkdv_reduce_kernel<Tag, D>), dim3(Nblk, BH), dim3(256), 0, st, nseg, slot0, part, (uint16_t*)dk,
-                     (uint16_t*)dv, lin, L, Nblk, (int)w.max_slots);
+  if (steps & SB_DKDV)
+    hipLaunchKernelGGL((bwd_dkdv_reduce_kernel<Tag, D>), dim3(Nblk, BH), dim3(256), 0, st, nseg, slot0, part, (uint16_t*)dk,
+                       (uint16_t*)dv, lin, L, Nblk, (int)w.max_slots);
   return check_launch("sparse_attn_bwd");
 }
 
-}  // namespace sla
-
-using namespace sla;
-
-static int attn_bwd_entry(const void* q, const void* k, const void* v, const int64_t* qkv_strides, const void* o,
-                          const void* d_o, const int64_t* do_strides, const float* lse, const int8_t* sparse_map,
-                          const void* lut, int lut_elem_bytes, void* dq, void* dk, void* dv, int dtype, int B, int H, int L,
-                          int D, int BLKQ, int BLKK, int topk, float qk_scale, void* workspace, int64_t workspace_bytes,
-                          void* stream) {
+int attn_bwd_steps(const void* q, const void* k, const void* v, const int64_t* qkv_strides, const void* o, const void* d_o,
+                   const int64_t* do_strides, const float* lse, const int8_t* sparse_map, const void* lut, int lut_elem_bytes,
+                   void* dq, void* dk, void* dv, int dtype, int B, int H, int L, int D, int BLKQ, int BLKK, int topk,
+                   float qk_scale, void* workspace, int64_t workspace_bytes, void* stream, int steps) {
   int rc = validate_attn_shape(dtype, B, H, L, D, BLKQ, BLKK, topk, lut_elem_bytes);
   if (rc) return rc;
   SLA_REQUIRE(q && k && v && o && d_o && lse && sparse_map && dq && dk && dv && workspace && (lut || topk == 0),
@@ -794,7 +794,7 @@ static int attn_bwd_entry(const void* q, const void* k, const void* v, const int
 #define SLA_BWD_CASE(TAG, DD, BQ)                                                                                          \
   if (D == DD && BLKQ == BQ)                                                                                               \
   return bwd_impl<TAG, DD, BQ>(q, k, v, o, d_o, lse, sparse_map, lut, lut64, dq, dk, dv, lin, ldo, BH, L, topk, qk_scale, \
-                               ws, st)
+                               ws, st, steps)
   if (dtype == SLA_BF16) {
     SLA_BWD_CASE(bf16_tag, 128, 64);
     SLA_BWD_CASE(bf16_tag, 128, 128);
@@ -811,12 +811,16 @@ static int attn_bwd_entry(const void* q, const void* k, const void* v, const int
   return SLA_ERR_UNSUPPORTED;
 }
 
+}  // namespace sla
+
+using namespace sla;
+
 extern "C" int sla_sparse_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o,
                                    const float* lse, const int8_t* sparse_map, const void* lut, int lut_elem_bytes,
                                    void* dq, void* dk, void* dv, int dtype, int B, int H, int L, int D, int BLKQ, int BLKK,
                                    int topk, float qk_scale, void* workspace, int64_t workspace_bytes, void* stream) {
-  return attn_bwd_entry(q, k, v, nullptr, o, d_o, nullptr, lse, sparse_map, lut, lut_elem_bytes, dq, dk, dv, dtype, B, H, L,
-                        D, BLKQ, BLKK, topk, qk_scale, workspace, workspace_bytes, stream);
+  return attn_bwd_steps(q, k, v, nullptr, o, d_o, nullptr, lse, sparse_map, lut, lut_elem_bytes, dq, dk, dv, dtype, B, H, L,
+                        D, BLKQ, BLKK, topk, qk_scale, workspace, workspace_bytes, stream, SB_ALL);
 }
 
 extern "C" int sla_sparse_attn_bwd_strided(const void* q, const void* k, const void* v, const int64_t* qkv_strides,
@@ -825,6 +829,6 @@ extern "C" int sla_sparse_attn_bwd_strided(const void* q, const void* k, const v
                                            void* dv, int dtype, int B, int H, int L, int D, int BLKQ, int BLKK, int topk,
                                            float qk_scale, void* workspace, int64_t workspace_bytes, void* stream) {
   SLA_REQUIRE(qkv_strides && do_strides, SLA_ERR_BAD_ARG, "null strides");
-  return attn_bwd_entry(q, k, v, qkv_strides, o, d_o, do_strides, lse, sparse_map, lut, lut_elem_bytes, dq, dk, dv, dtype, B,
-                        H, L, D, BLKQ, BLKK, topk, qk_scale, workspace, workspace_bytes, stream);
+  return attn_bwd_steps(q, k, v, qkv_strides, o, d_o, do_strides, lse, sparse_map, lut, lut_elem_bytes, dq, dk, dv, dtype, B,
+                        H, L, D, BLKQ, BLKK, topk, qk_scale, workspace, workspace_bytes, stream, SB_ALL);
 }

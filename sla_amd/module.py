@@ -7,10 +7,59 @@ import torch.nn as nn
 
 from . import _lib
 from .block_map import get_block_map
-from .linear import linear_bwd, linear_complement_bwd, linear_complement_fwd, linear_state_fwd, saved_states
+from .linear import linear_complement_bwd, linear_complement_fwd, linear_state_fwd, saved_states
 from .sparse_attn import sparse_attn_bwd, sparse_attn_fwd, sparse_attn_linear_fwd
 
 FEATURE_MAPS = ("elu", "relu", "softmax")
+
+
+def module_bwd(q, k, v, o_s, d_out, lse, sparse_map, lut, topk, BLKQ, BLKK, qk_scale, weight, bias, fmap, states=None,
+               grads=None, side_stream=None):
+    """Backward of the whole operator in one library call (``sla_module_bwd``): the kernels of
+    :func:`sparse_attn_bwd` and of :func:`linear_bwd` accumulating into the same gradients, bit for bit, with the
+    short kernels on ``side_stream`` beside the long ones when one is given.  Returns ``(dq, dk, dv, d_weight, d_bias)``.
+
+    q, k, v (and ``grads=(dq, dk, dv)`` when given) may be row-contiguous views sharing their strides, ``d_out`` a
+    row-contiguous view of its own; ``o_s`` and ``lse`` are contiguous.  ``states`` as in :func:`linear_bwd`."""
+    _lib.require_gpu(q, k, v, o_s, d_out, lse, sparse_map, lut, weight, bias)
+    B, H, L, D = q.shape
+    dev = q.device
+    dt = _lib.dtype_code(q.dtype)
+    dq, dk, dv = (torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)) if grads is None else grads
+    assert o_s.is_contiguous() and lse.is_contiguous() and sparse_map.is_contiguous() and lut.is_contiguous()
+    ws_s = _lib.workspace(_lib.WS_SPARSE_BWD, dt, B, H, L, D, BLKQ, BLKK, topk, dev)
+    ws_l = _lib.workspace(_lib.WS_LINEAR_BWD, dt, B, H, L, D, 64, 64, 0, dev)
+    flags = 0
+    if states is not None:
+        ws_l[:states.numel()].copy_(states)
+        flags |= _lib.BWD_STATES_READY
+    dw = torch.empty((D, D), dtype=torch.float32, device=dev)
+    db = torch.empty((D,), dtype=torch.float32, device=dev)
+    if all(t.is_contiguous() for t in (q, k, v, d_out, dq, dk, dv)):
+        s_qkv = s_do = None
+    else:
+        assert _lib.row_strided(q, k, v, dq, dk, dv) and _lib.row_strided(d_out), "tensors must be row-contiguous views"
+        s_qkv, s_do = _lib.strides_arg(q), _lib.strides_arg(d_out)
+    side = 0 if side_stream is None else side_stream.cuda_stream
+    rc = _lib.load().sla_module_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), s_qkv, o_s.data_ptr(), d_out.data_ptr(), s_do,
+                                    lse.data_ptr(), sparse_map.data_ptr(), lut.data_ptr(), lut.element_size(),
+                                    weight.data_ptr(), bias.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
+                                    dw.data_ptr(), db.data_ptr(), dt, _lib.FMAP[fmap], B, H, L, D, BLKQ, BLKK, topk,
+                                    float(qk_scale), flags, ws_s.data_ptr(), ws_s.numel(), ws_l.data_ptr(), ws_l.numel(),
+                                    _lib.stream_ptr(dev), side)
+    _lib.check(rc)
+    return dq, dk, dv, dw, db
+
+
+def _backward_side_stream(dev):
+    """The stream the short kernels of the backward go to: the one the forward's state build uses (default priority,
+    one per device); none while a graph is being captured (the work then stays on the capturing stream)."""
+    if torch.cuda.is_current_stream_capturing():
+        return None
+    side = _StateBuild._side.get(dev.index)
+    if side is None:
+        side = _StateBuild._side[dev.index] = torch.cuda.Stream(device=dev)
+    return side
 
 
 class _sla_core(torch.autograd.Function):
@@ -46,8 +95,8 @@ class _sla_core(torch.autograd.Function):
         q, k, v, weight, bias, sparse_map, lut, lse, o_s, states = ctx.saved_tensors
         topk, BLKQ, BLKK, fmap, qk_scale = ctx.cfg
         d_out = d_out.contiguous()
-        dq, dk, dv = sparse_attn_bwd(q, k, v, o_s, d_out, lse, sparse_map, lut, topk, BLKQ, BLKK, qk_scale)
-        _, _, _, dw, db = linear_bwd(q, k, v, weight, bias, d_out, fmap, accumulate_into=(dq, dk, dv), states=states)
+        dq, dk, dv, dw, db = module_bwd(q, k, v, o_s, d_out, lse, sparse_map, lut, topk, BLKQ, BLKK, qk_scale, weight, bias,
+                                        fmap, states=states, side_stream=_backward_side_stream(q.device))
         return dq, dk, dv, dw, db, None, None, None, None, None, None, None, None
 
 
@@ -117,8 +166,8 @@ class _sla_packed(torch.autograd.Function):
             d_out = d_out.contiguous()
         d_qkv = torch.empty_like(qkv)
         grads = tuple(d_qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
-        sparse_attn_bwd(q, k, v, o_s, d_out, lse, sparse_map, lut, topk, BLKQ, BLKK, qk_scale, grads=grads)
-        _, _, _, dw, db = linear_bwd(q, k, v, weight, bias, d_out, fmap, accumulate_into=grads, states=states)
+        _, _, _, dw, db = module_bwd(q, k, v, o_s, d_out, lse, sparse_map, lut, topk, BLKQ, BLKK, qk_scale, weight, bias,
+                                     fmap, states=states, grads=grads, side_stream=_backward_side_stream(qkv.device))
         return d_qkv, dw, db, None, None, None, None
 
 

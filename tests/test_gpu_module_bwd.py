@@ -118,3 +118,48 @@ def test_training_step_in_a_hip_graph(dev):
         with torch.no_grad():
             mod(qg, kg, vg)                   # eager work between the replays
         torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("layout", ["contiguous", "packed"])
+@pytest.mark.parametrize("with_states", [False, True])
+@pytest.mark.parametrize("dtype,L,D,BLKQ", [(torch.bfloat16, 2100, 128, 64), (torch.float16, 1000, 64, 128)])
+def test_one_call_backward_equals_the_two_calls(dev, layout, with_states, dtype, L, D, BLKQ):
+    """sla_module_bwd, on one stream and with the short kernels on a second one, against sla_sparse_attn_bwd followed
+    by the accumulating sla_linear_bwd: the same bits.  Ran twice with the side stream (the events are reused)."""
+    from sla_amd import get_block_map
+    from sla_amd.linear import linear_bwd, linear_state_fwd, saved_states
+    from sla_amd.module import module_bwd
+    from sla_amd.sparse_attn import sparse_attn_bwd, sparse_attn_linear_fwd
+
+    B, H, topk_ratio, fmap = 1, 3, 0.2, "elu"
+    gen = torch.Generator().manual_seed(L)
+    if layout == "packed":
+        qkv = torch.randn(B, L, 3, H, D, generator=gen).to(dtype).to(dev)
+        q, k, v = (qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+        d_out = torch.randn(B, L, H, D, generator=gen).to(dtype).to(dev).permute(0, 2, 1, 3)
+    else:
+        q, k, v, d_out = (torch.randn(B, H, L, D, generator=gen).to(dtype).to(dev) for _ in range(4))
+    w, b = (t.to(dev) for t in make_proj(D))
+    sparse_map, lut, topk = get_block_map(q, k, topk_ratio=topk_ratio, BLKQ=BLKQ, BLKK=64)
+    state_ws = linear_state_fwd(k, v, w, fmap)
+    _, o_s, lse = sparse_attn_linear_fwd(q, k, v, lut, topk, BLKQ, 64, D ** -0.5, state_ws, b, fmap, want_o_s=True)
+    states = saved_states(state_ws, q) if with_states else None
+
+    def new_grads():
+        if layout == "packed":
+            g = torch.full((B, L, 3, H, D), float("nan"), dtype=dtype, device=dev)
+            return g, tuple(g[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+        g = tuple(torch.full((B, H, L, D), float("nan"), dtype=dtype, device=dev) for _ in range(3))
+        return g, g
+
+    _, ref = new_grads()
+    sparse_attn_bwd(q, k, v, o_s, d_out, lse, sparse_map, lut, topk, BLKQ, 64, D ** -0.5, grads=ref)
+    _, _, _, dw_ref, db_ref = linear_bwd(q, k, v, w, b, d_out, fmap, accumulate_into=ref, states=states)
+    side = torch.cuda.Stream(device=dev)
+    for side_stream in (None, side, side):
+        _, grads = new_grads()
+        out = module_bwd(q, k, v, o_s, d_out, lse, sparse_map, lut, topk, BLKQ, 64, D ** -0.5, w, b, fmap, states=states,
+                         grads=grads, side_stream=side_stream)
+        torch.cuda.synchronize()
+        for name, a, r in zip(("dq", "dk", "dv", "dW", "db"), out, (*ref, dw_ref, db_ref)):
+            assert torch.equal(a, r), (name, side_stream is not None)
