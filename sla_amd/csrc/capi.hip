@@ -23,6 +23,8 @@ int check_launch(const char* what) {
 
 int make_layout(const int64_t* strides, int B, int H, int L, int D, int elem_bytes, RowLayout* out) {
   if (!strides) {
+    SLA_REQUIRE(((int64_t)(L + 255) * D + D) * elem_bytes < (1ll << 32), SLA_ERR_UNSUPPORTED,
+                "one head spans 4 GiB or more (L=%d D=%d)", L, D);
     *out = contiguous_layout(H, L, D);
     return SLA_OK;
   }
@@ -38,7 +40,9 @@ int make_layout(const int64_t* strides, int B, int H, int L, int D, int elem_byt
   SLA_REQUIRE(H == 1 || sh >= (int64_t)(L - 1) * sl + D || (sh >= D && sl >= (int64_t)(H - 1) * sh + D), SLA_ERR_BAD_ARG,
               "strides (%lld, %lld, %lld): rows of different heads overlap (H=%d L=%d D=%d)", (long long)sb, (long long)sh,
               (long long)sl, H, L, D);
-  SLA_REQUIRE(((int64_t)(L - 1) * sl + D) * elem_bytes < (1ll << 32) - 65536, SLA_ERR_UNSUPPORTED,
+  // (32-bit byte offsets inside a head; kernels that take whole tiles of rows form offsets of up to 255 rows past L,
+  //  which must still lie beyond the head's range instead of wrapping around)
+  SLA_REQUIRE(((int64_t)(L + 255) * sl + D) * elem_bytes < (1ll << 32), SLA_ERR_UNSUPPORTED,
               "one head spans 4 GiB or more with row stride %lld", (long long)sl);
   *out = RowLayout{sb, sh, sl, H};
   return SLA_OK;

@@ -45,11 +45,18 @@ static __device__ __forceinline__ void phi_row_pair(int fmap, float (&f)[DC][8],
     for (int c = 0; c < DC; ++c)
 #pragma unroll
       for (int j = 0; j < 8; ++j) f[c][j] = round16<Tag>(f[c][j] * inv);
+  } else if (fmap == SLA_FMAP_RELU) {
+    // (the choice of the map stays outside the loops over the elements: inside, every element's map would sit
+    //  behind a branch of its own)
+#pragma unroll
+    for (int c = 0; c < DC; ++c)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) f[c][j] = fmap_pointwise<Tag>(SLA_FMAP_RELU, f[c][j]);
   } else {
 #pragma unroll
     for (int c = 0; c < DC; ++c)
 #pragma unroll
-      for (int j = 0; j < 8; ++j) f[c][j] = fmap_pointwise<Tag>(fmap, f[c][j]);
+      for (int j = 0; j < 8; ++j) f[c][j] = fmap_pointwise<Tag>(SLA_FMAP_ELU, f[c][j]);
   }
 }
 

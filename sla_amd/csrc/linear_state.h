@@ -100,9 +100,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
         const float inv = 1.0f / sum;
 #pragma unroll
         for (int e = 0; e < 8; ++e) f[e] = round16<Tag>(f[e] * inv);
+      } else if (fmap == SLA_FMAP_RELU) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) f[e] = fmap_pointwise<Tag>(SLA_FMAP_RELU, f[e]);
       } else {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) f[e] = fmap_pointwise<Tag>(fmap, f[e]);
+        for (int e = 0; e < 8; ++e) f[e] = fmap_pointwise<Tag>(SLA_FMAP_ELU, f[e]);
       }
       i16x8_t fk;
 #pragma unroll

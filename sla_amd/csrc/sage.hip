@@ -48,14 +48,20 @@ __global__ __launch_bounds__(256) void quant_int8_kernel(const uint16_t* __restr
 #pragma unroll
     for (int e = 0; e < 8; ++e) cm[e] = E::to_float((uint16_t)m[e]);
   }
+  // every row of the block is asked for before the first is used (rows past L lie outside the descriptor and read as
+  // zero): one memory latency per block instead of one per row group
+  const __amdgpu_buffer_rsrc_t xb = make_rsrc(x + lay.head(bh), lay.head_range_bytes(L, D));
+  i16x8_t raw[NP];
+#pragma unroll
+  for (int p = 0; p < NP; ++p)
+    raw[p] = buf_load_b128(xb, (uint32_t)(blk * BLK + lrow + p * RPP) * (uint32_t)(lay.sl * 2) + (uint32_t)lcol * 2u);
   float val[NP][8];
   float amax = 0.f;
 #pragma unroll
   for (int p = 0; p < NP; ++p) {
     const int grow = blk * BLK + lrow + p * RPP;
-    i16x8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
+    i16x8_t v = raw[p];
     const bool ok = grow < L;
-    if (ok) v = *reinterpret_cast<const i16x8_t*>(x + lay.head(bh) + (size_t)grow * (size_t)lay.sl + lcol);
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       val[p][e] = ok ? E::to_float((uint16_t)v[e]) - cm[e] : 0.f;
