@@ -679,6 +679,17 @@ static int linear_bwd_impl(const void* q, const void* k, const void* v, const fl
     hipLaunchKernelGGL(linear_bwd_reduce_heads_kernel, dim3(cdiv(D * D, 256)), dim3(256), 0, st,
                        (const float*)(ws + w.dw_head), (const float*)(ws + w.db_head), d_weight, d_bias, BH, D);
   if (!(steps & LB_KEYS)) return check_launch("linear_bwd");
+  if constexpr (D == 128) if (streamed) {
+#define SLA_LBK_LAUNCH(FM)                                                                                                \
+  hipLaunchKernelGGL((linear_bwd_keys_kernel<Tag, FM>), dim3(w.ss.nsplit, BH), dim3(512), 0, st, (const uint16_t*)k,        \
+                     (const uint16_t*)v, (const uint16_t*)(ws + w.ds), (const uint16_t*)(ws + w.dst),                       \
+                     (const float*)(ws + w.dz), (uint16_t*)dk, (uint16_t*)dv, lin, L, w.ss.rows_per_split, accumulate)
+    if (fmap == SLA_FMAP_ELU) SLA_LBK_LAUNCH(SLA_FMAP_ELU);
+    else if (fmap == SLA_FMAP_RELU) SLA_LBK_LAUNCH(SLA_FMAP_RELU);
+    else SLA_LBK_LAUNCH(SLA_FMAP_SOFTMAX);
+#undef SLA_LBK_LAUNCH
+    return check_launch("linear_bwd");
+  }
   if (lin.sl == D)
     hipLaunchKernelGGL((linear_bwd_kv_kernel<Tag, D, NW_KV, true>), dim3(cdiv(L, 32 * NW_KV * tiles_kv), BH), dim3(64 * NW_KV),
                        0, st, (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)(ws + w.ds),

@@ -363,6 +363,228 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   }
 }
 
+// Key side of the same backward, head dim 128: dv = c dS, dc = v dS^T + dz, dk = phi'(k) dc with c = phi(k).
+// grid (slices of L, heads), 8 waves; dS [d1][d2] and dS^T [d2][d1] (16 bit, rows padded by 16 bytes) and dz stay in LDS,
+// every wave walks its own 16-key tiles of the slice and never meets another wave after the staging barrier:
+//   rows of k, v (fetched a tile ahead) -> two wave-private swizzled 4 KB tiles; phi(k) takes the place of k;
+//   dv^T = dS^T c^T and dc^T = dS v^T as 16x16x32 products (a key's row spread over 4 lanes, B operands read row-wise
+//   from the wave's tiles); dk, dv go back over the tiles and leave as whole rows, added to what dk, dv held (asked
+//   for at the start of the tile) when accumulating.
+template <typename Tag, int FMAP>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void linear_bwd_keys_kernel(
+    const uint16_t* __restrict__ k, const uint16_t* __restrict__ v, const uint16_t* __restrict__ ds,
+    const uint16_t* __restrict__ dst, const float* __restrict__ dz, uint16_t* __restrict__ dk, uint16_t* __restrict__ dv,
+    const RowLayout lin, int L, int rows_per_split, int accumulate) {
+  using E = Elem<Tag>;
+  constexpr int fmap = FMAP;
+  constexpr int D = 128;
+  constexpr int PSTR = D * 2 + 16;               // row pitch of the staged matrices
+  constexpr int WT = 16 * D * 2;                 // bytes of a wave's tile
+  __shared__ __attribute__((aligned(16))) char smem[2 * D * PSTR + D * 4 + 8 * 2 * WT];
+  char* const sDS = smem;                        // dS   [d1][d2]: A operand of dc^T = dS v^T
+  char* const sDST = smem + D * PSTR;            // dS^T [d2][d1]: A operand of dv^T = dS^T c^T
+  float* const sDZ = reinterpret_cast<float*>(smem + 2 * D * PSTR);
+
+  const int split = blockIdx.x, bh = blockIdx.y;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  char* const tK = smem + 2 * D * PSTR + D * 4 + wave * 2 * WT;    // k rows, then phi(k), then dk
+  char* const tV = tK + WT;                                          // v rows, then dv
+  const int row_begin = split * rows_per_split;
+  const int row_end = min(L, row_begin + rows_per_split);
+  {
+    const uint16_t* s0 = ds + (size_t)bh * D * D;
+    const uint16_t* s1 = dst + (size_t)bh * D * D;
+    for (int idx = tid; idx < D * D / 8; idx += 512) {
+      const int row = idx / (D / 8), col = (idx % (D / 8)) * 8;
+      *reinterpret_cast<i16x8_t*>(sDS + row * PSTR + col * 2) = *reinterpret_cast<const i16x8_t*>(s0 + (size_t)row * D + col);
+      *reinterpret_cast<i16x8_t*>(sDST + row * PSTR + col * 2) = *reinterpret_cast<const i16x8_t*>(s1 + (size_t)row * D + col);
+    }
+    if (tid < D) sDZ[tid] = dz[(size_t)bh * D + tid];
+  }
+  __syncthreads();
+
+  const uint32_t range = lin.head_range_bytes(L, D);
+  const __amdgpu_buffer_rsrc_t k_rs = make_rsrc(k + lin.head(bh), range);
+  const __amdgpu_buffer_rsrc_t v_rs = make_rsrc(v + lin.head(bh), range);
+  const __amdgpu_buffer_rsrc_t dk_rs = make_rsrc(dk + lin.head(bh), accumulate ? range : 0u);
+  const __amdgpu_buffer_rsrc_t dv_rs = make_rsrc(dv + lin.head(bh), accumulate ? range : 0u);
+  uint16_t* const dkh = dk + lin.head(bh);
+  uint16_t* const dvh = dv + lin.head(bh);
+  const size_t pitch = (size_t)lin.sl;
+  const uint32_t pitch_b = (uint32_t)lin.sl * 2u;
+
+  // loader / writer layout of a wave's tile: lane -> row lane / 16 + 4 p, 16-byte piece lane % 16
+  const int frow = lane >> 4, lp = lane & 15;
+  uint32_t f_off[4];
+#pragma unroll
+  for (int p = 0; p < 4; ++p) f_off[p] = lbs_off(frow + 4 * p, 8 * lp);
+  // product layout: lane = (key l of the tile's 16, quarter h): d = 16 T + 4 h + j
+  const int l = lane & 15, h = lane >> 4;
+  uint32_t acc_off[8];        // (l, 16 T + 4 h)
+#pragma unroll
+  for (int T = 0; T < 8; ++T) acc_off[T] = lbs_off(l, 16 * T + 4 * h);
+  uint32_t b_off[4];          // (l, 32 c + 8 h): B-operand order
+#pragma unroll
+  for (int c = 0; c < 4; ++c) b_off[c] = lbs_off(l, 32 * c + 8 * h);
+  const uint32_t a_base = (uint32_t)l * PSTR + (uint32_t)h * 16u;     // row 16 T + l of a staged matrix: + 16 PSTR per T, + 64 per c
+
+  i16x8_t rk[4], rv[4];
+  auto fetch_kv = [&](int r0) __attribute__((always_inline)) {
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      const uint32_t o = (uint32_t)(r0 + frow + 4 * p) * pitch_b + 16 * lp;      // rows past L read as zero
+      rk[p] = buf_load_b128(k_rs, o);
+      rv[p] = buf_load_b128(v_rs, o);
+    }
+  };
+  const int first = row_begin + 16 * wave;
+  if (first < row_end) fetch_kv(first);
+  for (int r0 = first; r0 < row_end; r0 += 128) {
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      *reinterpret_cast<i16x8_t*>(tK + f_off[p]) = rk[p];
+      *reinterpret_cast<i16x8_t*>(tV + f_off[p]) = rv[p];
+    }
+    wave_lds_fence();
+    // what dk, dv hold (for this tile) and the next tile's rows: both have the whole tile to arrive
+    i16x8_t rdk[4], rdv[4];
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      const uint32_t o = (uint32_t)(r0 + frow + 4 * p) * pitch_b + 16 * lp;
+      rdk[p] = buf_load_b128(dk_rs, o);
+      rdv[p] = buf_load_b128(dv_rs, o);
+    }
+    if (r0 + 128 < row_end) fetch_kv(r0 + 128);
+
+    i16x4_t xraw[8];
+#pragma unroll
+    for (int T = 0; T < 8; ++T) xraw[T] = *reinterpret_cast<const i16x4_t*>(tK + acc_off[T]);
+    auto xv = [&](int T, int j) __attribute__((always_inline)) { return E::to_float((uint16_t)xraw[T][j]); };
+    float mx = 0.f, inv = 1.f;
+    {
+      float a[8][4];
+      if (fmap == SLA_FMAP_SOFTMAX) {
+        mx = xv(0, 0);
+#pragma unroll
+        for (int T = 0; T < 8; ++T)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) mx = fmaxf(mx, xv(T, j));
+        mx = fmaxf(mx, __shfl_xor(mx, 16));
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        float sum = 0.f;
+#pragma unroll
+        for (int T = 0; T < 8; ++T)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            a[T][j] = __expf(xv(T, j) - mx);
+            sum += a[T][j];
+          }
+        sum += __shfl_xor(sum, 16);
+        sum += __shfl_xor(sum, 32);
+        inv = 1.0f / sum;
+#pragma unroll
+        for (int T = 0; T < 8; ++T)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) a[T][j] = round16<Tag>(a[T][j] * inv);
+      } else {
+#pragma unroll
+        for (int T = 0; T < 8; ++T)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) a[T][j] = fmap_pointwise<Tag>(fmap, xv(T, j));
+      }
+      // c = phi(k) over the raw rows (this lane's own places; a key's gradients depend on its own row only, so rows
+      // past the end, which are never written, need no care)
+#pragma unroll
+      for (int T = 0; T < 8; ++T) {
+        i32x2_t w;
+        w[0] = (int)E::pack2(a[T][0], a[T][1]);
+        w[1] = (int)E::pack2(a[T][2], a[T][3]);
+        *reinterpret_cast<i32x2_t*>(tK + acc_off[T]) = w;
+      }
+    }
+    wave_lds_fence();
+    // dv^T = dS^T c^T ; dc^T = dS v^T
+    f32x4_t dva[8], dca[8];
+#pragma unroll
+    for (int T = 0; T < 8; ++T) {
+      dva[T] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      dca[T] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    }
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const i16x8_t cf = *reinterpret_cast<const i16x8_t*>(tK + b_off[c]);
+      const i16x8_t vf = *reinterpret_cast<const i16x8_t*>(tV + b_off[c]);
+#pragma unroll
+      for (int T = 0; T < 8; ++T) {
+        dva[T] = E::mfma16(*reinterpret_cast<const i16x8_t*>(sDST + a_base + T * 16 * PSTR + c * 64), cf, dva[T]);
+        dca[T] = E::mfma16(*reinterpret_cast<const i16x8_t*>(sDS + a_base + T * 16 * PSTR + c * 64), vf, dca[T]);
+      }
+    }
+    wave_lds_fence();      // (the tiles are rewritten below: every read of them above comes first)
+    // dc += dz ; dk = phi'(k) dc
+#pragma unroll
+    for (int T = 0; T < 8; ++T) {
+      const f32x4_t zz = *reinterpret_cast<const f32x4_t*>(sDZ + 16 * T + 4 * h);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) dca[T][j] += zz[j];
+    }
+    if (fmap == SLA_FMAP_RELU) {
+#pragma unroll
+      for (int T = 0; T < 8; ++T)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) dca[T][j] = xv(T, j) > 0.f ? dca[T][j] : 0.f;
+    } else if (fmap == SLA_FMAP_ELU) {
+#pragma unroll
+      for (int T = 0; T < 8; ++T)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) dca[T][j] = xv(T, j) > 0.f ? dca[T][j] : dca[T][j] * __expf(xv(T, j));
+    } else {
+      float dot = 0.f;
+#pragma unroll
+      for (int T = 0; T < 8; ++T)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) dot += __expf(xv(T, j) - mx) * inv * dca[T][j];       // the unrounded softmax
+      dot += __shfl_xor(dot, 16);
+      dot += __shfl_xor(dot, 32);
+#pragma unroll
+      for (int T = 0; T < 8; ++T)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) dca[T][j] = __expf(xv(T, j) - mx) * inv * (dca[T][j] - dot);
+    }
+#pragma unroll
+    for (int T = 0; T < 8; ++T) {
+      i32x2_t wk, wv;
+      wk[0] = (int)E::pack2(dca[T][0], dca[T][1]);
+      wk[1] = (int)E::pack2(dca[T][2], dca[T][3]);
+      wv[0] = (int)E::pack2(dva[T][0], dva[T][1]);
+      wv[1] = (int)E::pack2(dva[T][2], dva[T][3]);
+      *reinterpret_cast<i32x2_t*>(tK + acc_off[T]) = wk;
+      *reinterpret_cast<i32x2_t*>(tV + acc_off[T]) = wv;
+    }
+    wave_lds_fence();
+    // whole rows out: 16-bit value + what the tensor held, one rounded add (nothing held when not accumulating)
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      const int grow = r0 + frow + 4 * p;
+      const i16x8_t k16 = *reinterpret_cast<const i16x8_t*>(tK + f_off[p]);
+      const i16x8_t v16 = *reinterpret_cast<const i16x8_t*>(tV + f_off[p]);
+      i32x4_t wk, wv;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        wk[j] = (int)E::pack2(E::to_float((uint16_t)k16[2 * j]) + E::to_float((uint16_t)rdk[p][2 * j]),
+                              E::to_float((uint16_t)k16[2 * j + 1]) + E::to_float((uint16_t)rdk[p][2 * j + 1]));
+        wv[j] = (int)E::pack2(E::to_float((uint16_t)v16[2 * j]) + E::to_float((uint16_t)rdv[p][2 * j]),
+                              E::to_float((uint16_t)v16[2 * j + 1]) + E::to_float((uint16_t)rdv[p][2 * j + 1]));
+      }
+      if (grow < row_end) {
+        *reinterpret_cast<i32x4_t*>(dkh + (size_t)grow * pitch + 8 * lp) = wk;
+        *reinterpret_cast<i32x4_t*>(dvh + (size_t)grow * pitch + 8 * lp) = wv;
+      }
+    }
+    wave_lds_fence();      // the next tile's rows go over these
+  }
+}
+
 // Sums of the slices' partials in ascending slice order: M per head (fp32, both orientations), dz, db per head.
 // grid (cdiv(D*D, 256), BH).
 __global__ __launch_bounds__(256) void linear_bwd_sum_kernel(const float* __restrict__ m_part, const float* __restrict__ dz_part,
