@@ -185,7 +185,8 @@ int sla_sparse_attn_linear_fwd_strided(const void* q, const void* k, const void*
  * per-key-block lists of the map, and the per-head reductions and small products of the linear branch - so that they run
  * beside the long dQ and dK/dV kernels instead of between them; `stream` waits for all of it before the call's last
  * kernel, so later work needs ordering against `stream` only.  The streams must belong to the current device and have the
- * same (default) priority.
+ * same (default) priority.  The first call with a second stream on a device creates four events (no device memory), kept
+ * for later calls; calls from several host threads take turns enqueueing.
  * Replaces autograd through SparseLinearAttention.forward, sparse_linear_attention/core.py:88-100 with
  * kernel.py:277-320. */
 int sla_module_bwd(const void* q, const void* k, const void* v, const int64_t* qkv_strides, const void* o_s,
