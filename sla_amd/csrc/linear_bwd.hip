@@ -616,6 +616,7 @@ template <typename Tag, int D>
 static int linear_bwd_impl(const void* q, const void* k, const void* v, const float* weight, const void* d_out, void* dq,
                            void* dk, void* dv, const RowLayout& lin, const RowLayout& ldo, float* d_weight, float* d_bias,
                            int fmap, int BH, int L, int flags, char* ws, hipStream_t st, int steps) {
+  if (steps == 0) return SLA_OK;        // (arguments checked, nothing asked for)
   const LinBwdWs w = lin_bwd_ws(BH, L, D);
   const int accumulate = flags & SLA_BWD_ACCUMULATE;
   if ((steps & LB_STATES) && !(flags & SLA_BWD_STATES_READY)) {

@@ -65,6 +65,9 @@ extern "C" int sla_module_bwd(const void* q, const void* k, const void* v, const
                             H, L, D, lflags, linear_workspace, linear_workspace_bytes, s, steps);
   };
   int rc;
+  // every argument of both calls is checked before the first kernel of either is launched
+  if ((rc = sparse(st, 0))) return rc;
+  if ((rc = linear(st, 0))) return rc;
   if (!side || side == st) {
     // one stream: the same order, the short kernels in between
     if ((rc = sparse(st, SB_ALL))) return rc;

@@ -710,6 +710,7 @@ static int bwd_impl(const void* q, const void* k, const void* v, const void* o, 
                     const int8_t* sparse_map, const void* lut, int lut64, void* dq, void* dk, void* dv,
                     const RowLayout& lin, const RowLayout& ldo, int BH, int L, int topk, float qk_scale, char* ws,
                     hipStream_t st, int steps) {
+  if (steps == 0) return SLA_OK;        // (arguments checked, nothing asked for)
   const BwdWs w = bwd_ws(BH, L, D, BLKQ, 64, topk);
   const int Mblk = cdiv(L, BLKQ), Nblk = cdiv(L, 64);
   float* delta = (float*)(ws + w.delta);

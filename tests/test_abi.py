@@ -65,6 +65,7 @@ def test_attention_rejects_bad_shapes_before_launch():
 
 
 def test_other_entry_points_validate():
+    import ctypes
     lib = _lib.load()
     assert lib.sla_mean_pool(None, FAKE, 1, 1, 64, 64, 64, None) == _lib.ERR_BAD_ARG
     assert lib.sla_mean_pool(FAKE, FAKE, 1, 1, 64, 60, 64, None) == _lib.ERR_UNSUPPORTED
@@ -100,6 +101,17 @@ def test_other_entry_points_validate():
     assert states < lib.sla_workspace_bytes(_lib.WS_LINEAR_FWD, 1, 1, 12, 32760, 128, 64, 64, 0)
     assert lib.sla_sparse_attn_bwd(FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, 8, FAKE, FAKE, FAKE, 1, 1, 1, 128, 128, 64,
                                    64, 1, 0.1, FAKE, 8, None) == _lib.ERR_WORKSPACE
+    # the one-call backward: its own arguments first, then what the two calls it stands for check
+    mb = lambda **kw: lib.sla_module_bwd(  # noqa: E731
+        FAKE, FAKE, FAKE, kw.get("qs"), FAKE, FAKE, kw.get("dos"), FAKE, FAKE, FAKE, 8, kw.get("w", FAKE), FAKE, FAKE, FAKE,
+        FAKE, FAKE, FAKE, 1, kw.get("fmap", 0), 1, 1, 128, 128, 64, 64, 1, 0.1, kw.get("flags", 0), FAKE,
+        kw.get("ws_s", 1 << 30), FAKE, kw.get("ws_l", 1 << 30), None, None)
+    assert mb(flags=1) == _lib.ERR_BAD_ARG and "flag" in _lib.last_error()           # accumulation is implied, not a flag
+    assert mb(qs=(ctypes.c_int64 * 3)(16384, 16384, 128)) == _lib.ERR_BAD_ARG and "stride" in _lib.last_error()
+    assert mb(ws_s=8) == _lib.ERR_WORKSPACE
+    assert mb(ws_l=8) == _lib.ERR_WORKSPACE
+    assert mb(w=None) == _lib.ERR_BAD_ARG
+    assert mb(fmap=5) == _lib.ERR_BAD_ARG
     assert lib.sage_quant_qk(FAKE, FAKE, 1, 1, 1, 128, 128, 64, 64, FAKE, FAKE, FAKE, FAKE, FAKE, 1 << 30, None) == _lib.ERR_UNSUPPORTED
     assert "BLKQ=128" in _lib.last_error()
     assert lib.sage_quant_v(FAKE, 1, 1, 1, 128, 32, FAKE, FAKE, 448.0, FAKE, 1 << 30, None) == _lib.ERR_UNSUPPORTED
