@@ -9,6 +9,15 @@ static __device__ __forceinline__ float round16(float x) {
   return Elem<Tag>::to_float(Elem<Tag>::from_float(x));
 }
 
+// Two values rounded to 16 bit with one packing conversion; returns the packed pair (a in the low half).
+template <typename Tag>
+static __device__ __forceinline__ uint32_t round16_pair(float a, float b, float& ra, float& rb) {
+  const uint32_t p = Elem<Tag>::pack2(a, b);
+  ra = Elem<Tag>::to_float((uint16_t)(p & 0xffffu));
+  rb = Elem<Tag>::to_float((uint16_t)(p >> 16));
+  return p;
+}
+
 // relu(x) or elu(x)+1, rounded to 16 bit where the reference materialises a 16-bit tensor
 // (elu: once after elu and again after the +1).
 template <typename Tag>

@@ -71,7 +71,21 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   const __amdgpu_buffer_rsrc_t kh = make_rsrc(k + head_off, head_bytes);
   const __amdgpu_buffer_rsrc_t vh = make_rsrc(v + head_off, head_bytes);
 
-  // This wave's 64 query rows are requested first, straight in B-operand order (lane = row, 16 bytes per 16-wide
+  // ---- the two look-up rows -> per-wave step lists
+  const size_t rowA = ((size_t)bh * Mblk + 2 * pj) * topk;
+  const size_t rowB = pair_full ? rowA + topk : rowA;
+  auto lut_at = [&](size_t i) __attribute__((always_inline)) -> int {       // (the low word of a 64-bit entry)
+    return reinterpret_cast<const int*>(lut)[lut64 ? 2 * i : i];
+  };
+  // The first 64 entries of both rows are asked for before anything else: the schedule of the pair hangs on them, and
+  // loads come back in the order they were issued.  They stay in registers for the passes below (lanes past the end
+  // of a row hold its last entry and are not looked at).
+  int a_raw = 0, b_raw = 0;
+  if (topk > 0) {                              // (an empty look-up table may be a null pointer)
+    a_raw = lut_at(rowA + min(lane, topk - 1));
+    b_raw = lut_at(rowB + min(lane, topk - 1));
+  }
+  // This wave's 64 query rows are requested next, straight in B-operand order (lane = row, 16 bytes per 16-wide
   // chunk of the head dim): they arrive while the look-up rows are merged.  (A lane-per-row access touches 32 memory
   // lines per instruction; it happens once per workgroup and spares a trip through LDS and a barrier.)
   const int qrow0 = mb * 64;
@@ -92,12 +106,7 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     for (int i = 0; i < 4 * SLOT / (128 * 16); ++i) reinterpret_cast<i32x4_t*>(smem + 4 * SLOT)[i * 128 + tid] = i32x4_t{0, 0, 0, 0};
   }
 
-  // ---- the two look-up rows -> per-wave step lists
-  const size_t rowA = ((size_t)bh * Mblk + 2 * pj) * topk;
-  const size_t rowB = pair_full ? rowA + topk : rowA;
-  auto lut_at = [&](size_t i) __attribute__((always_inline)) -> int {
-    return lut64 ? (int)reinterpret_cast<const long long*>(lut)[i] : reinterpret_cast<const int*>(lut)[i];
-  };
+  // ---- per-wave step lists
   // (The split assumes what the mask builder guarantees: no key block twice in a row, every index below 4096.  A row
   //  that names a block twice makes the pair walk both rows unshared, in the order given, each block as often as it
   //  is named; an index is only ever used modulo 4096 here, and as it is where the rows of K and V are addressed,
@@ -106,17 +115,11 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   bitmap[1][tid] = 0;
   if (tid == 0) repeated = 0;
   __syncthreads();
-  // Every wave reads both rows (the first 64 entries of either stay in registers: the passes below would otherwise each
-  // wait for memory again) and marks its own row's blocks.
-  int a_first = 0, b_first = 0;
+  // Every wave reads both rows and marks its own row's blocks.
   for (int c0 = 0; c0 < topk; c0 += 64) {
     const int i = c0 + lane;
     if (i < topk) {
-      const int a = lut_at(rowA + i) & 4095, b = lut_at(rowB + i) & 4095;
-      if (c0 == 0) {
-        a_first = a;
-        b_first = b;
-      }
+      const int a = (c0 == 0 ? a_raw : lut_at(rowA + i)) & 4095, b = (c0 == 0 ? b_raw : lut_at(rowB + i)) & 4095;
       const int x = w ? b : a;
       const uint32_t seen = atomicOr(&bitmap[w][x >> 5], 1u << (x & 31));
       if ((seen >> (x & 31)) & 1u) repeated = 1;
@@ -124,10 +127,10 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   }
   __syncthreads();
   auto row_a = [&](int c0, int i) __attribute__((always_inline)) -> int {
-    return c0 == 0 ? a_first : (i < topk ? lut_at(rowA + i) & 4095 : 0);
+    return c0 == 0 ? (a_raw & 4095) : (i < topk ? lut_at(rowA + i) & 4095 : 0);
   };
   auto row_b = [&](int c0, int i) __attribute__((always_inline)) -> int {
-    return c0 == 0 ? b_first : (i < topk ? lut_at(rowB + i) & 4095 : 0);
+    return c0 == 0 ? (b_raw & 4095) : (i < topk ? lut_at(rowB + i) & 4095 : 0);
   };
   // Step p of the pair follows entry p of the first row: a key block the second row names as well is a shared step;
   // otherwise it is an own step, on which wave 0 takes that block and wave 1 the next block (in the order of its row)
@@ -545,13 +548,12 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   __syncthreads();
   const size_t out_off = lout.head(bh) + (size_t)qrow0 * (size_t)lout.sl;
   // Fused linear branch: the per-head state KVW^T (D x D, 16 bit) goes into the V ring the way K half-tiles do (four
-  // slots of 32 rows, swizzled pieces, each wave requests half), the unscaled q rows come again in B-operand order.
-  // z and the bias come up front as well: at one wave per SIMD nothing hides a load issued where it is used.
-  i16x8_t qraw[2][DC], zreg[DC];
+  // slots of 32 rows, swizzled pieces, each wave requests half); the q rows are the resident B operands of the score
+  // products.  z and the bias come up front as well: at one wave per SIMD nothing hides a load issued where it is used.
+  i16x8_t zreg[DC];
   f32x4_t breg[DT][4];
   if (FUSED) {
     const __amdgpu_buffer_rsrc_t sth = make_rsrc(kvwt + (size_t)bh * D * D, D * D * 2);
-    const __amdgpu_buffer_rsrc_t qh = make_rsrc(q + head_off, head_bytes);
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       // instruction i of this wave: rows 64w + 4i .. +3 of the state -> slot 4 + 2w + i / 8, rows 4 (i % 8) ..
@@ -559,11 +561,6 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
       const uint32_t soff = (uint32_t)(4 * j + lrow) * ROWB + ((lslot ^ ((4 * j + lrow) & 15)) * 16);
       SLA_PAIR_FETCH(sth, soff, (uint32_t)((64 * w + 4 * (i - j)) * ROWB), smem_addr, (4 + 2 * w + (i >> 3)) * SLOT + (i & 7) * 1024);
     }
-#pragma unroll
-    for (int qt = 0; qt < 2; ++qt)
-#pragma unroll
-      for (int c = 0; c < DC; ++c)
-        qraw[qt][c] = buf_load_b128(qh, ((uint32_t)(qrow0 + 32 * qt + r) * pitch + 16 * c + 8 * g) * 2);
     const uint16_t* z_h = zst + (size_t)bh * D;
 #pragma unroll
     for (int c = 0; c < DC; ++c) zreg[c] = *reinterpret_cast<const i16x8_t*>(z_h + 16 * c + 8 * g);
@@ -572,8 +569,10 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 #pragma unroll
       for (int i4 = 0; i4 < 4; ++i4) {
         const f32x4_t b4 = *reinterpret_cast<const f32x4_t*>(bias + 32 * et + 8 * i4 + 4 * g);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) breg[et][i4][j] = round16<Tag>(b4[j]);
+        float b0, b1, b2, b3;
+        round16_pair<Tag>(b4[0], b4[1], b0, b1);
+        round16_pair<Tag>(b4[2], b4[3], b2, b3);
+        breg[et][i4] = f32x4_t{b0, b1, b2, b3};
       }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
@@ -609,25 +608,60 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
       flush_rows(o + out_off + (size_t)(32 * qt) * (size_t)lout.sl, (size_t)lout.sl);
     } else {
       // ---- linear branch of the same rows (see sparse_fwd_kernel) ----
-      // (the resident fragments hold q scaled for the attention: these are the unscaled rows)
-      float f[DC][8];
-#pragma unroll
-      for (int c = 0; c < DC; ++c)
-#pragma unroll
-        for (int j = 0; j < 8; ++j) f[c][j] = E::to_float((uint16_t)qraw[qt][c][j]);
-      float row_mx, row_inv;
-      phi_row_pair<Tag, DC>(fmap, f, row_mx, row_inv);
+      // (the resident B operands of the score products are the rows of q as they came from memory)
+      // Values that the reference rounds to 16 bit are rounded two at a time (one conversion instruction packs two) and
+      // taken apart again where the arithmetic goes on in fp32; a packed pair of phi(q) is a register of the B operand.
       float den = 0.f;
       i16x8_t fq[DC];
+      auto pair_done = [&](int c, int j2, float v0, float v1, i32x4_t& pw) __attribute__((always_inline)) {
+        float g0, g1, p0, p1;
+        pw[j2] = (int)round16_pair<Tag>(v0, v1, g0, g1);
+        const uint32_t zz = (uint32_t)__builtin_bit_cast(i32x4_t, zreg[c])[j2];
+        round16_pair<Tag>(g0 * E::to_float((uint16_t)(zz & 0xffffu)), g1 * E::to_float((uint16_t)(zz >> 16)), p0, p1);
+        den += p0;
+        den += p1;
+      };
+      if (fmap == SLA_FMAP_SOFTMAX) {
+        float f[DC][8];
 #pragma unroll
-      for (int c = 0; c < DC; ++c) {
-        const i16x8_t zc = zreg[c];
-        i32x4_t pw;
+        for (int c = 0; c < DC; ++c)
 #pragma unroll
-        for (int j = 0; j < 8; ++j) den += round16<Tag>(f[c][j] * E::to_float((uint16_t)zc[j]));
+          for (int j = 0; j < 8; ++j) f[c][j] = E::to_float((uint16_t)qf[qt][c][j]);
+        float row_mx, row_inv;
+        phi_row_pair<Tag, DC>(fmap, f, row_mx, row_inv);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) pw[j] = (int)E::pack2(f[c][2 * j], f[c][2 * j + 1]);
-        fq[c] = __builtin_bit_cast(i16x8_t, pw);
+        for (int c = 0; c < DC; ++c) {
+          i32x4_t pw;
+#pragma unroll
+          for (int j2 = 0; j2 < 4; ++j2) pair_done(c, j2, f[c][2 * j2], f[c][2 * j2 + 1], pw);
+          fq[c] = __builtin_bit_cast(i16x8_t, pw);
+        }
+      } else if (fmap == SLA_FMAP_RELU) {
+        // (the choice of the map stays outside the loops over the elements)
+#pragma unroll
+        for (int c = 0; c < DC; ++c) {
+          i32x4_t pw;
+#pragma unroll
+          for (int j2 = 0; j2 < 4; ++j2) {
+            const uint32_t xx = (uint32_t)__builtin_bit_cast(i32x4_t, qf[qt][c])[j2];
+            pair_done(c, j2, fmaxf(E::to_float((uint16_t)(xx & 0xffffu)), 0.f), fmaxf(E::to_float((uint16_t)(xx >> 16)), 0.f), pw);
+          }
+          fq[c] = __builtin_bit_cast(i16x8_t, pw);
+        }
+      } else {
+#pragma unroll
+        for (int c = 0; c < DC; ++c) {
+          i32x4_t pw;
+#pragma unroll
+          for (int j2 = 0; j2 < 4; ++j2) {
+            const uint32_t xx = (uint32_t)__builtin_bit_cast(i32x4_t, qf[qt][c])[j2];
+            const float x0 = E::to_float((uint16_t)(xx & 0xffffu)), x1 = E::to_float((uint16_t)(xx >> 16));
+            float e0, e1;                                    // elu, rounded; then + 1, rounded by pair_done
+            round16_pair<Tag>(x0 > 0.f ? x0 : (__expf(x0) - 1.0f), x1 > 0.f ? x1 : (__expf(x1) - 1.0f), e0, e1);
+            pair_done(c, j2, e0 + 1.0f, e1 + 1.0f, pw);
+          }
+          fq[c] = __builtin_bit_cast(i16x8_t, pw);
+        }
       }
       den += __shfl_xor(den, 32);
       den = round16<Tag>(1e-5f + round16<Tag>(den));
@@ -653,8 +687,9 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 #pragma unroll
           for (int h = 0; h < 2; ++h) {
             const uint32_t x = (uint32_t)ws[h];
-            const float l0 = round16<Tag>(pin_f32(__builtin_fmaf(acc[4 * i4 + 2 * h], inv_den, b4[2 * h])));
-            const float l1 = round16<Tag>(pin_f32(__builtin_fmaf(acc[4 * i4 + 2 * h + 1], inv_den, b4[2 * h + 1])));
+            float l0, l1;
+            round16_pair<Tag>(pin_f32(__builtin_fmaf(acc[4 * i4 + 2 * h], inv_den, b4[2 * h])),
+                              pin_f32(__builtin_fmaf(acc[4 * i4 + 2 * h + 1], inv_den, b4[2 * h + 1])), l0, l1);
             wo[h] = (int)E::pack2(E::to_float((uint16_t)(x & 0xffff)) + l0, E::to_float((uint16_t)(x >> 16)) + l1);
           }
           *reinterpret_cast<i32x2_t*>(&stage_q[r * SSTR + e0]) = wo;
