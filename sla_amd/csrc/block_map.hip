@@ -430,7 +430,7 @@ static __device__ __forceinline__ int wave_inclusive_sum(int x, int lane) {
   return x;
 }
 
-// One wavefront per (bh, m) row (four rows per workgroup): radix-select the T-th largest key, then emit
+// One wavefront per (bh, m) row (four rows per workgroup): find the T-th largest key, then emit
 // winners in ascending index order (ties at the threshold value go to the lowest indices).  Writes the int8 map row and the look-up-table row.
 // EPL > 0: the row's keys live in EPL registers per lane (N <= 64*EPL); EPL == 0: keys in LDS.
 // LOW_BIT: lowest key bit that can differ (16 for 16-bit score dtypes, whose low bits are zero).
@@ -464,7 +464,7 @@ __global__ __launch_bounds__(256) void topk_kernel(const typename IO::raw* __res
     const int i = e * 64 + lane;
     return i < N ? keys[i] : 0u;
   };
-  // Radix select, eight key bits per pass (two passes for bf16 scores): the keys that agree with the digits found
+  // Keys in LDS: radix select, eight key bits per pass (two passes for bf16 scores): the keys that agree with the digits found
   // so far are counted per value of the next digit in a 256-bin histogram (LDS atomics of this wave on its own
   // bins); lane l then owns the four highest undecided digits 255 - 4l .. 252 - 4l, a prefix sum over the lanes
   // gives the number of keys above them, and the one lane whose digits straddle the wanted rank names the digit.
@@ -476,8 +476,25 @@ __global__ __launch_bounds__(256) void topk_kernel(const typename IO::raw* __res
   uint32_t thr = 0;          // digits decided so far
   int need = T;              // rank of the threshold among the keys that agree with them
   uint32_t* hist = hist_all[wave];
+  if (EPL > 0) {
+    // Keys in registers: the threshold is built bit by bit from the top, keeping a bit when at least T keys are at or
+    // above the value it gives (one compare per key and bit, counted through the wave's ballot: no memory traffic and no
+    // serialised atomics on the few histogram bins that the exponents of a row of scores fall into).  Slots past the
+    // end of the row hold key 0 and are never at or above a candidate, which has at least one bit set.
+    for (int b = 31; b >= LOW_BIT; --b) {
+      const uint32_t cand = thr | (1u << b);
+      int cnt = 0;
 #pragma unroll
-  for (int hi = 32; hi > LOW_BIT;) {
+      for (int e = 0; e < NR; ++e) cnt += __popcll(__ballot(kreg[e] >= cand));
+      if (cnt >= T) thr = cand;
+    }
+    int above = 0;
+#pragma unroll
+    for (int e = 0; e < NR; ++e) above += __popcll(__ballot(kreg[e] > thr));
+    need = T - above;        // how many of the keys equal to the threshold are taken
+  }
+#pragma unroll
+  for (int hi = EPL > 0 ? LOW_BIT : 32; hi > LOW_BIT;) {
     const int w = (hi - LOW_BIT) < 8 ? (hi - LOW_BIT) : 8;
     const int shift = hi - w;
     *reinterpret_cast<i32x4_t*>(&hist[4 * lane]) = i32x4_t{0, 0, 0, 0};
