@@ -130,7 +130,7 @@ static int linear_state_impl(const void* k, const void* v, const RowLayout& lay,
                              char* ws, hipStream_t st) {
   const LinWs w = lin_ws(BH, L, D);
   launch_state_build<Tag, D>(k, v, lay, weight, fmap, BH, L, ws, w, st, false);
-  hipLaunchKernelGGL((linear_fold_kernel<Tag>), dim3(cdiv(D * D, 256), BH), dim3(256), 0, st,
+  hipLaunchKernelGGL((linear_fold_kernel<Tag>), dim3(D / (1024 / D), BH), dim3(256), 0, st,
                      (const uint16_t*)(ws + w.kvt), weight, (uint16_t*)(ws + w.kvwt), (uint16_t*)(ws + w.wt), D);
   return check_launch("linear_state_fwd");
 }

@@ -622,7 +622,7 @@ static int linear_bwd_impl(const void* q, const void* k, const void* v, const fl
   if ((steps & LB_STATES) && !(flags & SLA_BWD_STATES_READY)) {
     // everything the forward's state build leaves: transposed state, z, and (fold) the folded state + 16-bit weight
     launch_state_build<Tag, D>(k, v, lin, weight, fmap, BH, L, ws, w.fwd, st, false);
-    hipLaunchKernelGGL((linear_fold_kernel<Tag>), dim3(cdiv(D * D, 256), BH), dim3(256), 0, st,
+    hipLaunchKernelGGL((linear_fold_kernel<Tag>), dim3(D / (1024 / D), BH), dim3(256), 0, st,
                        (const uint16_t*)(ws + w.fwd.kvt), weight, (uint16_t*)(ws + w.fwd.kvwt), (uint16_t*)(ws + w.fwd.wt), D);
   }
   uint16_t* kvt = (uint16_t*)(ws + w.fwd.kvt);

@@ -220,24 +220,48 @@ __global__ void linear_prep_weight_kernel(const float* __restrict__ weight, uint
 // ---- kernel 3 (forward, and a backward that has to rebuild the states): fold the projection into the state -------------------------------------------------
 // kvwt[bh][e][d1] = round16( sum_d2 round16(W[e][d2]) * KVT[d2][d1] ), fp32 accumulation in ascending d2.
 // (phi(Q) KV / den) W^T = (phi(Q) (KV W^T)) / den, so the output kernel needs one product per query tile.
-// grid (D*D/256, BH): thread (e, d1); the 256 threads of a workgroup share at most two rows e.
+// grid (D / (1024 / D), BH), 256 threads: a workgroup forms 1024 / D rows e for all d1, thread = (row e, four adjacent d1).
+// It sits between the state kernels and the attention kernel with nothing to overlap it, and its arithmetic is nothing:
+// the head's state and the workgroup's rows of W come into LDS with every load in flight at once, the sums then run
+// out of LDS.
 // The workgroups of head 0 also leave the 16-bit transposed weight wt[d][e] that a backward reads (what
 // linear_prep_weight_kernel writes), which saves the forward one launch in its chain of small kernels.
 template <typename Tag>
 __global__ __launch_bounds__(256) void linear_fold_kernel(const uint16_t* __restrict__ kvt, const float* __restrict__ weight,
                                                           uint16_t* __restrict__ kvwt, uint16_t* __restrict__ wt, int D) {
   using E = Elem<Tag>;
-  const int bh = blockIdx.y;
-  const int i = blockIdx.x * 256 + threadIdx.x;
-  if (i >= D * D) return;
-  const int e = i / D, d1 = i % D;
-  if (bh == 0) wt[d1 * D + e] = E::from_float(weight[i]);
-  const uint16_t* s = kvt + (size_t)bh * D * D + d1;
-  const float* w = weight + (size_t)e * D;
-  float acc = 0.f;
+  __shared__ __attribute__((aligned(16))) uint16_t s_kv[128 * 128];      // [d2][d1]
+  __shared__ float s_w[16 * 128];                                          // [row][d2], rounded to 16 bit
+  const int bh = blockIdx.y, tid = threadIdx.x;
+  const int groups = D >> 2;                       // threads per row e
+  const int rows = 256 / groups;                   // rows e per workgroup (8 at D 128, 16 at D 64)
+  const int e0 = blockIdx.x * rows;
+  const uint16_t* src = kvt + (size_t)bh * D * D;
+  for (int i = tid; i < D * D / 8; i += 256)
+    reinterpret_cast<i16x8_t*>(s_kv)[i] = reinterpret_cast<const i16x8_t*>(src)[i];
+  for (int i = tid; i < rows * D; i += 256) {
+    const float wv = weight[(size_t)e0 * D + i];
+    s_w[i] = round16<Tag>(wv);
+    if (bh == 0) {
+      const int e = e0 + i / D, d = i % D;
+      wt[d * D + e] = E::from_float(wv);
+    }
+  }
+  __syncthreads();
+  const int el = tid / groups, d1 = (tid % groups) * 4;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  const float* w = s_w + el * D;
 #pragma unroll 8
-  for (int d2 = 0; d2 < D; ++d2) acc += round16<Tag>(w[d2]) * E::to_float(s[(size_t)d2 * D]);
-  kvwt[(size_t)bh * D * D + i] = E::from_float(acc);
+  for (int d2 = 0; d2 < D; ++d2) {
+    const i16x4_t kv4 = *reinterpret_cast<const i16x4_t*>(&s_kv[d2 * D + d1]);
+    const float wv = w[d2];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[j] += wv * E::to_float((uint16_t)kv4[j]);
+  }
+  i32x2_t out;
+  out[0] = (int)E::pack2(acc[0], acc[1]);
+  out[1] = (int)E::pack2(acc[2], acc[3]);
+  *reinterpret_cast<i32x2_t*>(kvwt + (size_t)bh * D * D + (size_t)(e0 + el) * D + d1) = out;
 }
 
 // ---- workspace layout of the state build -----------------------------------------------------
