@@ -79,6 +79,13 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   // wave 0 fetches the log-sum-exps of a unit, wave 1 its deltas
   const __amdgpu_buffer_rsrc_t ldh = make_rsrc((w ? delta : lse) + (size_t)bh * L, (uint32_t)L * 4);
 
+  // The length of this key block's list and the first 128 entries of this work item's part of it are asked for before
+  // the fragments below (loads come back in the order they were issued, and the first requests for Q and dO hang on
+  // the entries); entries past the end of the list are read from inside its row of Mblk words and never used.
+  const int* mylist = list + ((size_t)bh * Nblk + nb) * Mblk;
+  const int e0 = sg * seg;
+  const int count_lane = count[(size_t)bh * Nblk + nb];
+  const int first_entry = mylist[min(e0 + tid, Mblk - 1)];
   // K^T and V^T fragments (B operands): this lane's key column, 8 adjacent d per chunk; parked in accumulation registers
   const int krow = nb * 64 + w * 32 + r;
   const bool kok = krow < L;
@@ -104,15 +111,13 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     }
 
   // this work item's part of the list, in units of 32 query rows (two per listed query block)
-  const int* mylist = list + ((size_t)bh * Nblk + nb) * Mblk;
-  const int e0 = sg * seg;
-  const int e1 = min(__builtin_amdgcn_readfirstlane(count[(size_t)bh * Nblk + nb]), (sg + 1) * seg);
+  const int e1 = min(__builtin_amdgcn_readfirstlane(count_lane), (sg + 1) * seg);
   const int nunits = 2 * (e1 - e0);
   auto entry_row0 = [&](int e) __attribute__((always_inline)) -> int {          // past the end: the last entry again (fetched, never used)
     return __builtin_amdgcn_readfirstlane(entries[min(e, e1 - e0 - 1)]) * 64;
   };
-
-  for (int i = tid; i < e1 - e0; i += 128) entries[i] = mylist[e0 + i];
+  if (tid < seg) entries[tid] = first_entry;
+  for (int i = 128 + tid; i < e1 - e0; i += 128) entries[i] = mylist[e0 + i];
 
   // ---- addressing ----
   // A request moves 4 rows (64 lanes x 16 bytes): lane -> row 4j + lane / 16 of this wave's 16 rows, 16-byte slot
@@ -161,9 +166,7 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 
   // ---- prologue: units 0, 1, 2 requested; S and dP of unit 0 ----
   f32x16_t s_a, dp_a, s_b, dp_b;
-#pragma unroll
-  for (int c = 0; c < DC; ++c) asm volatile("" : "+a"(kf[c]), "+a"(vf[c]));
-  __syncthreads();                                             // the zeros are in place before anything is requested
+  __syncthreads();                                             // the zeros and the entries are in place before anything is requested
   // first query rows of the listed blocks: E0 = of the entry of units u and u + 1, E1 = of the next one, E2 = of the one after
   int E0 = 0, E1 = 0, E2 = 0;
   if (nunits > 0) {
@@ -173,6 +176,11 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     request(E0, 0);
     request(E0 + 32, 1);
     request(E1, 2);
+  }
+  // (the wait for the K^T and V^T fragments comes here, behind the first requests, which only needed the list)
+#pragma unroll
+  for (int c = 0; c < DC; ++c) asm volatile("" : "+a"(kf[c]), "+a"(vf[c]));
+  if (nunits > 0) {
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NREQ) : "memory");
     __syncthreads();
 #pragma unroll
@@ -399,6 +407,12 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 1))) void
   const __amdgpu_buffer_rsrc_t vh = make_rsrc(v + head_off, lin.head_range_bytes(L, D));
   const int qrow0 = mb * 64;
 
+  // The first 64 entries of the look-up row are asked for before anything else: the first requests for K and V hang on
+  // them, and loads come back in the order they were issued (the low word of a 64-bit entry is the entry).
+  const size_t lut_row = ((size_t)bh * Mblk + mb) * topk;
+  auto lut_at = [&](size_t i) __attribute__((always_inline)) -> int { return reinterpret_cast<const int*>(lut)[lut64 ? 2 * i : i]; };
+  int first_entries = 0;
+  if (topk > 0) first_entries = lut_at(lut_row + min(lane, topk - 1));      // (an empty table may be a null pointer)
   // Q^T and dO^T fragments (B operands; rows past L read as zero), per-lane scalars of the two query tiles
   i16x8_t qf[2][DC], dof[2][DC];
   float lse_q[2], delta_q[2];
@@ -414,10 +428,8 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 1))) void
     lse_q[qt] = qrow < L ? lse[(size_t)bh * L + qrow] : INFINITY;
     delta_q[qt] = qrow < L ? delta[(size_t)bh * L + qrow] : 0.f;
   }
-  const size_t lut_row = ((size_t)bh * Mblk + mb) * topk;
-  for (int i = lane; i < topk; i += 64)
-    entries[i] = (uint16_t)(lut64 ? (int)reinterpret_cast<const long long*>(lut)[lut_row + i]
-                                  : reinterpret_cast<const int*>(lut)[lut_row + i]);
+  if (lane < topk) entries[lane] = (uint16_t)first_entries;
+  for (int i = 64 + lane; i < topk; i += 64) entries[i] = (uint16_t)lut_at(lut_row + i);
   // key rows past L are never written into LDS: what LDS holds in their place has to be finite (their probabilities
   // are masked to exactly 0 below)
 #pragma unroll
@@ -466,11 +478,6 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 1))) void
       const int piece = 4 * dt + 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);
       tfo[h][dt] = row * ROWB + ((piece ^ swz(row & 15)) * 16) + (lane & 1) * 8;
     }
-#pragma unroll
-  for (int qt = 0; qt < 2; ++qt)
-#pragma unroll
-    for (int c = 0; c < DC; ++c) asm volatile("" : "+a"(qf[qt][c]), "+a"(dof[qt][c]));
-
   // One unit = 32 keys, 48 MFMAs.  GEN = u % 2.
   f32x16_t s0, dp0, s1, dp1;
   auto unit = [&](int GEN, int key0, int key0_next2) __attribute__((always_inline)) {
@@ -583,6 +590,12 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 1))) void
     request(key_cur, 0);
     request(key_n1, 1);
   }
+  // Q^T and dO^T are only ever MFMA operands and are parked in the accumulation registers (the wait for them comes
+  // here, behind the first requests for K and V, which only needed the look-up row)
+#pragma unroll
+  for (int qt = 0; qt < 2; ++qt)
+#pragma unroll
+    for (int c = 0; c < DC; ++c) asm volatile("" : "+a"(qf[qt][c]), "+a"(dof[qt][c]));
   for (int u = 0; u < nunits; u += 2) {
     const int key_n2 = unit_rows(u + 2), key_n3 = unit_rows(u + 3);
     unit(0, key_cur, key_n2);
