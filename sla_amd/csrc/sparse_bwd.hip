@@ -718,9 +718,6 @@ static int bwd_impl(const void* q, const void* k, const void* v, const void* o, 
   int* list = (int*)(ws + w.list);
   const size_t rows = (size_t)BH * L;
   constexpr int RPB = 256 / (D / 8);
-  if (steps & SB_DQ)
-    hipLaunchKernelGGL((bwd_delta_kernel<Tag, D>), dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, st,
-                       (const uint16_t*)o, (const uint16_t*)d_o, ldo, delta, rows, L);
   if (steps & SB_LISTS) launch_col_lists(sparse_map, list, count, BH, Mblk, Nblk, st);
   int* nseg = (int*)(ws + w.nseg);
   int* slot0 = (int*)(ws + w.slot0);
@@ -736,12 +733,16 @@ static int bwd_impl(const void* q, const void* k, const void* v, const void* o, 
   const bool stream_dkdv = D == 128 && BLKQ == 64 && (uint64_t)lin.sl * 2u * (uint64_t)L < (1ull << 31) &&
                            (uint64_t)ldo.sl * 2u * (uint64_t)L < (1ull << 31);
   const bool stream_dq = stream_dkdv && topk <= DQ_STREAM_MAX_T && total_q >= 1024;      // (enough query blocks for a wave on every SIMD)
+  // delta = rowsum(dO * O): the dQ kernel of the common shape forms it for its own rows, the general one reads it
+  if ((steps & SB_DQ) && !stream_dq)
+    hipLaunchKernelGGL((bwd_delta_kernel<Tag, D>), dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, st,
+                       (const uint16_t*)o, (const uint16_t*)d_o, ldo, delta, rows, L);
 #define SLA_BWD_LAUNCH(CONTIG)                                                                                              \
   if (!(steps & SB_DQ)) {                                                                                                   \
   } else if (stream_dq)                                                                                                     \
     hipLaunchKernelGGL((bwd_dq_stream_kernel<Tag>), dim3(xcd_grid(total_q)), dim3(64), 0, st, (const uint16_t*)q,           \
-                       (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse, delta, lut, lut64, (uint16_t*)dq, \
-                       lin, ldo, L, Mblk, topk, qk_scale, total_q);                                                        \
+                       (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, (const uint16_t*)o, lse, delta, lut,   \
+                       lut64, (uint16_t*)dq, lin, ldo, L, Mblk, topk, qk_scale, total_q);                                  \
   else                                                                                                                      \
     hipLaunchKernelGGL((bwd_dq_kernel<Tag, D, BLKQ, CONTIG>), dim3(xcd_grid(total_q)), dim3(BLKQ * 2), 0, st,               \
                        (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse, delta, lut,   \

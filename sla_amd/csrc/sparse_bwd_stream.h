@@ -380,7 +380,7 @@ constexpr int DQ_STREAM_MAX_T = 2048;          // look-up rows longer than this 
 template <typename Tag>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 1))) void bwd_dq_stream_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ k, const uint16_t* __restrict__ v,
-    const uint16_t* __restrict__ d_o, const float* __restrict__ lse, const float* __restrict__ delta,
+    const uint16_t* __restrict__ d_o, const uint16_t* __restrict__ o, const float* __restrict__ lse, float* __restrict__ delta,
     const void* __restrict__ lut, int lut64, uint16_t* __restrict__ dq, const RowLayout lin, const RowLayout ldo, int L,
     int Mblk, int topk, float qk_scale, int total) {
   using E = Elem<Tag>;
@@ -414,8 +414,11 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 1))) void
   int first_entries = 0;
   if (topk > 0) first_entries = lut_at(lut_row + min(lane, topk - 1));      // (an empty table may be a null pointer)
   // Q^T and dO^T fragments (B operands; rows past L read as zero), per-lane scalars of the two query tiles
-  i16x8_t qf[2][DC], dof[2][DC];
+  // The rows of the forward's output come the same way: delta = rowsum(dO * O) (reference kernel.py:282-286, the
+  // preprocess step) is formed here, for this block's rows, and written out for the dK/dV kernel.
+  i16x8_t qf[2][DC], dof[2][DC], of[2][DC];
   float lse_q[2], delta_q[2];
+  const __amdgpu_buffer_rsrc_t oh = make_rsrc(o + (size_t)bh * L * D, (uint32_t)L * D * 2);      // (contiguous (B, H, L, D))
 #pragma unroll
   for (int qt = 0; qt < 2; ++qt) {
     const int qrow = qrow0 + 32 * qt + r;
@@ -423,10 +426,10 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 1))) void
     for (int c = 0; c < DC; ++c) {
       qf[qt][c] = buf_load_b128(qh, ((uint32_t)qrow * pitch + 16 * c + 8 * g) * 2);
       dof[qt][c] = buf_load_b128(doh, ((uint32_t)qrow * pitch_do + 16 * c + 8 * g) * 2);
+      of[qt][c] = buf_load_b128(oh, ((uint32_t)qrow * D + 16 * c + 8 * g) * 2);                  // rows past L: 0, delta 0
     }
     // rows past L: lse = +inf makes every probability exactly 0 (the reference loads `other=inf`)
     lse_q[qt] = qrow < L ? lse[(size_t)bh * L + qrow] : INFINITY;
-    delta_q[qt] = qrow < L ? delta[(size_t)bh * L + qrow] : 0.f;
   }
   if (lane < topk) entries[lane] = (uint16_t)first_entries;
   for (int i = 64 + lane; i < topk; i += 64) entries[i] = (uint16_t)lut_at(lut_row + i);
@@ -589,6 +592,27 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 1))) void
     key_n1 = unit_rows(1);
     request(key_cur, 0);
     request(key_n1, 1);
+  }
+  // delta of this lane's two rows.  The sum runs in the order of bwd_delta_kernel, whose thread t adds the eight products
+  // of columns 8t .. 8t+7 one after the other and then meets threads t^1, t^2, t^4, t^8: here t = 2c + g, so the first
+  // meeting is the one with lane^32 and the other three are between this lane's own chunks.
+#pragma unroll
+  for (int qt = 0; qt < 2; ++qt) {
+    float part[DC];
+#pragma unroll
+    for (int c = 0; c < DC; ++c) {
+      float acc = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc += E::to_float((uint16_t)of[qt][c][e]) * E::to_float((uint16_t)dof[qt][c][e]);
+      part[c] = acc + __shfl_xor(acc, 32);
+    }
+#pragma unroll
+    for (int sh = 1; sh < DC; sh <<= 1)
+#pragma unroll
+      for (int c = 0; c < DC; c += 2 * sh) part[c] = part[c] + part[c + sh];
+    delta_q[qt] = part[0];
+    const int qrow = qrow0 + 32 * qt + r;
+    if (g == 0 && qrow < L) delta[(size_t)bh * L + qrow] = part[0];
   }
   // Q^T and dO^T are only ever MFMA operands and are parked in the accumulation registers (the wait for them comes
   // here, behind the first requests for K and V, which only needed the look-up row)
