@@ -435,19 +435,22 @@ static int launch_fwd(const void* q, const void* k, const void* v, const void* l
   // neighbouring query blocks; it addresses a head with 32-bit byte offsets and indexes key blocks with 12 bits.
   // (Two query blocks per workgroup halve the number of workgroups: a launch too small to give every compute unit
   // its two workgroups keeps one query block per workgroup.)
-  const int total_p = BH * ((Mblk + 1) / 2);
-  if (D == 128 && BLKQ == 64 && topk <= PAIR_MAX_T && cdiv(L, 64) <= 4096 && (uint64_t)lin.sl * 2u * (uint64_t)L < (1ull << 31) &&
-      total_p >= 512) {
+  // 128-row query blocks go the same way: the two halves of a block are a pair whose rows of the table are one row.
+  const int Mblk64 = cdiv(L, 64);
+  const int total_p = BH * ((Mblk64 + 1) / 2);
+  if (D == 128 && (BLKQ == 64 || BLKQ == 128) && topk <= PAIR_MAX_T && Mblk64 <= 4096 &&
+      (uint64_t)lin.sl * 2u * (uint64_t)L < (1ull << 31) && total_p >= 512) {
     const int grid_p = xcd_grid(total_p);
+    const int one_row = BLKQ == 128;
     if (fl)
       hipLaunchKernelGGL((sparse_fwd_pair_kernel<Tag, true>), dim3(grid_p), dim3(128), 0, st, (const uint16_t*)q,
-                         (const uint16_t*)k, (const uint16_t*)v, lut, lut64, (uint16_t*)o, lse, lin, lout, L, Mblk, topk, c,
-                         total_p, fl->kvwt, fl->zst, fl->bias, fl->fmap, fl->o_s);
+                         (const uint16_t*)k, (const uint16_t*)v, lut, lut64, (uint16_t*)o, lse, lin, lout, L, Mblk64, topk, c,
+                         total_p, fl->kvwt, fl->zst, fl->bias, fl->fmap, fl->o_s, one_row);
     else
       hipLaunchKernelGGL((sparse_fwd_pair_kernel<Tag, false>), dim3(grid_p), dim3(128), 0, st, (const uint16_t*)q,
-                         (const uint16_t*)k, (const uint16_t*)v, lut, lut64, (uint16_t*)o, lse, lin, lout, L, Mblk, topk, c,
+                         (const uint16_t*)k, (const uint16_t*)v, lut, lut64, (uint16_t*)o, lse, lin, lout, L, Mblk64, topk, c,
                          total_p, (const uint16_t*)nullptr, (const uint16_t*)nullptr, (const float*)nullptr, 0,
-                         (uint16_t*)nullptr);
+                         (uint16_t*)nullptr, one_row);
     return check_launch("sparse_attn_fwd");
   }
 #define SLA_FWD_CASE(DD, BQ)                                                                                          \

@@ -36,7 +36,7 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ k, const uint16_t* __restrict__ v, const void* __restrict__ lut,
     int lut64, uint16_t* __restrict__ o, float* __restrict__ lse, const RowLayout lin, const RowLayout lout, int L, int Mblk,
     int topk, float scale_log2e, int total, const uint16_t* __restrict__ kvwt, const uint16_t* __restrict__ zst,
-    const float* __restrict__ bias, int fmap, uint16_t* __restrict__ o_s) {
+    const float* __restrict__ bias, int fmap, uint16_t* __restrict__ o_s, int one_row) {
   using E = Elem<Tag>;
   constexpr int D = 128, DC = D / 16, DT = D / 32;
   constexpr int ROWB = D * 2;                         // bytes per row in LDS (unpadded)
@@ -72,8 +72,10 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   const __amdgpu_buffer_rsrc_t vh = make_rsrc(v + head_off, head_bytes);
 
   // ---- the two look-up rows -> per-wave step lists
-  const size_t rowA = ((size_t)bh * Mblk + 2 * pj) * topk;
-  const size_t rowB = pair_full ? rowA + topk : rowA;
+  // (one_row: the pair is one 128-row query block of the caller's, whose look-up table has one row per pair: both
+  //  halves follow it, and every step is a shared one)
+  const size_t rowA = one_row ? ((size_t)bh * Mpair + pj) * topk : ((size_t)bh * Mblk + 2 * pj) * topk;
+  const size_t rowB = (pair_full && !one_row) ? rowA + topk : rowA;
   auto lut_at = [&](size_t i) __attribute__((always_inline)) -> int {       // (the low word of a 64-bit entry)
     return reinterpret_cast<const int*>(lut)[lut64 ? 2 * i : i];
   };

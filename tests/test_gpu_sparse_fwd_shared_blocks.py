@@ -124,3 +124,30 @@ def test_fused_linear_branch_on_a_split_pair(dev, dtype):
                                            want_o_s=True)
     assert max_abs(o_s.cpu(), o_s_ref) <= TOL_ABS
     assert max_abs(out.cpu(), ref) <= 3e-2 and cos_sim(out.cpu(), ref) >= TOL_COS
+
+
+@pytest.mark.parametrize("L", [1024,      # whole 128-row blocks
+                               1000,      # the last block's second half is ragged (and so is the last key block)
+                               960,       # the last block has no second half at all
+                               1217])
+def test_query_blocks_of_128_rows(dev, L):
+    """A 128-row query block goes through the same kernel as a pair of 64-row blocks whose two look-up rows are its one
+    row: against the oracle at BLOCK_M = 128 (the shape of the reference's evaluate/bench_kernel.py:60-61), and bit for
+    bit against the 64-row call with every row of the table written twice."""
+    T = 5
+    M, N = (L + 127) // 128, (L + 63) // 64
+    pairs_per_head = M
+    H = -(-512 // pairs_per_head)
+    g = torch.Generator().manual_seed(L)
+    q, k, v = _qkv(H, L, 200 + L)
+    lut = torch.stack([torch.stack([torch.randperm(N, generator=g)[:T] for _ in range(M)]) for _ in range(H)]).view(1, H, M, T)
+    o_ref, lse_ref = O.sparse_attn_fwd_gather(q, k, v, lut, 128, 64)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    o, lse = sparse_attn_fwd(qd, kd, vd, lut.to(dev), T, 128, 64, 128 ** -0.5)
+    assert torch.isfinite(o.float()).all()
+    assert max_abs(o.cpu(), o_ref) <= TOL_ABS and cos_sim(o.cpu(), o_ref) >= TOL_COS
+    assert max_abs(lse.cpu(), lse_ref) <= TOL_LSE
+    M64 = (L + 63) // 64
+    lut64 = lut.repeat_interleave(2, dim=2)[:, :, :M64].contiguous()
+    o2, lse2 = sparse_attn_fwd(qd, kd, vd, lut64.to(dev), T, 64, 64, 128 ** -0.5)
+    assert torch.equal(o, o2) and torch.equal(lse, lse2)
