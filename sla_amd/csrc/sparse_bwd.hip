@@ -685,7 +685,9 @@ static BwdWs bwd_ws(int BH, int L, int D, int BLKQ, int BLKK, int topk) {
   const int64_t entries = (int64_t)BH * M * topk;
   int64_t seg = (entries + 2047) / 2048;     // 512 resident workgroups, a quarter of the average each
   if (seg < 64) seg = 64;
-  if (seg > DKDV_STREAM_MAX_SEG) seg = DKDV_STREAM_MAX_SEG;      // (a work item's entries have to fit its LDS copy)
+  // (a work item's entries have to fit its LDS copy, which holds a 128-row query block as its two halves)
+  const int64_t seg_cap = BLKQ == 128 ? DKDV_STREAM_MAX_SEG / 2 : DKDV_STREAM_MAX_SEG;
+  if (seg > seg_cap) seg = seg_cap;
   w.seg = (int)seg;
   w.max_items = (int64_t)BH * N + entries / seg;
   w.max_slots = 2 * entries / seg;
@@ -729,10 +731,14 @@ static int bwd_impl(const void* q, const void* k, const void* v, const void* o, 
                        w.seg, (int)w.max_items, (int)w.max_slots);
   const int total_q = BH * Mblk;
   const bool contig = lin.sl == D && ldo.sl == D;
-  // head dim 128 with 64-row query blocks has a dK/dV kernel of its own (32-bit byte offsets inside a head)
-  const bool stream_dkdv = D == 128 && BLKQ == 64 && (uint64_t)lin.sl * 2u * (uint64_t)L < (1ull << 31) &&
+  // head dim 128 with 64-row query blocks has kernels of its own (32-bit byte offsets inside a head); a 128-row query
+  // block goes through them as its two halves (`wide`), which follow the block's row of the table and its list entries
+  const int wide = BLKQ == 128;
+  const int Mblk64 = cdiv(L, 64);
+  const int total_q64 = BH * Mblk64;
+  const bool stream_dkdv = D == 128 && (BLKQ == 64 || BLKQ == 128) && (uint64_t)lin.sl * 2u * (uint64_t)L < (1ull << 31) &&
                            (uint64_t)ldo.sl * 2u * (uint64_t)L < (1ull << 31);
-  const bool stream_dq = stream_dkdv && topk <= DQ_STREAM_MAX_T && total_q >= 1024;      // (enough query blocks for a wave on every SIMD)
+  const bool stream_dq = stream_dkdv && topk <= DQ_STREAM_MAX_T && total_q64 >= 1024;      // (enough query blocks for a wave on every SIMD)
   // delta = rowsum(dO * O): the dQ kernel of the common shape forms it for its own rows, the general one reads it
   if ((steps & SB_DQ) && !stream_dq)
     hipLaunchKernelGGL((bwd_delta_kernel<Tag, D>), dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, st,
@@ -740,9 +746,9 @@ static int bwd_impl(const void* q, const void* k, const void* v, const void* o, 
 #define SLA_BWD_LAUNCH(CONTIG)                                                                                              \
   if (!(steps & SB_DQ)) {                                                                                                   \
   } else if (stream_dq)                                                                                                     \
-    hipLaunchKernelGGL((bwd_dq_stream_kernel<Tag>), dim3(xcd_grid(total_q)), dim3(64), 0, st, (const uint16_t*)q,           \
+    hipLaunchKernelGGL((bwd_dq_stream_kernel<Tag>), dim3(xcd_grid(total_q64)), dim3(64), 0, st, (const uint16_t*)q,         \
                        (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, (const uint16_t*)o, lse, delta, lut,   \
-                       lut64, (uint16_t*)dq, lin, ldo, L, Mblk, topk, qk_scale, total_q);                                  \
+                       lut64, (uint16_t*)dq, lin, ldo, L, Mblk64, topk, qk_scale, total_q64, wide);                        \
   else                                                                                                                      \
     hipLaunchKernelGGL((bwd_dq_kernel<Tag, D, BLKQ, CONTIG>), dim3(xcd_grid(total_q)), dim3(BLKQ * 2), 0, st,               \
                        (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse, delta, lut,   \
@@ -751,7 +757,7 @@ static int bwd_impl(const void* q, const void* k, const void* v, const void* o, 
   } else if (stream_dkdv)                                                                                                   \
     hipLaunchKernelGGL((bwd_dkdv_stream_kernel<Tag>), dim3(xcd_grid(w.max_items)), dim3(128), 0, st, (const uint16_t*)q,    \
                        (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse, delta, list, count, items,       \
-                       totals, part, w.seg, (uint16_t*)dk, (uint16_t*)dv, lin, ldo, L, Mblk, Nblk, qk_scale);             \
+                       totals, part, w.seg, (uint16_t*)dk, (uint16_t*)dv, lin, ldo, L, Mblk, Nblk, qk_scale, wide);       \
   else                                                                                                                      \
     hipLaunchKernelGGL((bwd_dkdv_kernel<Tag, D, BLKQ, CONTIG>), dim3(xcd_grid(w.max_items)), dim3(256), 0, st,             \
                        (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)d_o, lse, delta, list,  \

@@ -41,7 +41,8 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     const uint16_t* __restrict__ d_o, const float* __restrict__ lse, const float* __restrict__ delta,
     const int* __restrict__ list, const int* __restrict__ count, const i32x4_t* __restrict__ items,
     const int* __restrict__ totals, float* __restrict__ part, int seg, uint16_t* __restrict__ dk, uint16_t* __restrict__ dv,
-    const RowLayout lin, const RowLayout ldo, int L, int Mblk, int Nblk, float qk_scale) {
+    const RowLayout lin, const RowLayout ldo, int L, int Mblk, int Nblk, float qk_scale, int wide) {
+  // (wide = 1: the lists name 128-row query blocks; an entry is then walked as its two 64-row halves)
   using E = Elem<Tag>;
   constexpr int D = 128, DC = D / 16, DT = D / 32;
   constexpr int ROWB = D * 2;               // bytes per row in LDS (unpadded)
@@ -85,7 +86,7 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   const int* mylist = list + ((size_t)bh * Nblk + nb) * Mblk;
   const int e0 = sg * seg;
   const int count_lane = count[(size_t)bh * Nblk + nb];
-  const int first_entry = mylist[min(e0 + tid, Mblk - 1)];
+  const int first_entry = mylist[min(e0 + (tid >> wide), Mblk - 1)];
   // K^T and V^T fragments (B operands): this lane's key column, 8 adjacent d per chunk; parked in accumulation registers
   const int krow = nb * 64 + w * 32 + r;
   const bool kok = krow < L;
@@ -112,12 +113,13 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 
   // this work item's part of the list, in units of 32 query rows (two per listed query block)
   const int e1 = min(__builtin_amdgcn_readfirstlane(count_lane), (sg + 1) * seg);
-  const int nunits = 2 * (e1 - e0);
+  const int nent = (e1 - e0) << wide;               // 64-row blocks this work item walks
+  const int nunits = 2 * nent;
   auto entry_row0 = [&](int e) __attribute__((always_inline)) -> int {          // past the end: the last entry again (fetched, never used)
-    return __builtin_amdgcn_readfirstlane(entries[min(e, e1 - e0 - 1)]) * 64;
+    return __builtin_amdgcn_readfirstlane(entries[min(e, nent - 1)]) * 64;
   };
-  if (tid < seg) entries[tid] = first_entry;
-  for (int i = 128 + tid; i < e1 - e0; i += 128) entries[i] = mylist[e0 + i];
+  if (tid < (seg << wide)) entries[tid] = (first_entry << wide) + (tid & wide);
+  for (int i = 128 + tid; i < nent; i += 128) entries[i] = (mylist[e0 + (i >> wide)] << wide) + (i & wide);
 
   // ---- addressing ----
   // A request moves 4 rows (64 lanes x 16 bytes): lane -> row 4j + lane / 16 of this wave's 16 rows, 16-byte slot
@@ -382,7 +384,8 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 1))) void
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ k, const uint16_t* __restrict__ v,
     const uint16_t* __restrict__ d_o, const uint16_t* __restrict__ o, const float* __restrict__ lse, float* __restrict__ delta,
     const void* __restrict__ lut, int lut64, uint16_t* __restrict__ dq, const RowLayout lin, const RowLayout ldo, int L,
-    int Mblk, int topk, float qk_scale, int total) {
+    int Mblk, int topk, float qk_scale, int total, int wide) {
+  // (Mblk: 64-row blocks per head.  wide = 1: the look-up table has one row per 128-row block, which both halves follow)
   using E = Elem<Tag>;
   constexpr int D = 128, DC = D / 16, DT = D / 32;
   constexpr int ROWB = D * 2;
@@ -409,7 +412,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 1))) void
 
   // The first 64 entries of the look-up row are asked for before anything else: the first requests for K and V hang on
   // them, and loads come back in the order they were issued (the low word of a 64-bit entry is the entry).
-  const size_t lut_row = ((size_t)bh * Mblk + mb) * topk;
+  const size_t lut_row = wide ? ((size_t)bh * ((Mblk + 1) >> 1) + (mb >> 1)) * topk : ((size_t)bh * Mblk + mb) * topk;
   auto lut_at = [&](size_t i) __attribute__((always_inline)) -> int { return reinterpret_cast<const int*>(lut)[lut64 ? 2 * i : i]; };
   int first_entries = 0;
   if (topk > 0) first_entries = lut_at(lut_row + min(lane, topk - 1));      // (an empty table may be a null pointer)

@@ -55,6 +55,25 @@ def test_many_query_blocks(dev, H, L, dtype, ratio):
         assert cos_sim(a, b) >= TOL_COS, name
 
 
+@pytest.mark.parametrize("H,L,dtype,ratio", [(64, 1024, torch.bfloat16, 0.25),   # whole 128-row blocks
+                                              (70, 970, torch.float16, 0.3),      # second half of the last block ragged
+                                              (68, 960, torch.bfloat16, 0.25)])   # last block without a second half
+def test_many_query_blocks_of_128_rows(dev, H, L, dtype, ratio):
+    """BLOCK_M = 128 (the reference's evaluate/bench_kernel.py:60-61) at the same launch sizes: the kernels above walk a
+    128-row query block as its two halves, both following the block's row of the table / its entry of the lists."""
+    g = torch.Generator().manual_seed(H + L + 1)
+    q, k, v, do = (torch.randn(1, H, L, 128, generator=g).to(dtype) for _ in range(4))
+    m, lut, T = O.get_block_map(q, k, ratio, 128, 64)
+    o_ref, lse_ref = O.sparse_attn_fwd_dense(q, k, v, m, 128, 64)
+    refs = O.sparse_attn_bwd_dense(q, k, v, o_ref, do, lse_ref, m, 128, 64)
+    o, dq, dk, dv = _grads(q, k, v, do, m, lut, T, 128, dev)
+    assert max_abs(o, o_ref) <= TOL_ABS
+    for name, a, b in zip(("dq", "dk", "dv"), (dq, dk, dv), refs):
+        assert torch.isfinite(a.float()).all(), name
+        assert max_abs(a, b) <= TOL_ABS, name
+        assert cos_sim(a, b) >= TOL_COS, name
+
+
 def test_full_selection_equals_sdpa_autograd(dev):
     g = torch.Generator().manual_seed(21)
     q, k, v, do = (torch.randn(2, 2, 300, 128, generator=g).to(torch.bfloat16) for _ in range(4))
