@@ -143,6 +143,17 @@ int sla_linear_state_fwd(const void* k, const void* v, const float* weight, int 
 int sla_linear_out_fwd(const void* q, const float* bias, const void* residual, void* out, int dtype, int fmap, int B,
                        int H, int L, int D, void* workspace, int64_t workspace_bytes, void* stream);
 
+/* sla_linear_state_fwd and sage_quant_v (further down) in one call, for the quantised module, which needs both of the
+ * same v: the state kernel streams v anyway and leaves the largest |v| of every column, so the quantiser's own pass over
+ * v for them is not made.  workspace (SLA_WS_LINEAR_FWD), v_fp8, v_scale, v_range as in the two calls; the results equal
+ * theirs bit for bit.  Kernels on `stream` in the order: states per slice of the sequence, scale, FP8 copy of v, sum of
+ * the slices, projection folded in.
+ * Replaces core.py:90-95 of sparse_linear_attention (feature map of k, calc_linear's k^T v and k sum) and
+ * SageSLA/core.py:127-129 (per-channel FP8 quantisation of v). */
+int sla_linear_state_quant_v_fwd(const void* k, const void* v, const float* weight, int dtype, int fmap, int B, int H,
+                                 int L, int D, void* workspace, int64_t workspace_bytes, uint8_t* v_fp8, float* v_scale,
+                                 float v_range, void* stream);
+
 /* For callers whose activations are not laid out as contiguous (B, H, L, D): strided variants of the calls that
  * touch q, k, v, out and their gradients.  `*_strides` = {batch, head, row} strides in
  * elements of a tensor indexed (b, h, l, d) whose last dimension is contiguous: {H*L*D, L*D, D} for the
@@ -158,6 +169,10 @@ int sla_block_map_fwd_strided(const void* q, const void* k, const int64_t* qk_st
 int sla_linear_state_fwd_strided(const void* k, const void* v, const int64_t* kv_strides, const float* weight, int dtype,
                                  int fmap, int B, int H, int L, int D, void* workspace, int64_t workspace_bytes,
                                  void* stream);
+int sla_linear_state_quant_v_fwd_strided(const void* k, const void* v, const int64_t* kv_strides, const float* weight,
+                                         int dtype, int fmap, int B, int H, int L, int D, void* workspace,
+                                         int64_t workspace_bytes, uint8_t* v_fp8, float* v_scale, float v_range,
+                                         void* stream);
 /* The two backward calls with strides: q, k, v, dq, dk, dv share `qkv_strides` (e.g. slices of one packed
  * (B, L, 3, H, D) buffer and of its gradient), d_o / d_out has `do_strides`; o (the saved o_s), lse and the
  * workspaces are contiguous as in the calls without the suffix. */

@@ -35,6 +35,8 @@ SIGNATURES = {
     "sla_block_map_fwd_static": (_I, [_P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _I, _P]),
     "sla_block_map_fwd_strided": (_I, [_P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _I64, _P, _P, _I, _P]),
     "sla_linear_state_fwd_strided": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I64, _P]),
+    "sla_linear_state_quant_v_fwd": (_I, [_P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I64, _P, _P, _F, _P]),
+    "sla_linear_state_quant_v_fwd_strided": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I64, _P, _P, _F, _P]),
     "sla_sparse_attn_linear_fwd_strided": (_I, [_P, _P, _P, _P, _P, _I, _P, _I64, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I,
                                                 _I, _I, _I, _I, _F, _P]),
     "sla_sparse_attn_bwd_strided": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I,

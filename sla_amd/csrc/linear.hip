@@ -17,6 +17,7 @@
 //                   per-query divisor is a per-lane scalar; the tile is scaled, biased, parked in LDS
 //                   and written (plus the residual) with whole-row 16-byte accesses.
 #include "linear_state.h"
+#include "sage_steps.h"
 
 namespace sla {
 
@@ -135,6 +136,27 @@ static int linear_state_impl(const void* k, const void* v, const RowLayout& lay,
   return check_launch("linear_state_fwd");
 }
 
+// The same with v quantised to FP8 on the way: the state kernel, which streams v anyway, leaves the column maxima of
+// |v| per slice, so that the quantiser's own pass over v for them is not needed; the scale and the FP8 copy of v come
+// right behind the state kernel, the small kernels that finish the states after them.
+template <typename Tag, int D>
+static int linear_state_quant_v_impl(const void* k, const void* v, const RowLayout& lay, const float* weight, int dtype, int fmap,
+                                     int BH, int L, char* ws, uint8_t* v_fp8, float* v_scale, float v_range, hipStream_t st) {
+  const LinWs w = lin_ws(BH, L, D);
+  hipLaunchKernelGGL((linear_state_partial_kernel<Tag, D, false, false, true>), dim3(w.nsplit, BH), dim3(256), 0, st,
+                     (const uint16_t*)k, (const uint16_t*)v, lay, (float*)(ws + w.kv_part), (float*)(ws + w.z_part), L,
+                     w.rows_per_split, fmap, (const float*)nullptr, (float*)(ws + w.vmax_part));
+  int rc = quant_v_from_partial_amax(v, lay, dtype, BH, L, D, (const float*)(ws + w.vmax_part), w.nsplit, v_fp8, v_scale,
+                                     v_range, st);
+  if (rc) return rc;
+  hipLaunchKernelGGL((linear_state_reduce_kernel<Tag>), dim3(cdiv(D * D, 256), BH), dim3(256), 0, st,
+                     (const float*)(ws + w.kv_part), (const float*)(ws + w.z_part), (uint16_t*)(ws + w.kvt),
+                     (uint16_t*)(ws + w.kvp), (uint16_t*)(ws + w.z), w.nsplit, D * D, D);
+  hipLaunchKernelGGL((linear_fold_kernel<Tag>), dim3(D / (1024 / D), BH), dim3(256), 0, st,
+                     (const uint16_t*)(ws + w.kvt), weight, (uint16_t*)(ws + w.kvwt), (uint16_t*)(ws + w.wt), D);
+  return check_launch("linear_state_quant_v_fwd");
+}
+
 template <typename Tag, int D>
 static int linear_out_impl(const void* q, const RowLayout& lq, const float* bias, const void* residual, void* out,
                            const RowLayout& lout, int fmap, int BH, int L, char* ws, hipStream_t st) {
@@ -210,6 +232,51 @@ extern "C" int sla_linear_state_fwd_strided(const void* k, const void* v, const 
                                             int64_t workspace_bytes, void* stream) {
   SLA_REQUIRE(kv_strides, SLA_ERR_BAD_ARG, "null strides");
   return linear_state_entry(k, v, kv_strides, weight, dtype, fmap, B, H, L, D, workspace, workspace_bytes, stream);
+}
+
+static int linear_state_quant_v_entry(const void* k, const void* v, const int64_t* strides, const float* weight, int dtype,
+                                      int fmap, int B, int H, int L, int D, void* workspace, int64_t workspace_bytes,
+                                      uint8_t* v_fp8, float* v_scale, float v_range, void* stream) {
+  int rc = validate_linear(dtype, fmap, B, H, L, D);
+  if (rc) return rc;
+  rc = validate_v_range(v_range);
+  if (rc) return rc;
+  SLA_REQUIRE(k && v && weight && v_fp8 && v_scale, SLA_ERR_BAD_ARG, "null pointer");
+  SLA_REQUIRE(((uintptr_t)k | (uintptr_t)v | (uintptr_t)weight | (uintptr_t)v_fp8) % 16 == 0, SLA_ERR_BAD_ARG,
+              "pointers must be 16-byte aligned");
+  const int BH = B * H;
+  rc = check_linear_ws(BH, L, D, workspace, workspace_bytes);
+  if (rc) return rc;
+  RowLayout lay;
+  rc = make_layout(strides, B, H, L, D, 2, &lay);
+  if (rc) return rc;
+  hipStream_t st = (hipStream_t)stream;
+  char* ws = (char*)workspace;
+#define SLA_LIN_CASE(TAG, DD) \
+  return linear_state_quant_v_impl<TAG, DD>(k, v, lay, weight, dtype, fmap, BH, L, ws, v_fp8, v_scale, v_range, st)
+  if (dtype == SLA_BF16) {
+    if (D == 128) SLA_LIN_CASE(bf16_tag, 128);
+    SLA_LIN_CASE(bf16_tag, 64);
+  }
+  if (D == 128) SLA_LIN_CASE(f16_tag, 128);
+  SLA_LIN_CASE(f16_tag, 64);
+#undef SLA_LIN_CASE
+}
+
+extern "C" int sla_linear_state_quant_v_fwd(const void* k, const void* v, const float* weight, int dtype, int fmap, int B,
+                                            int H, int L, int D, void* workspace, int64_t workspace_bytes, uint8_t* v_fp8,
+                                            float* v_scale, float v_range, void* stream) {
+  return linear_state_quant_v_entry(k, v, nullptr, weight, dtype, fmap, B, H, L, D, workspace, workspace_bytes, v_fp8, v_scale,
+                                    v_range, stream);
+}
+
+extern "C" int sla_linear_state_quant_v_fwd_strided(const void* k, const void* v, const int64_t* kv_strides,
+                                                    const float* weight, int dtype, int fmap, int B, int H, int L, int D,
+                                                    void* workspace, int64_t workspace_bytes, uint8_t* v_fp8,
+                                                    float* v_scale, float v_range, void* stream) {
+  SLA_REQUIRE(kv_strides, SLA_ERR_BAD_ARG, "null strides");
+  return linear_state_quant_v_entry(k, v, kv_strides, weight, dtype, fmap, B, H, L, D, workspace, workspace_bytes, v_fp8,
+                                    v_scale, v_range, stream);
 }
 
 static int linear_out_entry(const void* q, const int64_t* q_strides, const float* bias, const void* residual, void* out,

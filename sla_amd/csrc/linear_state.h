@@ -9,12 +9,15 @@ namespace sla {
 // OUT16: the D x D partial is written rounded to 16 bit (per-key-block states of the complement mode).
 // ZW: zweight holds one fp32 per row of the head, (BH, L), and the z partial becomes sum_rows zweight * phi(k)
 // instead of sum_rows phi(k) (used by the complement backward, where "k" is q and "v" a row gradient).
-template <typename Tag, int D, bool OUT16 = false, bool ZW = false>
+// VMAX: the largest |v| of every column over the slice goes to vmax_part[bh][split][D] (what the FP8 quantiser of v
+// needs of v before it can start: v is streamed here anyway).
+template <typename Tag, int D, bool OUT16 = false, bool ZW = false, bool VMAX = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void linear_state_partial_kernel(const uint16_t* __restrict__ k,
                                                                    const uint16_t* __restrict__ v, const RowLayout lay,
                                                                    void* __restrict__ kv_part_, float* __restrict__ z_part,
                                                                    int L, int rows_per_split, int fmap,
-                                                                   const float* __restrict__ zweight = nullptr) {
+                                                                   const float* __restrict__ zweight = nullptr,
+                                                                   float* __restrict__ vmax_part = nullptr) {
   using E = Elem<Tag>;
   constexpr int TR = 64;                 // rows per LDS tile
   constexpr int STR = D + 16;            // LDS row stride: transposed reads of 4 rows hit disjoint banks
@@ -49,6 +52,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
   float zacc[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) zacc[e] = 0.f;
+  // |v| of this thread's eight columns as 16-bit patterns without their sign bits: for bf16 and f16 alike the larger
+  // magnitude has the larger pattern, so a packed unsigned maximum keeps two columns per register
+  typedef unsigned short u16x2_t __attribute__((ext_vector_type(2)));
+  u16x2_t vmx[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) vmx[j] = u16x2_t{0, 0};
 
   const int tr_row = (lane & 15) >> 2;
   const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
@@ -116,6 +125,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
       }
       *reinterpret_cast<i16x8_t*>(&sK[row * STR + lcol]) = fk;
       *reinterpret_cast<i16x8_t*>(&sV[row * STR + lcol]) = vv;
+      if (VMAX) {                          // (rows past the end were fetched as zeros)
+        const i32x4_t vw = __builtin_bit_cast(i32x4_t, vv);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          vmx[j] = __builtin_elementwise_max(vmx[j], __builtin_bit_cast(u16x2_t, vw[j] & 0x7fff7fff));
+      }
     }
     __syncthreads();
     if (r0 + TR < row_end) fetch(r0 + TR);     // after the barrier: its fence would wait for these loads
@@ -166,6 +181,21 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
 #pragma unroll
     for (int r = 0; r < RPP; ++r) s += sZ[r][tid];
     z_part[((size_t)bh * nsplit + split) * D + tid] = s;
+  }
+  if (VMAX) {
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      sZ[lrow][lcol + 2 * j] = E::to_float(vmx[j][0]);
+      sZ[lrow][lcol + 2 * j + 1] = E::to_float(vmx[j][1]);
+    }
+    __syncthreads();
+    if (tid < D) {
+      float a = 0.f;
+#pragma unroll
+      for (int r = 0; r < RPP; ++r) a = fmaxf(a, sZ[r][tid]);
+      vmax_part[((size_t)bh * nsplit + split) * D + tid] = a;
+    }
   }
 }
 
@@ -269,7 +299,7 @@ __global__ __launch_bounds__(256) void linear_fold_kernel(const uint16_t* __rest
 // forward and put back at the start of the backward's workspace instead of having them rebuilt.
 struct LinWs {
   int nsplit, rows_per_split;
-  size_t kvt, kvp, kvwt, z, wt, states_end, kv_part, z_part, total;
+  size_t kvt, kvp, kvwt, z, wt, states_end, kv_part, z_part, vmax_part, total;
 };
 
 static inline LinWs lin_ws(int BH, int L, int D) {
@@ -289,6 +319,7 @@ static inline LinWs lin_ws(int BH, int L, int D) {
   w.states_end = off;
   w.kv_part = off; off += align_up((int64_t)BH * w.nsplit * D * D * 4, 256);
   w.z_part = off;  off += align_up((int64_t)BH * w.nsplit * D * 4, 256);
+  w.vmax_part = off; off += align_up((int64_t)BH * w.nsplit * D * 4, 256);      // (filled on request: column maxima of |v| per slice)
   w.total = off;
   return w;
 }

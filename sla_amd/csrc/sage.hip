@@ -11,6 +11,7 @@
 //   O = (e4m3(c P) . v_fp8) * sv / sum(e4m3(c P)), c = 112 with P <= 4 (reference maximum lagging by <= 2).
 // The look-up table of the bf16 path is used as is (no delta encoding is needed here).
 #include "common.h"
+#include "sage_steps.h"
 
 namespace sla {
 
@@ -505,7 +506,7 @@ static int validate_sage(int dtype, int B, int H, int L, int D, int BLKQ, int BL
 }
 
 // range of the e4m3 values v is quantised to: the format's largest finite value (448) or less
-static int validate_v_range(float v_range) {
+int validate_v_range(float v_range) {
   SLA_REQUIRE(v_range > 0.f && v_range <= 448.f, SLA_ERR_BAD_ARG, "v_range=%g outside (0, 448]", (double)v_range);
   return SLA_OK;
 }
@@ -565,6 +566,23 @@ static int quant_v_impl(const void* v, const RowLayout& lay, int BH, int L, uint
   hipLaunchKernelGGL((v_quant_fp8_kernel<Tag, D>), dim3(cdiv(L, RPP), BH), dim3(256), 0, st, (const uint16_t*)v, lay, vs, v8,
                      L);
   return check_launch("sage_quant_v");
+}
+
+int quant_v_from_partial_amax(const void* v, const RowLayout& lay, int dtype, int BH, int L, int D, const float* part,
+                              int nparts, uint8_t* v8, float* vs, float v_range, hipStream_t st) {
+  hipLaunchKernelGGL(v_scale_kernel, dim3(D / 16, BH), dim3(256), 0, st, part, vs, nparts, D, v_range);
+#define SAGE_VQ_CASE(TAG, DD)                                                                                         \
+  hipLaunchKernelGGL((v_quant_fp8_kernel<TAG, DD>), dim3(cdiv(L, 256 / (DD / 8)), BH), dim3(256), 0, st, (const uint16_t*)v, \
+                     lay, vs, v8, L)
+  if (dtype == SLA_BF16) {
+    if (D == 128) SAGE_VQ_CASE(bf16_tag, 128);
+    else SAGE_VQ_CASE(bf16_tag, 64);
+  } else {
+    if (D == 128) SAGE_VQ_CASE(f16_tag, 128);
+    else SAGE_VQ_CASE(f16_tag, 64);
+  }
+#undef SAGE_VQ_CASE
+  return check_launch("linear_state_quant_v");
 }
 
 }  // namespace sla

@@ -43,6 +43,31 @@ def linear_state_fwd(k, v, weight, fmap: str):
     return ws
 
 
+def linear_state_quant_v_fwd(k, v, weight, fmap: str, v_range: float = 448.0):
+    """:func:`linear_state_fwd` and the per-channel FP8 quantisation of ``v`` (``sage.quant_v``) in one library call:
+    the state kernel streams ``v`` anyway and leaves the column maxima the quantiser needs, which spares the
+    quantiser's own pass over ``v`` for them.  Returns ``(workspace, v_fp8, v_scale)``, bit for bit what the two
+    calls return."""
+    _lib.require_gpu(k, v, weight)
+    B, H, L, D = k.shape
+    dt = _lib.dtype_code(k.dtype)
+    ws = _lib.workspace(_lib.WS_LINEAR_FWD, dt, B, H, L, D, 64, 64, 0, k.device)
+    v8 = torch.empty((B, H, L, D), dtype=torch.float8_e4m3fn, device=v.device)
+    vs = torch.empty((B, H, D), dtype=torch.float32, device=v.device)
+    if k.is_contiguous() and v.is_contiguous():
+        rc = _lib.load().sla_linear_state_quant_v_fwd(k.data_ptr(), v.data_ptr(), weight.data_ptr(), dt, _lib.FMAP[fmap], B,
+                                                      H, L, D, ws.data_ptr(), ws.numel(), v8.data_ptr(), vs.data_ptr(),
+                                                      float(v_range), _lib.stream_ptr(k.device))
+    else:
+        assert _lib.row_strided(k, v), "k and v must be contiguous or share row-contiguous strides"
+        rc = _lib.load().sla_linear_state_quant_v_fwd_strided(k.data_ptr(), v.data_ptr(), _lib.strides_arg(k),
+                                                              weight.data_ptr(), dt, _lib.FMAP[fmap], B, H, L, D,
+                                                              ws.data_ptr(), ws.numel(), v8.data_ptr(), vs.data_ptr(),
+                                                              float(v_range), _lib.stream_ptr(k.device))
+    _lib.check(rc)
+    return ws, v8, vs
+
+
 def linear_out_fwd(q, bias, residual, state_ws, fmap: str):
     """Second half of :func:`linear_fwd`: ``residual + proj(phi(q) state / divisor)``.
 

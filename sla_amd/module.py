@@ -7,7 +7,7 @@ import torch.nn as nn
 
 from . import _lib
 from .block_map import get_block_map
-from .linear import linear_complement_bwd, linear_complement_fwd, linear_state_fwd, saved_states
+from .linear import linear_complement_bwd, linear_complement_fwd, linear_state_fwd, linear_state_quant_v_fwd, saved_states
 from .sparse_attn import sparse_attn_bwd, sparse_attn_fwd, sparse_attn_linear_fwd
 
 FEATURE_MAPS = ("elu", "relu", "softmax")
@@ -178,8 +178,18 @@ class _StateBuild:
 
     _side = {}
 
-    def __init__(self, k, v, weight, fmap):
+    def __init__(self, k, v, weight, fmap, quant_v_range=None):
+        """``quant_v_range``: also quantise ``v`` to FP8 with that range in the same library call (``self.v_fp8``,
+        ``self.v_scale``, ready after ``join``)."""
         dev = k.device
+        self.v_fp8 = self.v_scale = None
+
+        def build():
+            if quant_v_range is None:
+                self.ws = linear_state_fwd(k, v, weight, fmap)
+            else:
+                self.ws, self.v_fp8, self.v_scale = linear_state_quant_v_fwd(k, v, weight, fmap, quant_v_range)
+
         cur = torch.cuda.current_stream(dev)
         if torch.cuda.is_current_stream_capturing():
             side = None          # inside a graph capture the work stays on the capturing stream
@@ -189,11 +199,14 @@ class _StateBuild:
                 side = self._side[dev.index] = torch.cuda.Stream(device=dev)
         self.side = side
         if side is None:
-            self.ws = linear_state_fwd(k, v, weight, fmap)
+            build()
             return
         side.wait_stream(cur)    # k, v and the weight were produced on the calling stream
         with torch.cuda.stream(side):
-            self.ws = linear_state_fwd(k, v, weight, fmap)
+            build()
+        for t in (self.v_fp8, self.v_scale):
+            if t is not None:
+                t.record_stream(cur)         # allocated under the side stream, consumed on the calling one
 
     def also(self, fn, *args):
         """Runs ``fn(*args)`` behind the state build, on the same side stream; its results are ready after ``join``."""

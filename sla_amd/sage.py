@@ -160,10 +160,10 @@ class SageSparseLinearAttention(nn.Module):
         # The k/v half of the linear branch runs on a side stream beside the preparation and the attention
         # kernel (measured best when started first: 0.570 against 0.593 ms serial at H12 L32760).
         if q.dtype == k.dtype == v.dtype == self.dtype:
-            state = _StateBuild(k, v, self.proj_l.weight, self.feature_map)
-            # v, which neither the mask nor the q / k quantisers need, is quantised behind the state build on the side
-            # stream (0.557 against 0.568 ms at H12 L32760)
-            v8, vs = state.also(quant_v, v)
+            # v, which neither the mask nor the q / k quantisers need, is quantised with the state build on the side
+            # stream: the state kernel streams v anyway and finds the column maxima the quantiser starts from
+            state = _StateBuild(k, v, self.proj_l.weight, self.feature_map, quant_v_range=V_RANGE_E4M3)
+            v8, vs = state.v_fp8, state.v_scale
             # the mask sees the same values as the quantisers: one pass structure for both
             sparse_map, lut, real_topk, q8, qs, k8, ks, _, _ = sage_prepare(q, k, None, self.topk)
             state.join()

@@ -90,6 +90,15 @@ def test_other_entry_points_validate():
     assert need > lib.sla_workspace_bytes(_lib.WS_LINEAR_COMPLEMENT, 1, 1, 2, 128, 128, 64, 64, 1) > 0
     assert lib.sla_linear_state_fwd(FAKE, FAKE, FAKE, 1, 0, 1, 1, 64, 128, FAKE, 8, None) == _lib.ERR_WORKSPACE
     assert lib.sla_linear_state_fwd(FAKE, None, FAKE, 1, 0, 1, 1, 64, 128, FAKE, 1 << 30, None) == _lib.ERR_BAD_ARG
+    # the state build with the FP8 quantisation of v in the same call: the checks of both
+    sq = lib.sla_linear_state_quant_v_fwd
+    assert sq(FAKE, FAKE, FAKE, 1, 0, 1, 1, 64, 128, FAKE, 8, FAKE, FAKE, 448.0, None) == _lib.ERR_WORKSPACE
+    assert sq(FAKE, FAKE, FAKE, 1, 0, 1, 1, 64, 128, FAKE, 1 << 30, None, FAKE, 448.0, None) == _lib.ERR_BAD_ARG
+    assert sq(FAKE, FAKE, FAKE, 1, 0, 1, 1, 64, 128, FAKE, 1 << 30, FAKE, FAKE, 449.0, None) == _lib.ERR_BAD_ARG
+    assert "v_range" in _lib.last_error()
+    assert sq(FAKE, FAKE, FAKE, 1, 7, 1, 1, 64, 128, FAKE, 1 << 30, FAKE, FAKE, 448.0, None) == _lib.ERR_BAD_ARG
+    assert lib.sla_linear_state_quant_v_fwd_strided(FAKE, FAKE, None, FAKE, 1, 0, 1, 1, 64, 128, FAKE, 1 << 30, FAKE, FAKE,
+                                                    448.0, None) == _lib.ERR_BAD_ARG
     assert lib.sla_linear_out_fwd(FAKE, FAKE, None, FAKE, 0, 0, 1, 1, 64, 128, FAKE, 1 << 30, None) == _lib.ERR_UNSUPPORTED
     assert lib.sla_linear_out_fwd(FAKE, FAKE, None, FAKE, 1, 0, 1, 1, 64, 128, None, 1 << 30, None) == _lib.ERR_BAD_ARG
     assert lib.sla_linear_bwd(FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, 1, 0, 1, 1, 64, 128, 0, FAKE,

@@ -80,6 +80,32 @@ def test_one_call_preparation_equals_the_separate_calls(dev, L, D, ratio, dtype)
     assert torch.equal(v8.view(torch.uint8), v8b.view(torch.uint8)) and torch.equal(vs, vsb)
 
 
+@pytest.mark.parametrize("L,D,dtype,fmap,v_range", [(512, 128, torch.bfloat16, "softmax", 448.0), (1000, 128, torch.bfloat16, "elu", 2.25),
+                                                    (333, 64, torch.float16, "relu", 448.0), (4100, 128, torch.float16, "elu", 448.0)])
+def test_state_build_with_v_quantised_in_the_same_call(dev, L, D, dtype, fmap, v_range):
+    """The state kernel's column maxima of |v| instead of the quantiser's own pass over v: the states, the FP8 copy of v
+    and its scales are bit for bit those of the two separate calls (and so of the oracle's quantiser), also on a
+    (B, L, H, D) activation read in place."""
+    from sla_amd.linear import linear_out_fwd, linear_state_fwd, linear_state_quant_v_fwd
+    q, k, v = (x.to(dtype) for x in _qkv(L, D, 11 * L + D))
+    v = v * torch.logspace(-2, 1, D).to(dtype)            # channels of very different size
+    w, b = make_proj(D)
+    qd, kd, vd, wd, bd = q.to(dev), k.to(dev), v.to(dev), w.to(dev), b.to(dev)
+    ws_ref = linear_state_fwd(kd, vd, wd, fmap)
+    out_ref = linear_out_fwd(qd, bd, None, ws_ref, fmap)
+    v8_ref, vs_ref = quant_v(vd, v_range)
+    ws, v8, vs = linear_state_quant_v_fwd(kd, vd, wd, fmap, v_range)
+    assert torch.equal(vs, vs_ref) and torch.equal(v8.view(torch.uint8), v8_ref.view(torch.uint8))
+    assert torch.equal(linear_out_fwd(qd, bd, None, ws, fmap), out_ref)          # (the states, through what reads them)
+    v8o, vso = O.sage_quant_v(v, v_range)
+    assert torch.equal(vs.cpu(), vso) and torch.equal(v8.cpu().view(torch.uint8), v8o.view(torch.uint8))
+    # rows as they lie in a (B, L, H, D) activation
+    kt, vt = (x.transpose(1, 2).contiguous().transpose(1, 2) for x in (kd, vd))
+    ws2, v82, vs2 = linear_state_quant_v_fwd(kt, vt, wd, fmap, v_range)
+    assert torch.equal(vs2, vs_ref) and torch.equal(v82.view(torch.uint8), v8_ref.view(torch.uint8))
+    assert torch.equal(linear_out_fwd(qd, bd, None, ws2, fmap), out_ref)
+
+
 @pytest.mark.parametrize("L,D,ratio", [(512, 128, 0.5), (1000, 128, 0.3), (333, 64, 0.5), (2048, 128, 0.1)])
 def test_attention_vs_fp32_and_vs_quantised_oracle(dev, L, D, ratio):
     q, k, v = _qkv(L, D, L + 1)
