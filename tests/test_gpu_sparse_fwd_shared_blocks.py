@@ -151,3 +151,15 @@ def test_query_blocks_of_128_rows(dev, L):
     lut64 = lut.repeat_interleave(2, dim=2)[:, :, :M64].contiguous()
     o2, lse2 = sparse_attn_fwd(qd, kd, vd, lut64.to(dev), T, 64, 64, 128 ** -0.5)
     assert torch.equal(o, o2) and torch.equal(lse, lse2)
+    # the same with the linear branch in the epilogue
+    from sla_amd.inputs import make_proj
+    from sla_amd.linear import linear_state_fwd
+    from sla_amd.sparse_attn import sparse_attn_linear_fwd
+    w, b = make_proj(128)
+    ws = linear_state_fwd(kd, vd, w.to(dev), "elu")
+    out, o_s, lse3 = sparse_attn_linear_fwd(qd, kd, vd, lut.to(dev), T, 128, 64, 128 ** -0.5, ws, b.to(dev), "elu", want_o_s=True)
+    out2, o_s2, lse4 = sparse_attn_linear_fwd(qd, kd, vd, lut64.to(dev), T, 64, 64, 128 ** -0.5, ws, b.to(dev), "elu", want_o_s=True)
+    assert torch.equal(o_s, o) and torch.equal(lse3, lse)
+    assert torch.equal(out, out2) and torch.equal(o_s, o_s2) and torch.equal(lse3, lse4)
+    ref = o_ref + O.linear_branch(q, k, v, w, b, "elu", torch.bfloat16).float()
+    assert max_abs(out.cpu(), ref) <= 3e-2 and cos_sim(out.cpu(), ref) >= TOL_COS
