@@ -280,18 +280,22 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     l_run[qt] *= f;
     // The output accumulators live in the accumulation registers and, on the common path, are only ever touched by
     // MFMAs.  They are scaled in place through one temporary, so that the register allocator has no reason to
-    // move the whole accumulator through the vector registers around the loop.
+    // move the whole accumulator through the vector registers around the loop.  (Not on the first unit, which every
+    // wave sends through here to set its reference: nothing has been accumulated yet, and 64 registers times zero
+    // would be 200 instructions for nothing.)
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");     // (the last products into these registers and into sn have landed)
+    if (!first) {
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
+      for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        float x = oacc[dt][qt][i], t;
-        asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 %0, %1"
-                     : "+a"(x), "=&v"(t)
-                     : "v"(f));
-        oacc[dt][qt][i] = x;
-      }
+        for (int i = 0; i < 16; ++i) {
+          float x = oacc[dt][qt][i], t;
+          asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 %0, %1"
+                       : "+a"(x), "=&v"(t)
+                       : "v"(f));
+          oacc[dt][qt][i] = x;
+        }
+    }
     const float nm = -m_used[qt];
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
