@@ -81,60 +81,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     if (residual) res.fetch(residual + off, rows_valid, lane);
     if (tt + 1 < tiles_per_wg && row0 + 128 < L)
       qt.fetch(qh + (size_t)(row0 + 128) * pitch_q, min(32, L - row0 - 128), lane, pitch_q);
-    // divisor: 1e-5 + sum_d round16(fq*z), each step rounded to 16 bit as the reference's tensors are.  Values are
-    // rounded two at a time (one packing conversion for two) and taken apart again where the arithmetic goes on in fp32;
-    // a packed pair of phi(q) is a register of the B operand.
-    float den = 0.f;
+    // divisor: 1e-5 + sum_d round16(fq*z), each step rounded to 16 bit as the reference's tensors are
     i16x8_t qf[DC];
-    auto pair_done = [&](int c, int j2, float v0, float v1, i32x4_t& pw) __attribute__((always_inline)) {
-      float g0, g1, p0, p1;
-      pw[j2] = (int)round16_pair<Tag>(v0, v1, g0, g1);
-      round16_pair<Tag>(g0 * sZ[16 * c + 8 * g + 2 * j2], g1 * sZ[16 * c + 8 * g + 2 * j2 + 1], p0, p1);
-      den += p0;
-      den += p1;
-    };
-    if (fmap == SLA_FMAP_SOFTMAX) {
-      float f[DC][8];
-#pragma unroll
-      for (int c = 0; c < DC; ++c)
-#pragma unroll
-        for (int j = 0; j < 8; ++j) f[c][j] = E::to_float((uint16_t)xq[c][j]);
-      float row_mx, row_inv;
-      phi_row_pair<Tag, DC>(fmap, f, row_mx, row_inv);
-#pragma unroll
-      for (int c = 0; c < DC; ++c) {
-        i32x4_t pw;
-#pragma unroll
-        for (int j2 = 0; j2 < 4; ++j2) pair_done(c, j2, f[c][2 * j2], f[c][2 * j2 + 1], pw);
-        qf[c] = __builtin_bit_cast(i16x8_t, pw);
-      }
-    } else if (fmap == SLA_FMAP_RELU) {
-      // (the choice of the map stays outside the loops over the elements)
-#pragma unroll
-      for (int c = 0; c < DC; ++c) {
-        i32x4_t pw;
-#pragma unroll
-        for (int j2 = 0; j2 < 4; ++j2) {
-          const uint32_t xx = (uint32_t)__builtin_bit_cast(i32x4_t, xq[c])[j2];
-          pair_done(c, j2, fmaxf(E::to_float((uint16_t)(xx & 0xffffu)), 0.f), fmaxf(E::to_float((uint16_t)(xx >> 16)), 0.f), pw);
-        }
-        qf[c] = __builtin_bit_cast(i16x8_t, pw);
-      }
-    } else {
-#pragma unroll
-      for (int c = 0; c < DC; ++c) {
-        i32x4_t pw;
-#pragma unroll
-        for (int j2 = 0; j2 < 4; ++j2) {
-          const uint32_t xx = (uint32_t)__builtin_bit_cast(i32x4_t, xq[c])[j2];
-          const float x0 = E::to_float((uint16_t)(xx & 0xffffu)), x1 = E::to_float((uint16_t)(xx >> 16));
-          float e0, e1;                                    // elu, rounded; then + 1, rounded by pair_done
-          round16_pair<Tag>(x0 > 0.f ? x0 : (__expf(x0) - 1.0f), x1 > 0.f ? x1 : (__expf(x1) - 1.0f), e0, e1);
-          pair_done(c, j2, e0 + 1.0f, e1 + 1.0f, pw);
-        }
-        qf[c] = __builtin_bit_cast(i16x8_t, pw);
-      }
-    }
+    float den = phi_pack_den<Tag, DC>(fmap, xq, qf, [&](int c, int j) { return sZ[16 * c + 8 * g + j]; });
     den += __shfl_xor(den, 32);
     den = round16<Tag>(1e-5f + round16<Tag>(den));
     const float inv_den = 1.0f / den;

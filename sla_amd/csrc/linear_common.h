@@ -69,6 +69,67 @@ static __device__ __forceinline__ void phi_row_pair(int fmap, float (&f)[DC][8],
   }
 }
 
+// phi of a row whose raw 16-bit values are split between lane (xq: DC chunks of 8) and lane^32, packed to 16 bit in `qf`
+// (a packed pair is a register of an MFMA B operand), and this lane's part of the divisor's sum,
+// sum_d round16(phi_d * z_d), z_d = zat(c, j) for element j of chunk c.  Values the reference rounds to 16 bit are rounded
+// two at a time (one packing conversion for two) and taken apart again where the arithmetic goes on in fp32; the sum runs
+// over the elements in ascending order.  The pointwise maps never hold the row as 64 floats.
+template <typename Tag, int DC, typename ZAt>
+static __device__ __forceinline__ float phi_pack_den(int fmap, const i16x8_t (&xq)[DC], i16x8_t (&qf)[DC], ZAt zat) {
+  using E = Elem<Tag>;
+  float den = 0.f;
+  auto pair_done = [&](int c, int j2, float v0, float v1, i32x4_t& pw) __attribute__((always_inline)) {
+    float g0, g1, p0, p1;
+    pw[j2] = (int)round16_pair<Tag>(v0, v1, g0, g1);
+    round16_pair<Tag>(g0 * zat(c, 2 * j2), g1 * zat(c, 2 * j2 + 1), p0, p1);
+    den += p0;
+    den += p1;
+  };
+  if (fmap == SLA_FMAP_SOFTMAX) {
+    float f[DC][8];
+#pragma unroll
+    for (int c = 0; c < DC; ++c)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) f[c][j] = E::to_float((uint16_t)xq[c][j]);
+    float row_mx, row_inv;
+    phi_row_pair<Tag, DC>(fmap, f, row_mx, row_inv);
+#pragma unroll
+    for (int c = 0; c < DC; ++c) {
+      i32x4_t pw;
+#pragma unroll
+      for (int j2 = 0; j2 < 4; ++j2) pair_done(c, j2, f[c][2 * j2], f[c][2 * j2 + 1], pw);
+      qf[c] = __builtin_bit_cast(i16x8_t, pw);
+    }
+  } else if (fmap == SLA_FMAP_RELU) {
+    // (the choice of the map stays outside the loops over the elements)
+#pragma unroll
+    for (int c = 0; c < DC; ++c) {
+      i32x4_t pw;
+#pragma unroll
+      for (int j2 = 0; j2 < 4; ++j2) {
+        const uint32_t xx = (uint32_t)__builtin_bit_cast(i32x4_t, xq[c])[j2];
+        pair_done(c, j2, fmaxf(E::to_float((uint16_t)(xx & 0xffffu)), 0.f), fmaxf(E::to_float((uint16_t)(xx >> 16)), 0.f), pw);
+      }
+      qf[c] = __builtin_bit_cast(i16x8_t, pw);
+    }
+  } else {
+#pragma unroll
+    for (int c = 0; c < DC; ++c) {
+      i32x4_t pw;
+#pragma unroll
+      for (int j2 = 0; j2 < 4; ++j2) {
+        const uint32_t xx = (uint32_t)__builtin_bit_cast(i32x4_t, xq[c])[j2];
+        const float x0 = E::to_float((uint16_t)(xx & 0xffffu)), x1 = E::to_float((uint16_t)(xx >> 16));
+        float e0, e1;                                    // elu, rounded; then + 1, rounded by pair_done
+        round16_pair<Tag>(x0 > 0.f ? x0 : (__expf(x0) - 1.0f), x1 > 0.f ? x1 : (__expf(x1) - 1.0f), e0, e1);
+        pair_done(c, j2, e0 + 1.0f, e1 + 1.0f, pw);
+      }
+      qf[c] = __builtin_bit_cast(i16x8_t, pw);
+    }
+  }
+  return den;
+}
+
 // Gradient through phi for one row held in accumulator layout: `x` raw inputs, `gr` the gradient
 // w.r.t. phi(x), both DT tiles of 16 values (this lane's half of the row; lane^32 has the rest).
 template <int DT>

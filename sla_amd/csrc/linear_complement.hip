@@ -327,27 +327,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       const int qrow = mb * BLKQ + wave * 32 + r;
       const bool ok = qrow < L;
       const size_t off = ((size_t)bh * L + qrow) * D;
-      float f[DC][8];
+      i16x8_t xq[DC];
 #pragma unroll
       for (int c = 0; c < DC; ++c) {
-        i16x8_t x = {0, 0, 0, 0, 0, 0, 0, 0};
-        if (ok) x = *reinterpret_cast<const i16x8_t*>(q + off + 16 * c + 8 * g);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) f[c][j] = E::to_float((uint16_t)x[j]);
+        xq[c] = i16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+        if (ok) xq[c] = *reinterpret_cast<const i16x8_t*>(q + off + 16 * c + 8 * g);
       }
-      float row_mx, row_inv;
-      phi_row_pair<Tag, DC>(fmap, f, row_mx, row_inv);
-      float den = 0.f;
       i16x8_t qf[DC];
-#pragma unroll
-      for (int c = 0; c < DC; ++c) {
-        i32x4_t pw;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) den += round16<Tag>(f[c][j] * sZ[16 * c + 8 * g + j]);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) pw[j] = (int)E::pack2(f[c][2 * j], f[c][2 * j + 1]);
-        qf[c] = __builtin_bit_cast(i16x8_t, pw);
-      }
+      float den = phi_pack_den<Tag, DC>(fmap, xq, qf, [&](int c, int j) { return sZ[16 * c + 8 * g + j]; });
       den += __shfl_xor(den, 32);
       den = round16<Tag>(1e-5f + round16<Tag>(den));
       const float inv_den = 1.0f / den;
