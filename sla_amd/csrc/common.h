@@ -172,6 +172,15 @@ struct TileRows {
       if (row < rows_valid) *reinterpret_cast<i16x8_t*>(gtile + (size_t)row * pitch + col) = x[i];
     }
   }
+  // registers -> global, as streaming stores: the rows are not read again by this kernel, and what does not stay behind as
+  // modified lines in L2 does not have to be written back when the kernel ends, before the next one may start
+  __device__ __forceinline__ void store_streaming(uint16_t* gtile, int rows_valid, int lane, size_t pitch = D) const {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const int idx = lane + 64 * i, row = idx / CPR, col = (idx % CPR) * 8;
+      if (row < rows_valid) __builtin_nontemporal_store(x[i], reinterpret_cast<i16x8_t*>(gtile + (size_t)row * pitch + col));
+    }
+  }
   // this += other, element-wise in fp32 with one rounding
   template <typename E>
   __device__ __forceinline__ void add(const TileRows& o) {

@@ -343,22 +343,34 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
       }
     return;
   }
-  if (kok) {
-    uint16_t* dkrow = dk + head_off + (size_t)krow * pitch;
-    uint16_t* dvrow = dv + head_off + (size_t)krow * pitch;
+  // The rounded rows go through LDS (both waves are done with the generations) and leave as whole rows in streaming
+  // stores: they are not read again here, and what does not stay behind as modified lines in L2 need not be written
+  // back when the kernel ends.
+  __syncthreads();
+  uint16_t* const stage = reinterpret_cast<uint16_t*>(smem) + w * (32 * TileRows<D>::SSTR);
+  const int krow0 = nb * 64 + w * 32;
+#pragma unroll
+  for (int which = 0; which < 2; ++which) {
+    constexpr int SSTR = TileRows<D>::SSTR;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
       for (int i4 = 0; i4 < 4; ++i4) {
-        const int d0 = 32 * dt + 8 * i4 + 4 * g;
         i32x2_t wv;
-        wv[0] = (int)E::pack2(dkacc[dt][4 * i4 + 0] * qk_scale, dkacc[dt][4 * i4 + 1] * qk_scale);
-        wv[1] = (int)E::pack2(dkacc[dt][4 * i4 + 2] * qk_scale, dkacc[dt][4 * i4 + 3] * qk_scale);
-        *reinterpret_cast<i32x2_t*>(dkrow + d0) = wv;
-        wv[0] = (int)E::pack2(dvacc[dt][4 * i4 + 0], dvacc[dt][4 * i4 + 1]);
-        wv[1] = (int)E::pack2(dvacc[dt][4 * i4 + 2], dvacc[dt][4 * i4 + 3]);
-        *reinterpret_cast<i32x2_t*>(dvrow + d0) = wv;
+        if (which == 0) {
+          wv[0] = (int)E::pack2(dkacc[dt][4 * i4 + 0] * qk_scale, dkacc[dt][4 * i4 + 1] * qk_scale);
+          wv[1] = (int)E::pack2(dkacc[dt][4 * i4 + 2] * qk_scale, dkacc[dt][4 * i4 + 3] * qk_scale);
+        } else {
+          wv[0] = (int)E::pack2(dvacc[dt][4 * i4 + 0], dvacc[dt][4 * i4 + 1]);
+          wv[1] = (int)E::pack2(dvacc[dt][4 * i4 + 2], dvacc[dt][4 * i4 + 3]);
+        }
+        *reinterpret_cast<i32x2_t*>(&stage[r * SSTR + 32 * dt + 8 * i4 + 4 * g]) = wv;
       }
+    wave_lds_fence();
+    TileRows<D> t;
+    t.unpark(stage, lane);
+    t.store_streaming((which == 0 ? dk : dv) + head_off + (size_t)krow0 * pitch, L - krow0, lane, pitch);
+    wave_lds_fence();
   }
 }
 
@@ -632,21 +644,26 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 1))) void
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // (nothing of this workgroup is in flight when it ends)
 
+  // The rounded rows go through LDS (the rings are free now) and leave as whole rows in streaming stores: they are not
+  // read again here, and what does not stay behind as modified lines in L2 need not be written back when the kernel ends.
+  uint16_t* const stage = reinterpret_cast<uint16_t*>(smem);
 #pragma unroll
   for (int qt = 0; qt < 2; ++qt) {
-    const int qrow = qrow0 + 32 * qt + r;
-    if (qrow < L) {
-      uint16_t* orow = dq + head_off + (size_t)qrow * pitch;
+    constexpr int SSTR = TileRows<D>::SSTR;
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt)
+    for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-        for (int i4 = 0; i4 < 4; ++i4) {
-          i32x2_t wv;
-          wv[0] = (int)E::pack2(dqacc[dt][qt][4 * i4 + 0] * qk_scale, dqacc[dt][qt][4 * i4 + 1] * qk_scale);
-          wv[1] = (int)E::pack2(dqacc[dt][qt][4 * i4 + 2] * qk_scale, dqacc[dt][qt][4 * i4 + 3] * qk_scale);
-          *reinterpret_cast<i32x2_t*>(orow + 32 * dt + 8 * i4 + 4 * g) = wv;
-        }
-    }
+      for (int i4 = 0; i4 < 4; ++i4) {
+        i32x2_t wv;
+        wv[0] = (int)E::pack2(dqacc[dt][qt][4 * i4 + 0] * qk_scale, dqacc[dt][qt][4 * i4 + 1] * qk_scale);
+        wv[1] = (int)E::pack2(dqacc[dt][qt][4 * i4 + 2] * qk_scale, dqacc[dt][qt][4 * i4 + 3] * qk_scale);
+        *reinterpret_cast<i32x2_t*>(&stage[r * SSTR + 32 * dt + 8 * i4 + 4 * g]) = wv;
+      }
+    wave_lds_fence();
+    TileRows<D> t;
+    t.unpark(stage, lane);
+    t.store_streaming(dq + head_off + (size_t)(qrow0 + 32 * qt) * pitch, L - qrow0 - 32 * qt, lane, pitch);
+    wave_lds_fence();
   }
 }
 

@@ -338,7 +338,7 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(D == 6
   auto flush_rows = [&](uint16_t* dst_tile, size_t dst_pitch) {   // staging tile -> global rows
     TileRows<D> t;
     t.unpark(stage_e, lane_e);
-    t.store(dst_tile, qrows_valid_e, lane_e, dst_pitch);
+    t.store_streaming(dst_tile, qrows_valid_e, lane_e, dst_pitch);
     wave_lds_fence();
   };
   if (!FUSED) {

@@ -606,7 +606,7 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     auto flush_rows = [&](uint16_t* dst_tile, size_t dst_pitch) __attribute__((always_inline)) {
       TileRows<D> t;
       t.unpark(stage_q, lane);
-      t.store(dst_tile, rows_valid, lane, dst_pitch);
+      t.store_streaming(dst_tile, rows_valid, lane, dst_pitch);
       wave_lds_fence();
     };
     if (!FUSED) {
