@@ -444,8 +444,15 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
     accumulate(vslot_prev, pb);
   }
   const float inv = 1.0f / lacc[0];        // P_SCALE cancels: numerator and l carry the same factor
-  if (qrow < L) {
-    uint16_t* orow = o + head_off + (size_t)qrow * D;
+  // The rounded rows go through LDS (every wave is done with the tiles) and leave as whole rows in streaming stores:
+  // they are not read again here, and what does not stay behind as modified lines in L2 need not be written back when
+  // the kernel ends.
+  __syncthreads();
+  {
+    constexpr int SSTR = TileRows<D>::SSTR;
+    static_assert(3 * 32 * SSTR * 2 <= (int)sizeof(sV) && 32 * SSTR * 2 <= (int)sizeof(sK), "staging tiles of four waves");
+    uint16_t* const stage = wave < 3 ? reinterpret_cast<uint16_t*>(&sV[0][0]) + wave * (32 * SSTR)
+                                     : reinterpret_cast<uint16_t*>(&sK[0][0]);
     const float* vs = v_scale + (size_t)bh * D;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
@@ -456,8 +463,13 @@ __global__ __launch_bounds__(BLKQ * 2) __attribute__((amdgpu_waves_per_eu(2, 2))
         i32x2_t w;
         w[0] = (int)EO::pack2(oacc[dt][4 * i4 + 0] * inv * sv[0], oacc[dt][4 * i4 + 1] * inv * sv[1]);
         w[1] = (int)EO::pack2(oacc[dt][4 * i4 + 2] * inv * sv[2], oacc[dt][4 * i4 + 3] * inv * sv[3]);
-        *reinterpret_cast<i32x2_t*>(orow + d0) = w;
+        *reinterpret_cast<i32x2_t*>(&stage[r * SSTR + d0]) = w;
       }
+    wave_lds_fence();
+    const int row0 = mb * BLKQ + wave * 32;
+    TileRows<D> t;
+    t.unpark(stage, lane);
+    t.store_streaming(o + head_off + (size_t)row0 * D, L - row0, lane, D);
   }
 }
 
