@@ -443,11 +443,11 @@ static int launch_fwd(const void* q, const void* k, const void* v, const void* l
     const int grid_p = xcd_grid(total_p);
     const int one_row = BLKQ == 128;
     if (fl)
-      hipLaunchKernelGGL((sparse_fwd_pair_kernel<Tag, true>), dim3(grid_p), dim3(128), 0, st, (const uint16_t*)q,
+      hipLaunchKernelGGL((sparse_fwd_pair_kernel<Tag, true>), dim3(grid_p), dim3(256), 0, st, (const uint16_t*)q,
                          (const uint16_t*)k, (const uint16_t*)v, lut, lut64, (uint16_t*)o, lse, lin, lout, L, Mblk64, topk, c,
                          total_p, fl->kvwt, fl->zst, fl->bias, fl->fmap, fl->o_s, one_row);
     else
-      hipLaunchKernelGGL((sparse_fwd_pair_kernel<Tag, false>), dim3(grid_p), dim3(128), 0, st, (const uint16_t*)q,
+      hipLaunchKernelGGL((sparse_fwd_pair_kernel<Tag, false>), dim3(grid_p), dim3(256), 0, st, (const uint16_t*)q,
                          (const uint16_t*)k, (const uint16_t*)v, lut, lut64, (uint16_t*)o, lse, lin, lout, L, Mblk64, topk, c,
                          total_p, (const uint16_t*)nullptr, (const uint16_t*)nullptr, (const float*)nullptr, 0,
                          (uint16_t*)nullptr, one_row);
