@@ -62,11 +62,29 @@ def measured_traffic(workload: str):
             "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a copy kernel of known size")
 
 
+def measured_clock_mhz(workload: str):
+    """Shader clock while the dominant kernel runs, from the committed counter readings: GRBM_GUI_ACTIVE (cycles the
+    graphics engine was busy during one dispatch) over the dispatch's duration in the same profiler run.  None when the
+    readings are missing or older than the kernel's sources."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            t = json.load(f)
+    except (OSError, ValueError):
+        return None
+    if t.get("workload") != workload or t.get("kernel_sources_sha256_16") != kernel_fingerprint():
+        return None
+    if not t.get("gui_active_cycles") or not t.get("dispatch_duration_us"):
+        return None
+    return t["gui_active_cycles"] / t["dispatch_duration_us"]
+
+
 def record_traffic(values):
-    fetch_kib, write_kib, fetch_factor, write_factor = values
+    fetch_kib, write_kib, fetch_factor, write_factor = values[:4]
     t = {"workload": "cfg3", "kernel": "sparse_fwd_pair_kernel<FUSED>", "fetch_size_kib": fetch_kib, "write_size_kib": write_kib,
          "fetch_factor": fetch_factor, "write_factor": write_factor, "kernel_sources_sha256_16": kernel_fingerprint(),
          "kernel_sources": list(KERNEL_SOURCES)}
+    if len(values) >= 6:
+        t["gui_active_cycles"], t["dispatch_duration_us"] = values[4], values[5]
     with open(TRAFFIC_FILE, "w") as f:
         json.dump(t, f, indent=1)
         f.write("\n")
@@ -98,6 +116,81 @@ def time_region(torch, fn, steps, warmup, preheat_s=0.15):
     e1.record()
     torch.cuda.synchronize()
     return e0.elapsed_time(e1) / steps
+
+
+def _median(xs):
+    xs = sorted(xs)
+    n = len(xs)
+    return xs[n // 2] if n % 2 else 0.5 * (xs[n // 2 - 1] + xs[n // 2])
+
+
+def time_steps(torch, fn, steps, warmup, preheat_s=0.15, flush=None):
+    """Times exactly `steps` calls, one event pair per call, on the current stream; returns their median and mean in ms.
+
+    Without `flush` the calls run back to back (caches warm from the call before, as the reference's README figures
+    were not: its script times with triton.testing.do_bench, which clears the L2 between calls).  With `flush`, a
+    tensor larger than the L2s and the memory-side cache together, that tensor is overwritten before every call,
+    outside the timed pair: every call then starts from cold caches.
+    """
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < preheat_s:
+        for _ in range(10):
+            fn()
+        torch.cuda.synchronize()
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    pairs = [_events(torch) for _ in range(steps)]
+    for e0, e1 in pairs:
+        if flush is not None:
+            flush.fill_(0)
+        e0.record()
+        fn()
+        e1.record()
+    torch.cuda.synchronize()
+    ms = [e0.elapsed_time(e1) for e0, e1 in pairs]
+    return _median(ms), sum(ms) / len(ms)
+
+
+def boundary_margins(torch, dev, path):
+    """Writes, per benchmark configuration, how far apart the last selected and the first rejected pooled score of a
+    query block lie, in units of the 16-bit format's spacing at that magnitude: a margin of 0 is a tie, which the
+    lowest block index decides; small margins are where a different summation order would select another block."""
+    from sla_amd import get_block_map
+    from sla_amd.block_map import mean_pool
+    from sla_amd.inputs import CONFIGS, make_inputs, make_inputs_on_device
+    lines = ["# Margin between the last selected and the first rejected pooled score, per query block", "",
+             "Written by `python3 bench.py --margins` on the GPU box.  Scores are formed as the mask builder forms them (block means of q",
+             "and of the smoothed k in the input dtype, fp32 products, rounded to the input dtype); the margin of a query block is the",
+             "T-th largest score of its row minus the (T+1)-th, in units of the dtype's spacing at the T-th score's magnitude.", "",
+             "| config | rows | T of N | margin 0 (ties) | 1 | 2-3 | 4-7 | 8-15 | 16-63 | >= 64 |", "|---|---|---|---|---|---|---|---|---|---|"]
+    for name in ("cfg1", "cfg2", "cfg3", "cfg4", "cfg5"):
+        cfg = CONFIGS[name]
+        if cfg.L > 40000:
+            q, k, _, _ = make_inputs_on_device(cfg, dev, 4, False)
+        else:
+            d = make_inputs(cfg)
+            q, k = d["q"].to(dev), d["k"].to(dev)
+        _, _, T = get_block_map(q, k, cfg.topk, cfg.BLKQ, cfg.BLKK)
+        km = k.float().mean(dim=-2, keepdim=True).to(k.dtype)
+        pq = mean_pool(q, cfg.BLKQ).float()
+        pk = mean_pool((k - km).contiguous(), cfg.BLKK).float()
+        s = torch.matmul(pq, pk.transpose(-1, -2)).to(q.dtype)
+        N = s.shape[-1]
+        if T >= N:
+            lines.append(f"| {name} | {s[..., 0].numel()} | {T} of {N} | every block selected | | | | | | |")
+            continue
+        top = torch.sort(s.float(), dim=-1, descending=True).values
+        a, b_ = top[..., T - 1], top[..., T]
+        mant = 8 if q.dtype == torch.bfloat16 else (11 if q.dtype == torch.float16 else 24)
+        ulp = torch.exp2(torch.floor(torch.log2(a.abs().clamp_min(1e-30))) - (mant - 1))
+        mg = torch.round((a - b_) / ulp).flatten()
+        edges = [0, 1, 2, 4, 8, 16, 64]
+        counts = [int(((mg >= lo) & (mg < hi)).sum()) for lo, hi in zip(edges, edges[1:] + [float("inf")])]
+        lines.append(f"| {name} | {mg.numel()} | {T} of {N} | " + " | ".join(str(c) for c in counts) + " |")
+        del q, k, s, top
+    with open(path, "w") as f:
+        f.write("\n".join(lines) + "\n")
 
 
 def cpu_baseline(cfg, heads, torch):
@@ -215,12 +308,17 @@ def main():
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run one plain 1 GiB read + 1 GiB write elementwise kernel, the known-size reference for "
                          "scaling the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
-    ap.add_argument("--record-traffic", type=float, nargs=4, metavar=("FETCH_KIB", "WRITE_KIB", "FETCH_FACTOR", "WRITE_FACTOR"),
+    ap.add_argument("--record-traffic", type=float, nargs="+",
+                    metavar="FETCH_KIB WRITE_KIB FETCH_FACTOR WRITE_FACTOR [GUI_ACTIVE_CYCLES DISPATCH_US]",
                     help="store the FETCH_SIZE / WRITE_SIZE readings (KiB per dispatch of the dominant kernel) and the "
-                         "calibration factors of two rocprofv3 --pmc runs, stamped with the kernel sources' fingerprint; "
-                         "needs no GPU")
+                         "calibration factors of two rocprofv3 --pmc runs and, optionally, GRBM_GUI_ACTIVE and the duration "
+                         "(us) of one dispatch from a third, stamped with the kernel sources' fingerprint; needs no GPU")
+    ap.add_argument("--margins", action="store_true",
+                    help="write profiles/pooled_score_boundary_margins.md (how close the block selection of every "
+                         "configuration is to a tie) and exit")
     args = ap.parse_args()
     if args.record_traffic:
+        assert len(args.record_traffic) in (4, 6), "--record-traffic takes 4 or 6 values"
         record_traffic(args.record_traffic)
         return
     if args.gpus != 1:
@@ -240,6 +338,9 @@ def main():
 
     cfg = CONFIGS[args.workload]
     dev = torch.device("cuda:0")
+    if args.margins:
+        boundary_margins(torch, dev, os.path.join(ROOT, "profiles", "pooled_score_boundary_margins.md"))
+        return
     d = make_inputs(cfg, with_do=True)
     q, k, v, do = (d[x].to(dev) for x in ("q", "k", "v", "do"))
     w, b = make_proj(cfg.D)
@@ -251,9 +352,12 @@ def main():
     M = -(-L // cfg.BLKQ)
     N = -(-L // cfg.BLKK)
 
-    # ---- the step: full module forward ----
+    # ---- the step: full module forward; exactly `steps` calls are timed, each with its own event pair; the
+    # headline is their median ----
+    flush_buf = torch.empty(512 << 20, dtype=torch.uint8, device=dev)      # larger than 8 x 4 MB of L2 + 256 MB behind them
     with torch.no_grad():
-        ms_fwd = time_region(torch, lambda: mod(q, k, v), args.steps, args.warmup)
+        ms_fwd, ms_fwd_mean = time_steps(torch, lambda: mod(q, k, v), args.steps, args.warmup)
+        ms_fwd_cold, _ = time_steps(torch, lambda: mod(q, k, v), max(args.steps // 2, 5), 2, preheat_s=0.05, flush=flush_buf)
     dense_flops = 4.0 * B * H * L * L * D
     eff_tflops = dense_flops / ms_fwd / 1e9
 
@@ -263,8 +367,27 @@ def main():
     scale = D ** -0.5
     wdev, bdev = mod.proj_l.weight.detach().contiguous(), mod.proj_l.bias.detach().contiguous()
     state_ws = linear_state_fwd(k, v, wdev, cfg.feature_map)
-    ms_sparse = time_region(torch, lambda: sparse_attn_linear_fwd(q, k, v, lut, T, cfg.BLKQ, cfg.BLKK, scale, state_ws,
-                                                                  bdev, cfg.feature_map, False), args.steps, args.warmup)
+    def attention():
+        return sparse_attn_linear_fwd(q, k, v, lut, T, cfg.BLKQ, cfg.BLKK, scale, state_ws, bdev, cfg.feature_map, False)
+    ms_sparse, ms_sparse_mean = time_steps(torch, attention, args.steps, args.warmup)
+    ms_sparse_cold, _ = time_steps(torch, attention, max(args.steps // 2, 5), 2, preheat_s=0.05, flush=flush_buf)
+    # the same launch where the module makes it: behind the mask builder on this stream and the state build on the
+    # module's second stream, caches as those kernels leave them
+    from sla_amd.module import _StateBuild
+    in_module = []
+    with torch.no_grad():
+        for i in range(args.warmup + args.steps):
+            st_build = _StateBuild(k, v, wdev, cfg.feature_map)
+            _, lut_i, _ = get_block_map(q, k, cfg.topk, cfg.BLKQ, cfg.BLKK)
+            ws_i = st_build.join()
+            e0, e1 = _events(torch)
+            e0.record()
+            sparse_attn_linear_fwd(q, k, v, lut_i, T, cfg.BLKQ, cfg.BLKK, scale, ws_i, bdev, cfg.feature_map, False)
+            e1.record()
+            if i >= args.warmup:
+                in_module.append((e0, e1))
+        torch.cuda.synchronize()
+    ms_sparse_in_module = _median([e0.elapsed_time(e1) for e0, e1 in in_module])
     # executed MFMA work: QK^T and PV over the selected tiles + phi(q) KVW of the epilogue
     sparse_flops = 4.0 * B * H * M * T * cfg.BLKQ * cfg.BLKK * D + 2.0 * B * H * L * D * D
     achieved = sparse_flops / ms_sparse / 1e9
@@ -274,6 +397,8 @@ def main():
         "value": eff_tflops,
         "unit": "TFLOP/s (dense-equivalent 4*B*H*L^2*D per full module forward)",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_fwd,
+        "ms_per_step_note": "median of the timed steps (one event pair each, back to back)",
+        "ms_per_step_mean": ms_fwd_mean, "ms_per_step_l2_flushed": ms_fwd_cold,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"{cfg.name}: SLA module forward B{B} H{H} L{L} D{D} BLKQ{cfg.BLKQ} BLKK{cfg.BLKK} "
                                f"topk{cfg.topk} (T={T} of N={N}) feature_map={cfg.feature_map}, structured q/k",
@@ -282,7 +407,16 @@ def main():
                      "frac": achieved / PEAK_BF16_TFLOPS,
                      "traffic": traffic, "traffic_note": traffic_note,
                      "traffic_unit": "HBM bytes per launch (fetch + write)", "kernel": "sparse_fwd_pair_kernel<FUSED=true>",
-                     "flops_per_launch": sparse_flops, "ms_per_launch": ms_sparse},
+                     "flops_per_launch": sparse_flops, "ms_per_launch": ms_sparse,
+                     "frac_note": "frac = flops_per_launch / ms_per_launch / peak; ms_per_launch is the median of the "
+                                  "kernel launched back to back (warm caches)",
+                     "ms_per_launch_mean": ms_sparse_mean, "ms_per_launch_l2_flushed": ms_sparse_cold,
+                     "ms_per_launch_in_module": ms_sparse_in_module,
+                     "frac_in_module": sparse_flops / ms_sparse_in_module / 1e9 / PEAK_BF16_TFLOPS,
+                     "frac_l2_flushed": sparse_flops / ms_sparse_cold / 1e9 / PEAK_BF16_TFLOPS,
+                     "clock_mhz": measured_clock_mhz(cfg.name),
+                     "clock_note": "GRBM_GUI_ACTIVE / dispatch duration of the kernel in a rocprofv3 --pmc run; the peak "
+                                   "is quoted at 2400 MHz"},
     }
     extra = {"sla_fwd_ms": ms_fwd, "attention_fused_ms": ms_sparse}
     if not args.no_extras:

@@ -510,6 +510,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   // the last unit's products (nunits is even: its probabilities are in pb_b, V_{nunits-1} is on its way into generation 1)
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
+  // (what the rest needs of the lane's number is formed again here, from an opaque copy, so that none of it is kept in
+  //  a register, or spilled, across the loop)
+  int lane_e = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+  asm volatile("" : "+v"(lane_e));
+  const int g_e = lane_e >> 5, r_e = lane_e & 31, lrow_e = lane_e >> 4, lslot_e = lane_e & 15;
   if (FUSED) {
     // Fused linear branch: the per-head state KVW^T (D x D, 16 bit) goes into the K ring, which nobody reads any more,
     // the way K half-tiles do (rows of 256 bytes, swizzled pieces, each wave requests a quarter), while the last
@@ -517,12 +522,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const uint8_t* st_b = reinterpret_cast<const uint8_t*>(kvwt + (size_t)bh * D * D);
     const uint64_t a = (uint64_t)(uintptr_t)st_b;
     const u32x4_t sth{(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)a),
-                      (uint32_t)__builtin_amdgcn_readfirstlane((int)((uint32_t)(a >> 32) & 0xffffu)), (uint32_t)(D * D * 2),
+                      (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(a >> 32)), (uint32_t)(D * D * 2),
                       0x00020000u};
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      const int row = 32 * w + 4 * i + lrow;                 // (lane part: row 4 (i % 4) + lrow of sixteen, swizzled piece)
-      const uint32_t soff = (uint32_t)(row * ROWB + ((lslot ^ ((4 * i + lrow) & 15)) * 16));
+      const int row = 32 * w + 4 * i + lrow_e;                 // (lane part: row 4 (i % 4) + lrow of sixteen, swizzled piece)
+      const uint32_t soff = (uint32_t)(row * ROWB + ((lslot_e ^ ((4 * i + lrow_e) & 15)) * 16));
       const uint32_t ldst = smem_addr + (uint32_t)((32 * w + 4 * i) * ROWB);
       asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(ldst), "v"(soff), "s"(sth) : "memory");
     }
@@ -546,8 +551,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int rows_valid = writes ? min(32, L - qrow0) : 0;
   const float l_tot = l_run + __shfl_xor(l_run, 32);
   const float inv = 1.0f / l_tot;
-  const int qrow = qrow0 + r;
-  if (qrow < L && g == 0 && writes) lse[(size_t)bh * L + qrow] = m_used * scale_log2e + fast_log2(l_tot);
+  const int qrow = qrow0 + r_e;
+  if (qrow < L && g_e == 0 && writes) lse[(size_t)bh * L + qrow] = m_used * scale_log2e + fast_log2(l_tot);
   auto park_attention = [&]() __attribute__((always_inline)) {
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
@@ -556,14 +561,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         i32x2_t wv;
         wv[0] = (int)E::pack2(oacc[dt][4 * i4 + 0] * inv, oacc[dt][4 * i4 + 1] * inv);
         wv[1] = (int)E::pack2(oacc[dt][4 * i4 + 2] * inv, oacc[dt][4 * i4 + 3] * inv);
-        *reinterpret_cast<i32x2_t*>(&stage[r * SSTR + 32 * dt + 8 * i4 + 4 * g]) = wv;
+        *reinterpret_cast<i32x2_t*>(&stage[r_e * SSTR + 32 * dt + 8 * i4 + 4 * g_e]) = wv;
       }
     wave_lds_fence();
   };
   auto flush_rows = [&](uint16_t* dst_tile, size_t dst_pitch) __attribute__((always_inline)) {
     TileRows<D> t;
-    t.unpark(stage, lane);
-    t.store_streaming(dst_tile, rows_valid, lane, dst_pitch);
+    t.unpark(stage, lane_e);
+    t.store_streaming(dst_tile, rows_valid, lane_e, dst_pitch);
     wave_lds_fence();
   };
   if (!FUSED) {
@@ -571,11 +576,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     flush_rows(o + out_off, (size_t)lout.sl);
   } else {
     // ---- linear branch of the same rows (see sparse_fwd_kernel) ----
-    // The q rows are the resident B operands of the score products, as they came from memory.
+    // The q rows are the resident B operands of the score products, as they came from memory.  (Taken over here from
+    // the accumulation registers the loop read them from: left to itself the compiler keeps a second copy of them
+    // across the loop for this use.)
+#pragma unroll
+    for (int c = 0; c < DC; ++c) asm volatile("" : "+a"(qf[c]));
     const uint16_t* z_h = zst + (size_t)bh * D;
     i16x8_t fq[DC], zreg[DC];
 #pragma unroll
-    for (int c = 0; c < DC; ++c) zreg[c] = *reinterpret_cast<const i16x8_t*>(z_h + 16 * c + 8 * g);
+    for (int c = 0; c < DC; ++c) zreg[c] = *reinterpret_cast<const i16x8_t*>(z_h + 16 * c + 8 * g_e);
     float den = phi_pack_den<Tag, DC>(fmap, qf, fq, [&](int c, int j) __attribute__((always_inline)) {
       return E::to_float((uint16_t)zreg[c][j]);
     });
@@ -587,7 +596,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       i16x8_t a[DC];
 #pragma unroll
       for (int c = 0; c < DC; ++c)
-        a[c] = *reinterpret_cast<const i16x8_t*>(smem + (32 * et + r) * ROWB + (((2 * c + g) ^ (r & 15)) * 16));
+        a[c] = *reinterpret_cast<const i16x8_t*>(smem + (32 * et + r_e) * ROWB + (((2 * c + g_e) ^ (r_e & 15)) * 16));
       f32x16_t acc;
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[i] = 0.f;
@@ -595,7 +604,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       for (int c = 0; c < DC; ++c) acc = E::mfma32(a[c], fq[c], acc);
 #pragma unroll
       for (int i4 = 0; i4 < 4; ++i4) {
-        const int e0 = 32 * et + 8 * i4 + 4 * g;
+        const int e0 = 32 * et + 8 * i4 + 4 * g_e;
         const f32x4_t b4 = *reinterpret_cast<const f32x4_t*>(bias + e0);
         float bb[4];
         round16_pair<Tag>(b4[0], b4[1], bb[0], bb[1]);
@@ -612,7 +621,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                             pin_f32(__builtin_fmaf(acc[4 * i4 + 2 * h + 1], inv_den, bb[2 * h + 1])), l0, l1);
           wo[h] = (int)E::pack2(E::to_float((uint16_t)(x & 0xffff)) + l0, E::to_float((uint16_t)(x >> 16)) + l1);
         }
-        *reinterpret_cast<i32x2_t*>(&stage[r * SSTR + e0]) = wo;
+        *reinterpret_cast<i32x2_t*>(&stage[r_e * SSTR + e0]) = wo;
       }
     }
     wave_lds_fence();
