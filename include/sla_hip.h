@@ -74,6 +74,8 @@ int sla_mean_pool(const void* x, void* out, int dtype, int BH, int L, int D, int
  * top-k (ties to the lowest index).  Writes the int8 0/1 map (B*H, M, N) and the
  * ascending look-up table (B*H, M, topk) with elements of lut_elem_bytes (4 or 8).
  * topk = min(N, int(ratio*N)) is computed by the caller.
+ * Limits: N = ceil(L/BLKK) <= 4096 key blocks (L <= 262144), B*H <= 65535; more returns SLA_ERR_UNSUPPORTED
+ * (sage_prepare has the same limits).
  * Replaces get_block_map, sparse_linear_attention/utils.py:55-67. */
 int sla_block_map_fwd(const void* q, const void* k, int dtype, int B, int H, int L, int D, int BLKQ, int BLKK,
                       int topk, void* workspace, int64_t workspace_bytes, int8_t* sparse_map, void* lut,

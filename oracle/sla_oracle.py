@@ -512,15 +512,3 @@ def sage_sparse_attn_fwd(q, k, v, lut, BLKQ=128, BLKK=64, qk_scale=None, heads=N
         ob = torch.bmm(p8, vg) * vs[b, h].view(1, 1, D) / (FP8_E4M3_MAX * l)
         o[b, h] = ob.reshape(M * BLKQ, D)[:L]
     return o
-
-
-def sage_sla_forward(q, k, v, weight, bias, topk_ratio, fmap="softmax",
-                     compute_dtype=torch.bfloat16):
-    """SageSLA module forward (SageSLA/core.py:75-163) with 128/64 blocks."""
-    in_dtype = q.dtype
-    sparse_map, lut, T = get_block_map(q, k, topk_ratio, 128, 64)
-    qc, kc, vc = q.to(compute_dtype), k.to(compute_dtype), v.to(compute_dtype)
-    o_s = sage_sparse_attn_fwd(qc, kc, vc, lut, 128, 64).to(compute_dtype)
-    o_l = linear_branch(qc, kc, vc, weight, bias, fmap, compute_dtype)
-    o = (o_s.float() + o_l.float()).to(in_dtype)
-    return o, o_s, o_l, sparse_map, lut, T

@@ -441,7 +441,8 @@ __global__ __launch_bounds__(256) void topk_kernel(const typename IO::raw* __res
                                                    int8_t* __restrict__ sparse_map, void* __restrict__ lut, int lut64, int N,
                                                    int T, size_t nrows) {
   extern __shared__ uint32_t lds_keys[];
-  __shared__ __attribute__((aligned(16))) uint32_t hist_all[4][256];
+  // (the histograms are only used when the keys live in LDS: the register instances carry a token array)
+  __shared__ __attribute__((aligned(16))) uint32_t hist_all[EPL == 0 ? 4 : 1][EPL == 0 ? 256 : 1];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const size_t row = (size_t)blockIdx.x * 4 + wave;
   if (row >= nrows) return;
@@ -477,7 +478,7 @@ __global__ __launch_bounds__(256) void topk_kernel(const typename IO::raw* __res
   }
   uint32_t thr = 0;          // digits decided so far
   int need = T;              // rank of the threshold among the keys that agree with them
-  uint32_t* hist = hist_all[wave];
+  uint32_t* hist = hist_all[EPL == 0 ? wave : 0];
   if (EPL > 0) {
     // Keys in registers: the threshold is built bit by bit from the top, keeping a bit when at least T keys are at or
     // above the value it gives (one compare per key and bit, counted through the wave's ballot: no memory traffic and no
@@ -738,7 +739,9 @@ static int block_map_entry(const void* q, const void* k, const int64_t* strides,
   if (rc) return rc;
   const int M = cdiv(L, BLKQ), N = cdiv(L, BLKK);
   SLA_REQUIRE(topk >= 0 && topk <= N, SLA_ERR_BAD_ARG, "topk=%d outside [0, %d]", topk, N);
-  SLA_REQUIRE(N <= 4096, SLA_ERR_UNSUPPORTED, "more than 4096 key blocks (%d)", N);   // top-k rows of 4 waves in 64 KB of LDS
+  // (rows longer than the register instances hold keep their keys in LDS: four waves' rows of 4096 keys are 64 KB, plus
+  //  4 KB of histograms, of the 160 KB a workgroup of this machine may use; L <= 262144 at 64-row key blocks)
+  SLA_REQUIRE(N <= 4096, SLA_ERR_UNSUPPORTED, "more than 4096 key blocks (%d)", N);
   SLA_REQUIRE((int64_t)BH * M < (1ll << 31), SLA_ERR_UNSUPPORTED, "too many query-block rows");
   SLA_REQUIRE(lut_elem_bytes == 4 || lut_elem_bytes == 8, SLA_ERR_BAD_ARG, "lut_elem_bytes must be 4 or 8, got %d",
               lut_elem_bytes);

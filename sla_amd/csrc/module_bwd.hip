@@ -30,9 +30,19 @@ int events_for_current_device(SideEvents** out) {
   SLA_REQUIRE(hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64, SLA_ERR_LAUNCH, "no current device");
   SideEvents& e = g_ev[dev];
   if (!e.fork) {
-    hipEvent_t* all[4] = {&e.fork, &e.lists, &e.query, &e.reduced};
-    for (hipEvent_t* p : all)
-      SLA_REQUIRE(hipEventCreateWithFlags(p, hipEventDisableTiming) == hipSuccess, SLA_ERR_LAUNCH, "hipEventCreate failed");
+    // all four or none: the set is published only when every event exists
+    hipEvent_t made[4] = {nullptr, nullptr, nullptr, nullptr};
+    for (int i = 0; i < 4; ++i) {
+      if (hipEventCreateWithFlags(&made[i], hipEventDisableTiming) != hipSuccess) {
+        for (int j = 0; j < i; ++j) (void)hipEventDestroy(made[j]);
+        set_error("hipEventCreate failed");
+        return SLA_ERR_LAUNCH;
+      }
+    }
+    e.lists = made[1];
+    e.query = made[2];
+    e.reduced = made[3];
+    e.fork = made[0];
   }
   *out = &e;
   return SLA_OK;
@@ -76,20 +86,32 @@ extern "C" int sla_module_bwd(const void* q, const void* k, const void* v, const
   std::lock_guard<std::mutex> lock(g_mu);
   SideEvents* ev;
   if ((rc = events_for_current_device(&ev))) return rc;
-  // side: lists of the map.  main: delta, dQ, then the query side of the linear branch
+  // Once the second stream has been made to wait on `stream`, no path leaves this call without `stream` waiting for
+  // the second one in turn: the caller orders later work (and the reuse of the workspaces) by `stream` alone, and a
+  // capture in progress must not be left forked.
+  const auto forked = [&]() -> int {
+    int r;
+    // side: lists of the map.  main: delta, dQ, then the query side of the linear branch
+    if ((r = sparse(side, SB_LISTS))) return r;
+    SLA_HIP_OK(hipEventRecord(ev->lists, side));
+    if ((r = sparse(st, SB_DQ))) return r;
+    if ((r = linear(st, LB_STATES | LB_QUERY))) return r;
+    SLA_HIP_OK(hipEventRecord(ev->query, st));
+    // side: the small products of the linear branch.  main: dK/dV, then the key side of the linear branch
+    SLA_HIP_OK(hipStreamWaitEvent(side, ev->query, 0));
+    if ((r = linear(side, LB_REDUCE))) return r;
+    SLA_HIP_OK(hipEventRecord(ev->reduced, side));
+    SLA_HIP_OK(hipStreamWaitEvent(st, ev->lists, 0));
+    if ((r = sparse(st, SB_DKDV))) return r;
+    SLA_HIP_OK(hipStreamWaitEvent(st, ev->reduced, 0));
+    return linear(st, LB_KEYS);
+  };
   SLA_HIP_OK(hipEventRecord(ev->fork, st));
   SLA_HIP_OK(hipStreamWaitEvent(side, ev->fork, 0));
-  if ((rc = sparse(side, SB_LISTS))) return rc;
-  SLA_HIP_OK(hipEventRecord(ev->lists, side));
-  if ((rc = sparse(st, SB_DQ))) return rc;
-  if ((rc = linear(st, LB_STATES | LB_QUERY))) return rc;
-  SLA_HIP_OK(hipEventRecord(ev->query, st));
-  // side: the small products of the linear branch.  main: dK/dV, then the key side of the linear branch
-  SLA_HIP_OK(hipStreamWaitEvent(side, ev->query, 0));
-  if ((rc = linear(side, LB_REDUCE))) return rc;
-  SLA_HIP_OK(hipEventRecord(ev->reduced, side));
-  SLA_HIP_OK(hipStreamWaitEvent(st, ev->lists, 0));
-  if ((rc = sparse(st, SB_DKDV))) return rc;
-  SLA_HIP_OK(hipStreamWaitEvent(st, ev->reduced, 0));
-  return linear(st, LB_KEYS);
+  rc = forked();
+  if (rc) {
+    // join whatever the second stream was given before the failure (its last event may never have been recorded)
+    if (hipEventRecord(ev->reduced, side) == hipSuccess) (void)hipStreamWaitEvent(st, ev->reduced, 0);
+  }
+  return rc;
 }

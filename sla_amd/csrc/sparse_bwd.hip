@@ -738,7 +738,8 @@ static int bwd_impl(const void* q, const void* k, const void* v, const void* o, 
   const int total_q64 = BH * Mblk64;
   const bool stream_dkdv = D == 128 && (BLKQ == 64 || BLKQ == 128) && (uint64_t)lin.sl * 2u * (uint64_t)L < (1ull << 31) &&
                            (uint64_t)ldo.sl * 2u * (uint64_t)L < (1ull << 31);
-  const bool stream_dq = stream_dkdv && topk <= DQ_STREAM_MAX_T && total_q64 >= 1024;      // (enough query blocks for a wave on every SIMD)
+  // (enough query blocks for a wave on every SIMD; the stream kernel keeps a look-up row as 16-bit key block indices)
+  const bool stream_dq = stream_dkdv && topk <= DQ_STREAM_MAX_T && total_q64 >= 1024 && Mblk64 <= 65535;
   // delta = rowsum(dO * O): the dQ kernel of the common shape forms it for its own rows, the general one reads it
   if ((steps & SB_DQ) && !stream_dq)
     hipLaunchKernelGGL((bwd_delta_kernel<Tag, D>), dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, st,

@@ -99,6 +99,12 @@ def test_largest_configuration_forward_backward(dev):
     scale = (q.double() * dq.double()).abs().sum((-1, -2)) + (k.double() * dk.double()).abs().sum((-1, -2))
     assert bool(((ta - tb).abs() <= 1e-3 * scale).all())
 
+    # the index sets of the first, a middle and the last head against the oracle's mask builder
+    for hh in (0, cfg.H // 2 - 1, cfg.H - 1):
+        m_h, lut_h, T_h = O.get_block_map(q[:, hh:hh + 1].cpu(), k[:, hh:hh + 1].cpu(), cfg.topk, cfg.BLKQ, cfg.BLKK)
+        assert T_h == T and torch.equal(m_h, m[:, hh:hh + 1].cpu()), f"map of head {hh} differs from the oracle's"
+        assert torch.equal(lut_h.long(), lut[:, hh:hh + 1].cpu().long()), f"look-up table of head {hh} differs"
+
     # the last head against the oracle (mask builder, forward, backward)
     h = cfg.H - 1
     qc, kc, vc, doc = (t[:, h:h + 1].cpu() for t in (q, k, v, do))

@@ -17,6 +17,14 @@ TOL_COS = 0.999
 TOL_LSE = 1e-3
 
 
+
+def _sum_tol(ref):
+    """Bound on the module output o_s + o_l: 2e-2 where the values stay below 4.  Above, the 16-bit format itself is the
+    limit: bf16 values in [4, 8) are 2^-5 apart, so the one rounding of the sum may already be 1.6e-2 off, before the
+    rounding of the linear branch (values of several units with this test's projection) that both sides carry; the bound
+    grows with the largest magnitude the way that spacing does."""
+    return 2e-2 * max(1.0, float(ref.abs().max()) / 4.0)
+
 def _heads(L):
     pairs_per_head = ((L + 63) // 64 + 1) // 2
     return -(-512 // pairs_per_head)
@@ -123,7 +131,7 @@ def test_fused_linear_branch_on_a_split_pair(dev, dtype):
     out, o_s, lse = sparse_attn_linear_fwd(qd, kd, vd, lut.to(dev), T, 64, 64, 128 ** -0.5, ws, b.to(dev), "softmax",
                                            want_o_s=True)
     assert max_abs(o_s.cpu(), o_s_ref) <= TOL_ABS
-    assert max_abs(out.cpu(), ref) <= 3e-2 and cos_sim(out.cpu(), ref) >= TOL_COS
+    assert max_abs(out.cpu(), ref) <= _sum_tol(ref) and cos_sim(out.cpu(), ref) >= TOL_COS
 
 
 @pytest.mark.parametrize("L", [1024,      # whole 128-row blocks
@@ -162,4 +170,4 @@ def test_query_blocks_of_128_rows(dev, L):
     assert torch.equal(o_s, o) and torch.equal(lse3, lse)
     assert torch.equal(out, out2) and torch.equal(o_s, o_s2) and torch.equal(lse3, lse4)
     ref = o_ref + O.linear_branch(q, k, v, w, b, "elu", torch.bfloat16).float()
-    assert max_abs(out.cpu(), ref) <= 3e-2 and cos_sim(out.cpu(), ref) >= TOL_COS
+    assert max_abs(out.cpu(), ref) <= _sum_tol(ref) and cos_sim(out.cpu(), ref) >= TOL_COS
