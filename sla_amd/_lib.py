@@ -11,7 +11,8 @@ import os
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libsla_hip.so")
+# (SLA_HIP_LIB names another build of the same library, e.g. the one with sanitizers in its host code)
+LIB_PATH = os.environ.get("SLA_HIP_LIB") or os.path.join(_HERE, "lib", "libsla_hip.so")
 
 SLA_F32, SLA_BF16, SLA_F16 = 0, 1, 2
 FMAP = {"elu": 0, "relu": 1, "softmax": 2}
