@@ -64,8 +64,8 @@ def measured_traffic(workload: str):
 
 def measured_clock_mhz(workload: str):
     """Shader clock while the dominant kernel runs, from the committed counter readings: GRBM_GUI_ACTIVE (cycles the
-    graphics engine was busy during one dispatch) over the dispatch's duration in the same profiler run.  None when the
-    readings are missing or older than the kernel's sources."""
+    graphics engine was busy during one dispatch, summed over the device's 8 XCDs) / 8 over the dispatch's duration
+    in the same profiler run.  None when the readings are missing or older than the kernel's sources."""
     try:
         with open(TRAFFIC_FILE) as f:
             t = json.load(f)
@@ -75,7 +75,7 @@ def measured_clock_mhz(workload: str):
         return None
     if not t.get("gui_active_cycles") or not t.get("dispatch_duration_us"):
         return None
-    return t["gui_active_cycles"] / t["dispatch_duration_us"]
+    return t["gui_active_cycles"] / 8.0 / t["dispatch_duration_us"]
 
 
 def record_traffic(values):
@@ -238,7 +238,12 @@ def other_configs(torch, dev, steps):
                      steps, 2, preheat_s=0.05)
     tiles = cfg.B * cfg.H * (-(-cfg.L // cfg.BLKQ)) * T
     ex["cfg3_sparse_bwd_ms"] = ms
+    # two conventions: the seven products per tile that the kernels execute (three in dQ, four in dK/dV: 2 flops
+    # each = 14), and the reference's "backward = 2.5 x forward" (evaluate/bench_kernel.py:97-98), i.e. five
+    # products per tile (10): it counts the scores recomputed once and dP formed once, where the two kernels
+    # here each form both
     ex["cfg3_sparse_bwd_mfma_frac"] = 14.0 * tiles * cfg.BLKQ * 64 * cfg.D / ms / 1e9 / PEAK_BF16_TFLOPS
+    ex["cfg3_sparse_bwd_mfma_frac_2p5x_fwd"] = 10.0 * tiles * cfg.BLKQ * 64 * cfg.D / ms / 1e9 / PEAK_BF16_TFLOPS
     del q, k, v, do, o, lse, m, lut
 
     # ---- cfg5: SageSLA module forward, and its attention kernel against the int8 / fp8 peak ----

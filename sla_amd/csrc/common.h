@@ -242,8 +242,14 @@ static __device__ __forceinline__ float pin_f32(float x) {
 // Matrix products with their result in vector registers (the vector ALU reads it next) and the resident B operand in
 // accumulation registers.  Written as instructions because the compiler gives every MFMA of a function that uses
 // accumulation registers an accumulation-register result and would copy the scores back one register at a time.
-// (The compiler sees no MFMA here and inserts no wait states: callers keep the vector ALU away from a result for the
-// length of the product, and alternate two chains so that consecutive dependent products are 64 cycles apart.)
+// INVARIANT the callers keep: the compiler sees no MFMA here, so its hazard recogniser inserts no wait states behind
+// these instructions.  Between the last product of a chain and the first vector-ALU (or LDS / memory) instruction
+// that reads or overwrites the chain's result registers there are either at least two further MFMAs (each holds
+// the matrix pipe for 8 passes = 32 cycles, which covers the wait states an 8-pass product needs) or an explicit
+// `s_nop 15; s_nop 15`.  The steady-state loops satisfy the first form by construction (the scores of a unit are
+// consumed beside the next unit's products); prologues, ragged-tile masks and the rare re-basing of the reference
+// maximum use the second.  Consecutive dependent products of one chain (result registers = C operand) need no
+// software wait states.
 template <typename Tag>
 static __device__ __forceinline__ void mfma_scores_first(f32x16_t& d, const i16x8_t& a, const i16x8_t& b) {
   if constexpr (__is_same(Tag, bf16_tag))
