@@ -18,17 +18,19 @@
 
 namespace sla {
 
-// 16 bytes per lane, memory -> LDS: lane l's piece lands at lds_base + lds_off + 16 l
+// 16 bytes per lane, memory -> LDS: lane l's piece lands at lds_base + lds_off + 16 l.  (Between a scalar write of M0
+// and a memory -> LDS load that reads it the hardware wants one wait state; the compiler adds it to its own code and
+// does not look into these instructions.)
 static __device__ __forceinline__ void lds_dma_b128(__amdgpu_buffer_rsrc_t rsrc, uint32_t byte_off, uint32_t lds_base,
                                                     uint32_t lds_off) {
-  asm volatile("s_add_u32 m0, %0, %3\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(lds_base), "v"(byte_off), "s"(rsrc),
+  asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(lds_base), "v"(byte_off), "s"(rsrc),
                "s"(lds_off)
                : "memory", "scc");
 }
 // 4 bytes per lane: lane l's word lands at lds_base + lds_off + 4 l
 static __device__ __forceinline__ void lds_dma_b32(__amdgpu_buffer_rsrc_t rsrc, uint32_t byte_off, uint32_t lds_base,
                                                    uint32_t lds_off) {
-  asm volatile("s_add_u32 m0, %0, %3\n\tbuffer_load_dword %1, %2, 0 offen lds" ::"s"(lds_base), "v"(byte_off), "s"(rsrc),
+  asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tbuffer_load_dword %1, %2, 0 offen lds" ::"s"(lds_base), "v"(byte_off), "s"(rsrc),
                "s"(lds_off)
                : "memory", "scc");
 }

@@ -247,9 +247,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   //  it knows to target LDS; the wait for these loads is the one before the barrier of the next iteration.  Rows past
   //  L lie outside the buffer range: nothing is written for them and LDS keeps what it held, which is either the zeros
   //  it was filled with at the start or rows of an earlier tile: finite values, whose scores are masked and whose
-  //  probabilities are 0)
+  //  probabilities are 0.  The s_nop is the wait state the hardware wants between a scalar write of M0 and a memory ->
+  //  LDS load that reads it.)
 #define SLA_PAIR_FETCH2(RSRC, LANEOFF, DST, RING)                                                                      \
-  asm volatile("s_add_u32 m0, %0, %4\n\tbuffer_load_dwordx4 %1, %3, 0 offen lds\n\t"                                  \
+  asm volatile("s_add_u32 m0, %0, %4\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %3, 0 offen lds\n\t"                                  \
                "buffer_load_dwordx4 %2, %3, 0 offen offset:1024 lds" ::"s"(DST), "v"((LANEOFF)[0]), "v"((LANEOFF)[1]),   \
                "s"(RSRC), "n"(RING)                                                                                    \
                : "memory", "scc")
@@ -529,7 +530,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       const int row = 32 * w + 4 * i + lrow_e;                 // (lane part: row 4 (i % 4) + lrow of sixteen, swizzled piece)
       const uint32_t soff = (uint32_t)(row * ROWB + ((lslot_e ^ ((4 * i + lrow_e) & 15)) * 16));
       const uint32_t ldst = smem_addr + (uint32_t)((32 * w + 4 * i) * ROWB);
-      asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(ldst), "v"(soff), "s"(sth) : "memory");
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(ldst), "v"(soff), "s"(sth) : "memory");
     }
   }
   if (nunits > 0) {
