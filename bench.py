@@ -278,6 +278,21 @@ def other_configs(torch, dev, steps):
     ex["cfg4_fwd_effective_tflops"] = dense / ex["cfg4_sla_fwd_ms"] / 1e9
     ex["cfg4_mask_ms"] = ms
     ex["cfg4_mask_hbm_gbs"] = 2.0 * q.numel() * 2 / ms / 1e6
+    # the attention kernel of that forward alone, against the bf16 MFMA peak (the cfg3 convention: executed flops of the
+    # selected tiles and of the epilogue's products)
+    from sla_amd.linear import linear_state_fwd
+    from sla_amd.sparse_attn import sparse_attn_linear_fwd
+    with torch.no_grad():
+        _, lut4, T4 = get_block_map(q, k, cfg.topk, cfg.BLKQ, cfg.BLKK)
+        ws4 = linear_state_fwd(k, v, mod.proj_l.weight, cfg.feature_map)
+        ms = time_region(torch, lambda: sparse_attn_linear_fwd(q, k, v, lut4, T4, cfg.BLKQ, cfg.BLKK, cfg.D ** -0.5, ws4,
+                                                               mod.proj_l.bias, cfg.feature_map, False),
+                         steps, 1, preheat_s=0.05)
+    flops4 = (4.0 * cfg.B * cfg.H * (-(-cfg.L // cfg.BLKQ)) * T4 * cfg.BLKQ * 64 * cfg.D
+              + 2.0 * cfg.B * cfg.H * cfg.L * cfg.D * cfg.D)
+    ex["cfg4_attention_fused_ms"] = ms
+    ex["cfg4_attention_fused_mfma_frac"] = flops4 / ms / 1e9 / PEAK_BF16_TFLOPS
+    del lut4, ws4
     qg, kg, vg = (t.requires_grad_(True) for t in (q, k, v))
 
     def fwd_bwd():
